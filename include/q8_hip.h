@@ -1,0 +1,166 @@
+/*
+ * q8_hip.h - C ABI of libq8_hip.so: the 8-bit inference hot path of q8_kernels
+ * (per-token quantizers, fast Hadamard transform, RMSNorm, RoPE, int8/fp8 GEMM
+ * with fused dequant+bias+GELU, fp8 flash-attention forward) as hand-written
+ * HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is
+ *     allocated, freed or retained by the library;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and the call returns without synchronising;
+ *   - the return value is Q8_OK (0) or a negative Q8_ERR_* code; on error no
+ *     kernel has been launched; q8_last_error() returns a thread-local text;
+ *   - no global mutable state: calls are re-entrant and thread-safe per stream.
+ *
+ * Each entry point cites the interface of the reference implementation
+ * (KONAKONA666/q8_kernels, paths relative to its root) that it replaces.
+ */
+#ifndef Q8_HIP_H
+#define Q8_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* q8_stream_t; /* hipStream_t */
+
+/* element types */
+enum {
+    Q8_I8 = 0,   /* signed 8-bit integer codes                   */
+    Q8_E4M3 = 1, /* OCP fp8 e4m3fn (bias 7, no inf, 0x7f = NaN)  */
+    Q8_BF16 = 2,
+    Q8_F16 = 3,
+    Q8_F32 = 4
+};
+
+/* status codes */
+enum {
+    Q8_OK = 0,
+    Q8_ERR_NULL = -1,      /* required pointer is NULL                      */
+    Q8_ERR_DTYPE = -2,     /* unsupported element type for this entry point */
+    Q8_ERR_SHAPE = -3,     /* unsupported or inconsistent sizes             */
+    Q8_ERR_ALIGN = -4,     /* pointer or stride not aligned as required     */
+    Q8_ERR_LAUNCH = -5,    /* the HIP runtime refused the launch            */
+    Q8_ERR_FLAGS = -6      /* unknown flag bits                             */
+};
+
+/* q8_quant_rows flags */
+enum {
+    Q8_QUANT_RNE = 1,        /* int8 codes: round half to even instead of the reference's
+                                round-half-away-from-zero                                  */
+    Q8_QUANT_SCALE_DIV = 2   /* stored scale = absmax/QMAX instead of the reference's
+                                1/(QMAX/absmax); the codes are unchanged                   */
+};
+
+/* q8_attn_fwd V layouts and flags */
+enum {
+    Q8_V_DS = 0, /* V given as [B,H,D,Nv] (the reference's pre-transposed contract), Nv >= N, Nv % 16 == 0 */
+    Q8_V_SD = 1  /* V given as [B,H,N,D]                                                                    */
+};
+enum {
+    Q8_ATTN_SUM_ROUNDED_P = 1 /* row sum accumulates the e4m3-rounded probabilities (what multiplies V)
+                                 instead of the unrounded fp32 ones                                        */
+};
+
+const char* q8_strerror(int status);
+const char* q8_last_error(void);
+
+/* CU count, peak engine clock (MHz), HBM bytes, and the gcn arch name (>= 32 bytes buffer, nullable). */
+int q8_device_info(int* cu_count, int* clock_mhz, int64_t* hbm_bytes, char* arch_name);
+
+/*
+ * Token-wise (per-row) absmax quantizer.
+ * Replaces quantizer._C.tokenwise_quant  (csrc/quantizer/tokenwise_quant.cpp:74-111,
+ * kernel csrc/quantizer/tokenwise_quant_cuda.cu:91-149).
+ *   a = max_j |x[r,j]|;  r = QMAX / a;  codes[r,j] = cast(x[r,j] * r);  scales[r] = 1 / r
+ *   QMAX = 127 (Q8_I8, rounding half away from zero, see flags) or 448 (Q8_E4M3, RNE).
+ *   A row of zeros yields codes 0 and scale 0.
+ * x: [rows, dim] of x_dtype in {BF16,F16,F32,E4M3}, row stride x_row_stride elements,
+ * unit column stride; codes: [rows, dim] contiguous; scales: [rows] fp32.
+ * dim % 8 == 0, dim <= 32768; x rows and codes rows 16-byte aligned.
+ */
+int q8_quant_rows(const void* x, int x_dtype, void* codes, int code_dtype, float* scales,
+                  int64_t rows, int dim, int64_t x_row_stride, int flags, q8_stream_t stream);
+
+/*
+ * Fast Walsh-Hadamard transform along the last dimension.
+ * Replaces ops._C.fast_hadamard_transform  (csrc/fast_hadamard/fast_hadamard_transform.cpp:70-121,
+ * kernel csrc/fast_hadamard/fast_hadamard_transform_cuda.cu:43-111).
+ *   y[r,:] = (H_N [x[r,:], 0...0])[:dim] * scale,  N = 2^ceil(log2 dim), H_N Sylvester;
+ *   butterflies in fp32 with ascending stride; cast to y_dtype (E4M3: RNE, |v| > 464 -> NaN).
+ * x_dtype, y_dtype in {BF16, E4M3}; dim % 8 == 0, dim <= 32768; rows contiguous
+ * (row stride = dim); x and y 16-byte aligned.
+ */
+int q8_fht(const void* x, int x_dtype, void* y, int y_dtype, int64_t rows, int dim, float scale,
+           q8_stream_t stream);
+
+/*
+ * RMSNorm forward.
+ * Replaces ops._C.rms_norm  (csrc/ops/rms_norm.cpp:103-154, kernel csrc/ops/rms_norm_cuda.cu:101-171).
+ *   rstd[r] = rsqrt(mean_j x[r,j]^2 + eps);  y[r,j] = (x[r,j] * rstd[r]) * w[j]   (w NULL = no affine)
+ *   The reference has no eps: pass eps = 0 for identical results.
+ * x_dtype, y_dtype in {BF16, E4M3}; w fp32 [dim] or NULL; rstd fp32 [rows] or NULL.
+ * dim % 8 == 0, dim <= 32768; rows contiguous.
+ */
+int q8_rmsnorm(const void* x, int x_dtype, const float* w, void* y, int y_dtype, float* rstd,
+               int64_t rows, int dim, float eps, q8_stream_t stream);
+
+/*
+ * Rotary embedding with full-shape tables.
+ * Replaces ops._C.rope  (csrc/ops/rope.cpp:96-146, kernel csrc/ops/rope_cuda.cu:68-106).
+ *   y[r,2i]   = x[r,2i]  *cos[r,2i]   - x[r,2i+1]*sin[r,2i]
+ *   y[r,2i+1] = x[r,2i+1]*cos[r,2i+1] + x[r,2i]  *sin[r,2i+1]
+ * x_dtype, y_dtype in {BF16, E4M3}; cos, sin fp32 [rows, dim]; dim % 8 == 0; rows contiguous.
+ */
+int q8_rope(const void* x, int x_dtype, const float* cos_t, const float* sin_t, void* y, int y_dtype,
+            int64_t rows, int dim, q8_stream_t stream);
+
+/*
+ * 8-bit GEMM with fused dequantisation, bias and tanh-GELU.
+ * Replaces gemm._C.q8_mm / q8_mm_bias / fp8_mm / fp8_mm_bias
+ * (csrc/gemm/q8_gemm_api.cpp:40-291; kernels csrc/gemm/{q8,fp8}_matmul{,_bias}.cu).
+ *   acc[z,m,n] = sum_k A[za,m,k] * B[zb,n,k]            (int32 exact for I8, fp32 for E4M3)
+ *   v = float(acc) * (sa[za*M+m] * sb[zb*N+n]) (+ bias[n]);  if fuse_gelu: v = gelu_tanh(v)
+ *   C[z,m,n] = bf16(v)  or  e4m3(v) saturating to +-448
+ * A: [batch_a, M, K], B: [batch_b, N, K] contiguous, both K-major; batch_a == batch_b or either == 1
+ * (the operand with batch 1 is broadcast); C: [max(batch_a,batch_b), M, N] contiguous.
+ * in_dtype in {I8, E4M3}; out_dtype in {BF16, E4M3}; bias fp32 [N] or NULL.
+ * K % 16 == 0 and A, B 16-byte aligned; M, N arbitrary (> 0); N % 8 == 0 for BF16 output rows to stay
+ * 16-byte aligned, N % 16 == 0 for E4M3 output.
+ */
+int q8_gemm(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C,
+            int batch_a, int batch_b, int M, int N, int K, int in_dtype, int out_dtype, int fuse_gelu,
+            q8_stream_t stream);
+
+/*
+ * Raw int32 accumulators of the int8 GEMM, C[m,n] = sum_k A[m,k]*B[n,k], for bit-exact checks.
+ * Same mainloop as q8_gemm with in_dtype = Q8_I8 (csrc/gemm/q8_matmul.cu:109-, accumulators
+ * before the float conversion at q8_matmul_bias.cu:315-320).
+ */
+int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int K, q8_stream_t stream);
+
+/*
+ * FP8 FlashAttention-2 forward, head dim 64, non-causal, optional per-batch valid KV length.
+ * Replaces flash_attention._C.flash_attention
+ * (csrc/flash_attention/flash_attention.cpp:18-48; kernels flash_attention_cuda.cu:254-534 and
+ * flash_attention_cuda_mask.cu:254-535).
+ *   s[i,j] = (q_i . k_j) * softmax_scale * (sq[i]*sk[j] if given);  keys j >= kv_len[b] (or >= N) masked
+ *   p[i,j] = exp(s[i,j] - max_j s[i,j]);  l_i = sum_j p[i,j]  (fp32, unrounded unless SUM_ROUNDED_P)
+ *   o_i = (sum_j e4m3_sat(p[i,j]) * v_j * (sv[j] if given)) / l_i;   rows with l_i == 0 or NaN divide by 1
+ *   O = bf16(o) or e4m3_sat(o)
+ * q: [B,H,M,64] e4m3; k: [B,H,N,64] e4m3; v: e4m3 in v_layout; o: [B,H,M,64] of out_dtype.
+ * kv_len: int32 [B] or NULL; sq: fp32 [B,H,M], sk, sv: fp32 [B,H,N] per-token dequantisation scales
+ * or NULL (all three given or none). D must be 64. softmax_scale is the plain (natural-log) scale.
+ */
+int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int32_t* kv_len,
+                const float* sq, const float* sk, const float* sv,
+                int B, int H, int M, int N, int D, int v_layout, int64_t v_row_stride,
+                float softmax_scale, int out_dtype, int flags, q8_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* Q8_HIP_H */

@@ -1,0 +1,283 @@
+"""Tensor-level entry points with the names, argument order and return shapes of the reference's four
+pybind11 modules (q8_kernels_cuda.{gemm,quantizer,ops,flash_attention}._C), implemented on top of the
+C ABI of libq8_hip.so. Outputs are allocated here with torch (as the reference's C++ glue does), inputs
+are borrowed, launches go to the current torch stream of the input's device and do not synchronise.
+"""
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from ._lib import Q8_BF16, Q8_E4M3, Q8_F16, Q8_F32, Q8_I8
+
+_DT = {
+    torch.int8: Q8_I8,
+    torch.float8_e4m3fn: Q8_E4M3,
+    torch.bfloat16: Q8_BF16,
+    torch.float16: Q8_F16,
+    torch.float32: Q8_F32,
+}
+
+
+def _dt(dtype, who):
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise RuntimeError("%s not implemented for type '%s'" % (who, dtype))
+
+
+def _require_gpu(t, name):
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA (HIP) tensor" % name)
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _as_rows(x):
+    """x.reshape(-1, dim) with unit last stride (csrc/quantizer/tokenwise_quant.cpp:79-82)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
+    return x2
+
+
+# ----------------------------------------------------------------------------- quantizer._C
+
+def tokenwise_quant(x: torch.Tensor, out_type: Optional[torch.dtype] = None, *, round_half_even: bool = False,
+                    scale_as_division: bool = False) -> List[torch.Tensor]:
+    """csrc/quantizer/tokenwise_quant.cpp:74-111. Returns [codes(x.shape), scales(x.shape[:-1]) fp32].
+
+    out_type None -> int8. The two keyword flags select the documented variants of the arithmetic
+    (int8 round-half-even; stored scale absmax/QMAX); the defaults reproduce the reference.
+    """
+    _require_gpu(x, "x")
+    shape = x.shape
+    x2 = _as_rows(x)
+    out_type = torch.int8 if out_type is None else out_type
+    if out_type not in (torch.int8, torch.float8_e4m3fn):
+        raise RuntimeError("tokenwise_quant not implemented for output type '%s'" % out_type)
+    rows, dim = x2.shape
+    out = torch.empty((rows, dim), dtype=out_type, device=x.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    flags = (_lib.Q8_QUANT_RNE if round_half_even else 0) | (_lib.Q8_QUANT_SCALE_DIV if scale_as_division else 0)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_quant_rows(x2.data_ptr(), _dt(x2.dtype, "tokenwise_quant"), out.data_ptr(),
+                                            _dt(out_type, "tokenwise_quant"), scales.data_ptr(), rows, dim,
+                                            x2.stride(0) if rows > 1 else dim, flags, _stream(x)))
+    return [out.reshape(shape), scales.reshape(shape[:-1])]
+
+
+# ----------------------------------------------------------------------------- ops._C
+
+def fast_hadamard_transform(x: torch.Tensor, scale: float, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/fast_hadamard/fast_hadamard_transform.cpp:70-121. out_type None -> x.dtype."""
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("fast_hadamard_transform: input must be bfloat16 or float8_e4m3fn")
+    _require_gpu(x, "x")
+    shape = x.shape
+    dim_og = shape[-1]
+    x2 = x.reshape(-1, dim_og)
+    if dim_og % 8 != 0:
+        if x2.dtype == torch.float8_e4m3fn:
+            x2 = torch.nn.functional.pad(x2.view(torch.uint8), (0, 8 - dim_og % 8)).view(torch.float8_e4m3fn)
+        else:
+            x2 = torch.nn.functional.pad(x2, (0, 8 - dim_og % 8))
+    x2 = x2.contiguous()
+    rows, dim = x2.shape
+    if dim > 32768:
+        raise RuntimeError("fast_hadamard_transform only supports hidden dimension at most 32768 for now")
+    out_type = x.dtype if out_type is None else out_type
+    if out_type not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("fast_hadamard_transform: output must be bfloat16 or float8_e4m3fn")
+    out = torch.empty((rows, dim), dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_fht(x2.data_ptr(), _DT[x2.dtype], out.data_ptr(), _DT[out_type], rows, dim,
+                                     float(scale), _stream(x)))
+    if dim_og % 8 != 0:
+        out = out[:, :dim_og]
+    return out.reshape(shape)
+
+
+def rms_norm(x: torch.Tensor, weights: Optional[torch.Tensor] = None, out_type: Optional[torch.dtype] = None, *,
+             eps: float = 0.0) -> List[torch.Tensor]:
+    """csrc/ops/rms_norm.cpp:103-154. Returns [y(x.shape), rstd(x.shape[:-1]) fp32]; no epsilon by default."""
+    _require_gpu(x, "x")
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("rms_norm: input must be bfloat16 or float8_e4m3fn")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).contiguous()
+    rows, dim = x2.shape
+    out_type = x.dtype if out_type is None else out_type
+    if out_type not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("rms_norm: output must be bfloat16 or float8_e4m3fn")
+    if weights is not None:
+        if weights.dtype != torch.float32 or not weights.is_cuda:
+            raise RuntimeError("rms norm: weights error")
+        if weights.numel() != dim:
+            raise RuntimeError("rms norm: weights must have %d elements" % dim)
+        weights = weights.contiguous()
+    out = torch.empty((rows, dim), dtype=out_type, device=x.device)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_rmsnorm(x2.data_ptr(), _DT[x2.dtype], _ptr(weights), out.data_ptr(), _DT[out_type],
+                                         rstd.data_ptr(), rows, dim, float(eps), _stream(x)))
+    return [out.reshape(shape), rstd.reshape(shape[:-1])]
+
+
+def rope(x: torch.Tensor, cos_freqs: torch.Tensor, sin_freqs: torch.Tensor,
+         out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/rope.cpp:96-146: interleaved-pair rotation with fp32 tables of x's shape."""
+    if cos_freqs.dtype != torch.float32 or sin_freqs.dtype != torch.float32:
+        raise RuntimeError("rope: cos/sin tables must be float32")
+    _require_gpu(x, "x")
+    _require_gpu(cos_freqs, "cos_freqs")
+    _require_gpu(sin_freqs, "sin_freqs")
+    if cos_freqs.shape != x.shape or sin_freqs.shape != x.shape:
+        raise RuntimeError("rope: cos/sin tables must have the shape of x")
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("rope: input must be bfloat16 or float8_e4m3fn")
+    shape = x.shape
+    dim = shape[-1]
+    x2 = x.reshape(-1, dim).contiguous()
+    c2 = cos_freqs.reshape(-1, dim).contiguous()
+    s2 = sin_freqs.reshape(-1, dim).contiguous()
+    out_type = x.dtype if out_type is None else out_type
+    if out_type not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("rope: output must be bfloat16 or float8_e4m3fn")
+    out = torch.empty(x2.shape, dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_rope(x2.data_ptr(), _DT[x2.dtype], c2.data_ptr(), s2.data_ptr(), out.data_ptr(),
+                                      _DT[out_type], x2.shape[0], dim, _stream(x)))
+    return out.reshape(shape)
+
+
+# ----------------------------------------------------------------------------- gemm._C
+
+def _check_input(t, name):
+    _require_gpu(t, name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+
+
+def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who):
+    """Shape rules of csrc/gemm/q8_gemm_api.cpp:45-91: a [.,M,K], b [.,N,K], result always [batch,M,N]."""
+    _check_input(a, "a")
+    _check_input(b, "b")
+    if a.dtype != in_dtype or b.dtype != in_dtype:
+        raise RuntimeError("%s: a and b must be %s" % (who, in_dtype))
+    if a.dim() not in (2, 3) or b.dim() not in (2, 3):
+        raise RuntimeError("%s: a and b must be 2-D or 3-D" % who)
+    bs_a, m = (a.shape[0], a.shape[1]) if a.dim() == 3 else (1, a.shape[0])
+    bs_b, n = (b.shape[0], b.shape[1]) if b.dim() == 3 else (1, b.shape[0])
+    k = a.shape[-1]
+    if b.shape[-1] != k:
+        raise RuntimeError("%s: K mismatch (%d vs %d)" % (who, k, b.shape[-1]))
+    if not (bs_a == bs_b or bs_a == 1 or bs_b == 1):
+        raise RuntimeError("Batch missmatch")
+    batch = max(bs_a, bs_b)
+    out_type = torch.float8_e4m3fn if out_type is None else out_type
+    if out_type not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("%s: out_type must be bfloat16 or float8_e4m3fn, got %s" % (who, out_type))
+    for t, name, cnt in ((a_scales, "a_scales", bs_a * m), (b_scales, "b_scales", bs_b * n)):
+        _check_input(t, name)
+        if t.dtype != torch.float32 or t.numel() != cnt:
+            raise RuntimeError("%s: %s must be float32 with %d elements" % (who, name, cnt))
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.dtype != torch.float32 or bias.numel() != n:
+            raise RuntimeError("%s: bias must be float32 with %d elements" % (who, n))
+    out = torch.empty((batch, m, n), dtype=out_type, device=a.device)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().q8_gemm(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
+                                      out.data_ptr(), bs_a, bs_b, m, n, k, _DT[in_dtype], _DT[out_type],
+                                      1 if fuse_gelu else 0, _stream(a)))
+    return out
+
+
+def q8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/gemm/q8_gemm_api.cpp:40-97."""
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm")
+
+
+def q8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/gemm/q8_gemm_api.cpp:100-164."""
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm_bias")
+
+
+def fp8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/gemm/q8_gemm_api.cpp:167-224."""
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm")
+
+
+def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/gemm/q8_gemm_api.cpp:227-291."""
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias")
+
+
+def q8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Raw int32 accumulators a @ b.T of the int8 GEMM mainloop (2-D operands), for bit-exact checks."""
+    _check_input(a, "a")
+    _check_input(b, "b")
+    if a.dtype != torch.int8 or b.dtype != torch.int8 or a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise RuntimeError("q8_mm_i32: a [M,K] and b [N,K] must be int8 with equal K")
+    out = torch.empty((a.shape[0], b.shape[0]), dtype=torch.int32, device=a.device)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().q8_gemm_i32(a.data_ptr(), b.data_ptr(), out.data_ptr(), a.shape[0], b.shape[0], a.shape[1],
+                                          _stream(a)))
+    return out
+
+
+# ----------------------------------------------------------------------------- flash_attention._C
+
+def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
+                    batch_mask: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
+                    q_scales: Optional[torch.Tensor] = None, k_scales: Optional[torch.Tensor] = None,
+                    v_scales: Optional[torch.Tensor] = None, sum_rounded_p: bool = False) -> torch.Tensor:
+    """csrc/flash_attention/flash_attention.cpp:18-48.
+
+    q [B,H,M,64], k [B,H,N,64], v [B,H,64,Nv] (pre-transposed, Nv >= N, Nv % 16 == 0), all e4m3 and contiguous;
+    batch_mask int32 [B] of valid KV lengths. Returns [B,H,M,64] in out_dtype (None -> e4m3 like the reference).
+    The keyword arguments are extensions: bf16 output and per-token dequantisation scales
+    (q_scales [B,H,M], k_scales / v_scales [B,H,N], fp32).
+    """
+    for t, name in ((q, "q"), (k, "k"), (v, "v")):
+        _check_input(t, name)
+        if t.dtype != torch.float8_e4m3fn or t.dim() != 4:
+            raise RuntimeError("flash_attention: %s must be a 4-D float8_e4m3fn tensor" % name)
+    bs, heads, m, d = q.shape
+    n = k.shape[2]
+    if k.shape[0] != bs or k.shape[1] != heads or k.shape[3] != d:
+        raise RuntimeError("flash_attention: k shape mismatch")
+    if v.shape[0] != bs or v.shape[1] != heads or v.shape[2] != d or v.shape[3] < n:
+        raise RuntimeError("flash_attention: v must be [B,H,D,Nv] with Nv >= N")
+    if batch_mask is not None:
+        if batch_mask.dtype != torch.int32:
+            raise RuntimeError("flash attn: mask type error")
+        if batch_mask.dim() != 1 or batch_mask.shape[0] != bs:
+            raise RuntimeError("flash attn: mask batch error")
+        _check_input(batch_mask, "batch_mask")
+    scales = (q_scales, k_scales, v_scales)
+    if any(s is not None for s in scales):
+        if any(s is None for s in scales):
+            raise RuntimeError("flash_attention: q_scales, k_scales and v_scales must be given together")
+        for s, cnt, name in ((q_scales, bs * heads * m, "q_scales"), (k_scales, bs * heads * n, "k_scales"),
+                             (v_scales, bs * heads * n, "v_scales")):
+            _check_input(s, name)
+            if s.dtype != torch.float32 or s.numel() != cnt:
+                raise RuntimeError("flash_attention: %s must be float32 with %d elements" % (name, cnt))
+    out_dtype = torch.float8_e4m3fn if out_dtype is None else out_dtype
+    if out_dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("flash_attention: out_dtype must be bfloat16 or float8_e4m3fn")
+    out = torch.empty((bs, heads, m, d), dtype=out_dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().q8_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(batch_mask),
+                                          _ptr(q_scales), _ptr(k_scales), _ptr(v_scales), bs, heads, m, n, d,
+                                          _lib.Q8_V_DS, v.shape[3], float(softmax_scale), _DT[out_dtype],
+                                          _lib.Q8_ATTN_SUM_ROUNDED_P if sum_rounded_p else 0, _stream(q)))
+    return out

@@ -1,0 +1,77 @@
+"""Multi-head attention over Q8Linear projections (reference: q8_kernels/modules/attention.py:15-106).
+
+attn_type 'q8_kernels' runs the fp8 flash-attention kernel, 'torch' (the reference's default) runs
+torch SDPA in `non_mm_precision`."""
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from .. import functional as Q8F
+from .linear import Q8Linear
+from .rms_norm import RMSNorm
+
+
+class Attention(nn.Module):
+    def __init__(self, query_dim: int, num_heads: int, head_dim: int, bias: bool = False, out_bias: bool = False,
+                 out_dim: Optional[int] = None, qk_rms_norm: bool = False, kv_dim: Optional[int] = None,
+                 use_rope: bool = False):
+        super().__init__()
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.query_dim = query_dim
+        self.bias = bias
+        self.out_bias = out_bias
+        self.inner_dim = num_heads * head_dim
+        self.qk_rms_norm = qk_rms_norm
+        if qk_rms_norm:
+            self.q_norm = RMSNorm(self.inner_dim)
+            self.k_norm = RMSNorm(self.inner_dim)
+        self.use_rope = use_rope
+        kv_dim = query_dim if kv_dim is None else kv_dim
+        out_dim = query_dim if out_dim is None else out_dim
+        self.to_q = Q8Linear(query_dim, self.inner_dim, bias=bias)
+        self.to_k = Q8Linear(kv_dim, self.inner_dim, bias=bias)
+        self.to_v = Q8Linear(kv_dim, self.inner_dim, bias=bias)
+        self.to_out = Q8Linear(self.inner_dim, out_dim, out_bias)
+
+    def _split_heads(self, t, batch):
+        return t.view(batch, -1, self.num_heads, self.head_dim).transpose(1, 2)
+
+    def forward(self, hidden_states, freqs_cis=None, encoder_hidden_states=None, attention_mask=None,
+                non_mm_precision=torch.bfloat16, mm_out_dtype=None, apply_qk_hadamard=True, attn_type="torch"):
+        if attention_mask is not None and attention_mask.ndim > 1 and attn_type == "q8_kernels":
+            # [B, Skv] 0/1 mask -> valid lengths, the reference's rule (first zero; an all-ones row gives 0)
+            attention_mask = attention_mask.argmin(-1).squeeze().int()
+
+        kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
+        query = self.to_q(hidden_states, out_dtype=mm_out_dtype)
+        key = self.to_k(kv_src, out_dtype=mm_out_dtype)
+        value = self.to_v(kv_src, out_dtype=mm_out_dtype)
+        if self.qk_rms_norm:
+            query = self.q_norm(query, non_mm_precision)
+            key = self.k_norm(key, non_mm_precision)
+        if encoder_hidden_states is None and self.use_rope:
+            query = Q8F.rope.apply_rope(query, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)
+            key = Q8F.rope.apply_rope(key, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)
+
+        batch = query.shape[0]
+        query, key, value = (self._split_heads(t, batch) for t in (query, key, value))
+
+        if attn_type == "q8_kernels":
+            hidden_states = Q8F.flash_attention.flash_attn_func(query, key, value, batch_mask=attention_mask,
+                                                                apply_qk_hadamard=apply_qk_hadamard)
+        elif attn_type == "torch":
+            query, key, value = (t.to(non_mm_precision) for t in (query, key, value))
+            if attention_mask is not None:
+                # [batch] valid lengths -> additive [batch, heads, 1, keys] mask
+                pos = torch.arange(key.shape[2], device=query.device).expand(batch, -1)
+                add = torch.where(pos < attention_mask.unsqueeze(-1), 0.0, float("-inf"))
+                attention_mask = add[:, None, None, :].expand(-1, self.num_heads, -1, -1).to(query.dtype)
+            hidden_states = torch.nn.functional.scaled_dot_product_attention(
+                query, key, value, attn_mask=attention_mask, dropout_p=0.0, is_causal=False)
+        else:
+            raise ValueError(f"Invalid attention type: {attn_type}")
+
+        hidden_states = hidden_states.transpose(1, 2).reshape(batch, -1, self.inner_dim).contiguous()
+        return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)

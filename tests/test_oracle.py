@@ -1,0 +1,357 @@
+"""Pins the CPU oracle (oracle/q8_oracle.py) against independent closed forms. The reference ships no
+tests or golden vectors, so every oracle function is checked against something that does not share its
+formula: the e4m3 bit layout, scipy's Hadamard matrix, integer matmul, torch's own gelu/SDPA, complex
+rotation, brute-force loops on tiny inputs."""
+import math
+
+import numpy as np
+import pytest
+import scipy.linalg
+import torch
+
+from oracle import q8_oracle as O
+
+E4M3 = torch.float8_e4m3fn
+
+
+# ------------------------------------------------------------------ e4m3 casts
+
+def _nearest_e4m3_bruteforce(vals):
+    """RNE to the e4m3fn grid by exhaustive search over the 254 finite codes (ties -> even mantissa)."""
+    table = O.e4m3_decode_table()
+    finite = [(table[c], c) for c in range(256) if not np.isnan(table[c])]
+    out = []
+    for v in vals:
+        if np.isnan(v):
+            out.append(None)
+            continue
+        best, best_codes = None, []
+        for t, c in finite:
+            d = abs(float(v) - t)
+            if best is None or d < best:
+                best, best_codes = d, [c]
+            elif d == best:
+                best_codes.append(c)
+        if len(best_codes) > 1:
+            # zero has two codes; otherwise pick the even mantissa
+            nz = [c for c in best_codes if table[c] != 0 or True]
+            even = [c for c in nz if (c & 1) == 0]
+            sign = 0x80 if np.signbit(v) else 0
+            even = [c for c in even if (c & 0x80) == sign] or even
+            best_codes = even
+        out.append(best_codes[0])
+    return out
+
+
+def test_e4m3_decode_table_matches_torch():
+    codes = torch.arange(256, dtype=torch.uint8)
+    t = codes.view(E4M3).to(torch.float64).numpy()
+    ref = O.e4m3_decode_table()
+    assert np.array_equal(np.isnan(t), np.isnan(ref))
+    assert np.array_equal(t[~np.isnan(t)], ref[~np.isnan(ref)])
+    assert ref[0x7E] == 448.0 and ref[0x01] == 2.0 ** -9 and ref[0x08] == 2.0 ** -6
+
+
+def test_e4m3_c10_is_rne_with_nan_above_464():
+    g = torch.Generator().manual_seed(1)
+    vals = torch.cat([
+        torch.randn(400, generator=g) * 3,
+        torch.randn(200, generator=g) * 200,
+        torch.randn(200, generator=g) * 0.01,
+        torch.tensor([0.0, -0.0, 448.0, -448.0, 464.0, -464.0, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -10, 1.0625, 1.1875, 0.0009765625]),
+    ]).to(torch.float32)
+    got = O.e4m3_c10(vals).view(torch.uint8).numpy()
+    inside = vals.abs() <= 464.0
+    want = _nearest_e4m3_bruteforce(vals[inside].numpy())
+    table = O.e4m3_decode_table()
+    for g_code, w_code, v in zip(got[inside.numpy()], want, vals[inside].numpy()):
+        assert table[g_code] == table[w_code], (v, g_code, w_code)
+    # above 464: NaN code with the sign kept
+    big = torch.tensor([464.0001, 465.0, 480.0, 1e6, -465.0, float("inf"), float("nan")], dtype=torch.float32)
+    codes = O.e4m3_c10(big).view(torch.uint8).tolist()
+    assert codes == [0x7F, 0x7F, 0x7F, 0x7F, 0xFF, 0x7F, 0x7F]
+
+
+def test_e4m3_sat_clamps_and_keeps_nan():
+    x = torch.tensor([500.0, -1e9, 448.0, 463.0, 3.0, float("nan"), float("inf")], dtype=torch.float32)
+    codes = O.e4m3_sat(x).view(torch.uint8).tolist()
+    assert codes[:5] == [0x7E, 0xFE, 0x7E, 0x7E, 0x44]
+    assert codes[5] & 0x7F == 0x7F and codes[6] == 0x7E
+
+
+# ------------------------------------------------------------------ FHT
+
+@pytest.mark.parametrize("dim", [8, 16, 64, 128, 512, 2048, 4096])
+def test_fht_matches_scipy_hadamard(dim):
+    g = torch.Generator().manual_seed(dim)
+    x = torch.randn(5, dim, generator=g).to(torch.bfloat16)
+    H = torch.tensor(scipy.linalg.hadamard(dim), dtype=torch.float64)
+    want = x.to(torch.float64) @ H / math.sqrt(dim)
+    got = O.ref_fht(x, out_type=torch.bfloat16)
+    # the docstring equivalence of the reference (fast_hadamard.py:33), up to bf16 rounding of the output
+    assert torch.equal(got, (want.to(torch.float32)).to(torch.bfloat16)) or \
+        (got.to(torch.float64) - want).abs().max() <= 2 ** -7 * want.abs().max()
+    # exact on small integers (every partial sum is exactly representable)
+    xi = torch.randint(-3, 4, (4, dim), generator=g).to(torch.bfloat16)
+    got_i = O.ref_fht(xi, scale=1.0, out_type=torch.bfloat16).to(torch.float64)
+    want_i = (xi.to(torch.float64) @ H).to(torch.float32).to(torch.bfloat16).to(torch.float64)
+    assert torch.equal(got_i, want_i)
+
+
+def test_fht_involution_and_parseval():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(3, 256, generator=g)
+    xb = x.to(torch.bfloat16)
+    # run in fp32 without the bf16 store in between: emulate by feeding exactly representable values
+    y = O.ref_fht(xb, out_type=torch.bfloat16)
+    e_in = (xb.to(torch.float64) ** 2).sum(-1)
+    e_out = (y.to(torch.float64) ** 2).sum(-1)
+    assert torch.allclose(e_in, e_out, rtol=2e-2)
+    z = O.ref_fht(y, out_type=torch.bfloat16)
+    assert (z.to(torch.float64) - xb.to(torch.float64)).abs().max() < 0.05
+
+
+@pytest.mark.parametrize("dim", [24, 40, 100, 1536])
+def test_fht_zero_pads_to_next_power_of_two(dim):
+    g = torch.Generator().manual_seed(dim)
+    x = torch.randint(-2, 3, (3, dim), generator=g).to(torch.bfloat16)
+    n = 1 << (dim - 1).bit_length()
+    H = torch.tensor(scipy.linalg.hadamard(n), dtype=torch.float64)
+    xp = torch.zeros(3, n, dtype=torch.float64)
+    xp[:, :dim] = x.to(torch.float64)
+    want = (xp @ H)[:, :dim]
+    got = O.ref_fht(x, scale=1.0, out_type=torch.bfloat16).to(torch.float64)
+    assert torch.equal(got, want.to(torch.float32).to(torch.bfloat16).to(torch.float64))
+
+
+def test_fht_fp8_output_uses_c10_cast():
+    x = torch.full((1, 64), 30.0).to(torch.bfloat16)
+    y = O.ref_fht(x, scale=1.0, out_type=E4M3).view(torch.uint8)
+    assert y[0, 0].item() == 0x7F  # 1920 > 464 -> NaN, not saturation
+    assert (y[0, 1:] == 0).all()
+
+
+# ------------------------------------------------------------------ quantizer
+
+@pytest.mark.parametrize("out_type,qmax", [(torch.int8, 127.0), (E4M3, 448.0)])
+def test_quant_closed_form_properties(out_type, qmax):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(16, 256, generator=g).to(torch.bfloat16)
+    codes, scales = O.ref_quant(x, out_type)
+    assert codes.shape == x.shape and scales.shape == x.shape[:-1] and scales.dtype == torch.float32
+    a = x.float().abs().amax(-1)
+    # scale * QMAX = absmax up to 1 ulp of the two fp32 divisions
+    assert torch.allclose(scales * qmax, a, rtol=3e-7)
+    deq = codes.to(torch.float32) * scales[:, None]
+    step = scales[:, None] * (1.0 if out_type == torch.int8 else 32.0)  # e4m3 step at the top binade is 32
+    assert ((deq - x.float()).abs() <= 0.5 * step + 1e-6).all()
+    # the absmax element maps to +-QMAX exactly
+    idx = x.float().abs().argmax(-1)
+    top = codes.to(torch.float32)[torch.arange(16), idx]
+    assert (top.abs() == qmax).all()
+
+
+def test_quant_rounding_modes_and_zero_row():
+    # x*r lands exactly on .5 -> half-away vs half-even differ
+    x = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -2.5, 0.0, 3.0]], dtype=torch.float32)
+    away, s = O.ref_quant(x, torch.int8)
+    even, _ = O.ref_quant(x, torch.int8, round_half_even=True)
+    assert away.tolist() == [[127, 1, 2, 3, -1, -3, 0, 3]]
+    assert even.tolist() == [[127, 0, 2, 2, 0, -2, 0, 3]]
+    assert s.item() == 1.0
+    z = torch.zeros(2, 8, dtype=torch.bfloat16)
+    for t in (torch.int8, E4M3):
+        c, sc = O.ref_quant(z, t)
+        assert (c.view(torch.uint8) == 0).all() and (sc == 0).all()
+
+
+def test_quant_scale_forms_agree_to_one_ulp():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(64, 64, generator=g).to(torch.bfloat16)
+    c1, s1 = O.ref_quant(x, E4M3)
+    c2, s2 = O.ref_quant(x, E4M3, scale_as_division=True)
+    assert torch.equal(c1.view(torch.uint8), c2.view(torch.uint8))
+    ulp = torch.abs(s1) * 2 ** -23
+    assert ((s1 - s2).abs() <= ulp).all()
+    assert torch.equal(s2, x.float().abs().amax(-1) / 448.0)
+
+
+# ------------------------------------------------------------------ GEMM
+
+def test_gemm_i32_exact_against_integer_matmul():
+    g = torch.Generator().manual_seed(11)
+    a = torch.randint(-128, 128, (37, 96), generator=g, dtype=torch.int8)
+    b = torch.randint(-128, 128, (29, 96), generator=g, dtype=torch.int8)
+    want = a.numpy().astype(np.int64) @ b.numpy().astype(np.int64).T
+    got = O.ref_gemm_i32(a, b)
+    assert got.dtype == torch.int32 and np.array_equal(got.numpy().astype(np.int64), want)
+    # worst case magnitude stays exact
+    a2 = torch.full((2, 4096), -128, dtype=torch.int8)
+    assert O.ref_gemm_i32(a2, a2)[0, 0].item() == 128 * 128 * 4096
+
+
+def test_gemm_fp8_acc_matches_bruteforce():
+    g = torch.Generator().manual_seed(12)
+    a = O.e4m3_c10(torch.randn(5, 32, generator=g) * 4)
+    b = O.e4m3_c10(torch.randn(6, 32, generator=g) * 4)
+    tab = O.e4m3_decode_table()
+    av, bv = tab[a.view(torch.uint8).numpy()], tab[b.view(torch.uint8).numpy()]
+    want = np.array([[sum(av[i, k] * bv[j, k] for k in range(32)) for j in range(6)] for i in range(5)])
+    assert np.allclose(O.ref_gemm_fp8_acc(a, b).numpy(), want, rtol=0, atol=1e-9)
+
+
+def test_epilogue_matches_torch_gelu_and_casts():
+    g = torch.Generator().manual_seed(13)
+    acc = torch.randint(-20000, 20000, (2, 7, 9), generator=g, dtype=torch.int32)
+    sa = torch.rand(2, 7, generator=g) * 1e-2
+    sb = torch.rand(1, 9, generator=g) * 1e-2
+    bias = torch.randn(9, generator=g)
+    v = acc.double() * (sa.float()[..., :, None] * sb.float()[..., None, :]).double() + bias.double()
+    want = torch.nn.functional.gelu(v, approximate="tanh")
+    got = O.ref_epilogue(acc, sa, sb, bias, True, torch.bfloat16)
+    assert got.dtype == torch.bfloat16
+    assert (got.double() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-6
+    # no gelu, e4m3 default output saturates
+    big = O.ref_epilogue(torch.tensor([[[10 ** 6, -10 ** 6, 3]]]), torch.ones(1, 1), torch.ones(1, 3), None, False, None)
+    assert big.dtype == E4M3 and big.view(torch.uint8).tolist() == [[[0x7E, 0xFE, 0x44]]]
+
+
+def test_mm_batch_broadcast_shapes():
+    g = torch.Generator().manual_seed(14)
+    a = torch.randint(-5, 6, (3, 4, 16), generator=g, dtype=torch.int8)
+    b = torch.randint(-5, 6, (8, 16), generator=g, dtype=torch.int8)
+    sa, sb = torch.ones(3, 4), torch.ones(8)
+    out = O.ref_q8_mm(a, b, None, sa, sb, False, torch.bfloat16)
+    assert out.shape == (3, 4, 8)
+    want = torch.einsum("zmk,nk->zmn", a.double(), b.double())
+    assert torch.equal(out.double(), want)
+    out2 = O.ref_q8_mm(a[0], b, None, sa[0], sb, False, torch.bfloat16)
+    assert out2.shape == (1, 4, 8)
+
+
+def test_linear_compositions_reduce_to_plain_matmul():
+    """(xH)(WH)^T = xW^T for the orthonormal rotation: both linears approximate the bf16 linear."""
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(2, 16, 128, generator=g).to(torch.bfloat16)
+    w = (torch.randn(32, 128, generator=g) * 0.05).to(torch.bfloat16)
+    bias = torch.randn(32, generator=g) * 0.1
+    want = x.double() @ w.double().T + bias.double()
+    for out in (O.ref_q8_linear(x, w, bias, out_dtype=torch.bfloat16),
+                O.ref_fp8_linear(x, w, bias, out_dtype=torch.bfloat16),
+                O.ref_fp8_linear(x, w, bias, use_hadamard=True, out_dtype=torch.bfloat16)):
+        assert out.shape == (2, 16, 32)
+        cos = torch.nn.functional.cosine_similarity(out.double().flatten(), want.flatten(), dim=0)
+        assert cos > 0.995
+
+
+# ------------------------------------------------------------------ attention
+
+def test_attention_unrounded_equals_torch_sdpa():
+    g = torch.Generator().manual_seed(21)
+    q = O.e4m3_c10(torch.randn(2, 3, 40, 64, generator=g))
+    k = O.e4m3_c10(torch.randn(2, 3, 50, 64, generator=g))
+    v = O.e4m3_c10(torch.randn(2, 3, 50, 64, generator=g))
+    lens = torch.tensor([50, 17], dtype=torch.int32)
+    got = O.ref_attention(q, k, v, 0.125, lens, round_p=False)
+    keep = torch.arange(50)[None, :] < lens[:, None]
+    mask = torch.zeros(2, 1, 1, 50, dtype=torch.float64).masked_fill(~keep[:, None, None, :], float("-inf"))
+    want = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), attn_mask=mask, scale=0.125)
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_attention_rounded_p_invariants():
+    g = torch.Generator().manual_seed(22)
+    q = O.e4m3_c10(torch.randn(1, 2, 33, 64, generator=g))
+    k = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
+    v = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
+    lens = torch.tensor([41], dtype=torch.int32)
+    o = O.ref_attention(q, k, v, 0.125, lens)
+    exact = O.ref_attention(q, k, v, 0.125, lens, round_p=False)
+    # e4m3 rounding of p is a <= 2^-4 relative perturbation of each weight
+    assert (o - exact).abs().max() < 0.07
+    # masked keys carry no weight: changing them changes nothing
+    v2 = v.clone().view(torch.uint8)
+    v2[:, :, 41:, :] = 0x7E
+    k2 = k.clone().view(torch.uint8)
+    k2[:, :, 41:, :] = 0x30
+    o2 = O.ref_attention(q, k2.view(E4M3), v2.view(E4M3), 0.125, lens)
+    assert torch.equal(o, o2)
+    # fully masked batch -> zeros (l = 0 divides by 1)
+    oz = O.ref_attention(q, k, v, 0.125, torch.tensor([0], dtype=torch.int32))
+    assert (oz == 0).all()
+    # per-token scales are plain dequantisation
+    sq, sk, sv = torch.rand(1, 2, 33, generator=g) + 0.5, torch.rand(1, 2, 70, generator=g) + 0.5, torch.rand(1, 2, 70, generator=g) + 0.5
+    os_ = O.ref_attention(q, k, v, 0.125, lens, sq, sk, sv, round_p=False)
+    want = O.ref_attention(q.double() * sq[..., None], k.double() * sk[..., None], v.double() * sv[..., None], 0.125, lens, round_p=False)
+    assert torch.allclose(os_, want, atol=1e-10)
+
+
+def test_flash_attn_func_hadamard_identity():
+    """(Hq).(Hk)/D = q.k: with the rotation the result approximates plain attention on the bf16 inputs."""
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(1, 2, 48, 64, generator=g).to(torch.bfloat16)
+    k = torch.randn(1, 2, 80, 64, generator=g).to(torch.bfloat16)
+    v = torch.randn(1, 2, 80, 64, generator=g).to(torch.bfloat16)
+    want = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double())
+    for had in (False, True):
+        o = O.ref_flash_attn_func(q, k, v, apply_qk_hadamard=had, out_dtype=torch.bfloat16)
+        assert o.shape == q.shape and o.dtype == torch.bfloat16
+        cos = torch.nn.functional.cosine_similarity(o.double().flatten(), want.flatten(), dim=0)
+        assert cos > 0.99
+    assert O.ref_flash_attn_func(q, k, v).dtype == E4M3
+
+
+# ------------------------------------------------------------------ RMSNorm / RoPE / tables
+
+def test_rms_norm_closed_form():
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(6, 128, generator=g).to(torch.bfloat16)
+    w = torch.rand(128, generator=g) + 0.5
+    y, rstd = O.ref_rms_norm(x, w, torch.bfloat16)
+    xd = x.double()
+    want_r = 1.0 / np.sqrt((xd.numpy() ** 2).mean(-1))
+    assert np.allclose(rstd.numpy(), want_r, rtol=1e-6)
+    want = xd * torch.tensor(want_r)[:, None] * w.double()
+    assert (y.double() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-6
+    y1, _ = O.ref_rms_norm(x, None, None)
+    assert y1.dtype == torch.bfloat16
+    # unit RMS after normalisation
+    assert torch.allclose((y1.double() ** 2).mean(-1), torch.ones(6, dtype=torch.float64), atol=2e-2)
+
+
+def test_rope_is_complex_rotation():
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(2, 5, 32, generator=g).to(torch.bfloat16)
+    ang = torch.rand(2, 5, 16, generator=g) * 6.28
+    cos = ang.cos().repeat_interleave(2, -1)
+    sin = ang.sin().repeat_interleave(2, -1)
+    y = O.ref_rope(x, cos, sin, torch.bfloat16)
+    z = torch.view_as_complex(x.float().reshape(2, 5, 16, 2).contiguous()) * torch.polar(torch.ones_like(ang), ang)
+    want = torch.view_as_real(z).reshape(2, 5, 32)
+    assert (y.float() - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-6
+    # per-element tables: the odd/even entries may differ, follow the formula literally
+    cos2, sin2 = torch.randn(1, 1, 4, generator=g), torch.randn(1, 1, 4, generator=g)
+    xx = torch.tensor([[[1.0, 2.0, 3.0, 4.0]]]).to(torch.bfloat16)
+    yy = O.ref_rope(xx, cos2, sin2, torch.bfloat16).float()[0, 0]
+    c, s = cos2[0, 0], sin2[0, 0]
+    want2 = torch.stack([1 * c[0] - 2 * s[0], 2 * c[1] + 1 * s[1], 3 * c[2] - 4 * s[2], 4 * c[3] + 3 * s[3]])
+    assert torch.equal(yy, want2.to(torch.bfloat16).float())
+
+
+def test_freqs_cis_against_loops():
+    dim, theta, max_pos = 26, 100.0, (20, 2048, 2048)
+    grid = torch.tensor([[[0.0, 3.0], [5.0, 100.0], [7.0, 2047.0]]])  # [1, 3, 2]
+    cos, sin = O.ref_freqs_cis(grid, dim, theta, max_pos)
+    assert cos.shape == (1, 2, dim) and cos.dtype == torch.float32
+    nf = dim // 6
+    for t in range(2):
+        assert cos[0, t, 0] == 1 and cos[0, t, 1] == 1 and sin[0, t, 0] == 0 and sin[0, t, 1] == 0  # dim % 6 = 2 pad
+        for f in range(nf):
+            w = theta ** (f / (nf - 1)) * math.pi / 2
+            for axis in range(3):
+                frac = grid[0, axis, t].item() / max_pos[axis]
+                a = w * (2 * frac - 1)
+                col = 2 + 2 * (f * 3 + axis)
+                assert abs(cos[0, t, col].item() - math.cos(a)) < 1e-5
+                assert cos[0, t, col] == cos[0, t, col + 1]
+                assert abs(sin[0, t, col].item() - math.sin(a)) < 1e-5
