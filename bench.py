@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the 8-bit hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A "step" is one launch of the headline kernel on resident synthetic data: the fp8 e4m3 GEMM with fused
+per-token / per-channel dequantisation + bias + tanh-GELU at M=6144, N=8192, K=2048 (bf16 output).
+After W warm-up steps exactly K steps are timed between two device synchronisations; the one JSON line
+printed at the end carries that throughput as `value` (TFLOP/s), the roofline of the kernel measured with
+HIP events on the launch stream, a CPU baseline (the torch oracle of the same semantics on the host
+cores, bounded sample), and in `extras` the other workloads of the metric: fp8 Hadamard self-attention
+(S=6144, D=64), cross-attention with a padding mask, the int8 GEMM, the memory-bound row kernels and the
+DiT block in milliseconds.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 / int8 MFMA, published (no sparsity)
+HBM_PEAK_GBS = 8000.0
+E4M3 = torch.float8_e4m3fn
+
+
+def _time(fn, steps, warmup):
+    """Mean seconds per call over exactly `steps` calls (HIP events on the current stream, which is the
+    stream the library launches on)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return start.elapsed_time(stop) * 1e-3 / steps, wall
+
+
+def _gemm_inputs(dev, m, n, k, seed=0):
+    from q8_kernels_amd import _C
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=g) * 0.02).to(torch.bfloat16).float()
+    xq, sx = _C.tokenwise_quant(x.to(dev), E4M3)
+    wq, sw = _C.tokenwise_quant(w.to(dev), E4M3)
+    return x, w, bias, xq, sx, wq, sw
+
+
+def _cpu_baseline_gemm(x, w, bias, budget_s=20.0):
+    """The oracle's fp8 linear + bias + GELU (quantize, dequantize to fp32, torch.matmul, tanh-GELU, bf16) on the
+    host cores, full-size problem, as many repeats as fit the budget (at least one)."""
+    from oracle import q8_oracle as O
+    threads = torch.get_num_threads()
+    xq, sx = O.ref_quant(x, E4M3)
+    wq, sw = O.ref_quant(w, E4M3)
+
+    def run():
+        acc = xq.to(torch.float32) @ wq.to(torch.float32).T
+        v = acc * (sx[:, None] * sw[None, :]) + bias
+        return torch.nn.functional.gelu(v, approximate="tanh").to(torch.bfloat16)
+
+    run()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 and (not times or time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sec = sorted(times)[len(times) // 2]
+    flop = 2.0 * x.shape[0] * w.shape[0] * x.shape[1]
+    return {"value": flop / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "full %dx%dx%d fp8 linear+bias+GELU (dequantised fp32 torch.matmul), median of %d runs, %.2f s each"
+                      % (x.shape[0], w.shape[0], x.shape[1], len(times), sec)}
+
+
+def _extras(dev, steps, warmup):
+    from q8_kernels_amd import _C
+    from q8_kernels_amd.blocks import Fp8DiTBlock
+    from oracle import q8_oracle as O
+    out = {}
+    g = torch.Generator().manual_seed(1)
+    # fp8 self-attention with Hadamard, per-token e4m3 (config 3) and reference-style direct casts
+    B, H, S = 2, 32, 6144
+    q, k, v = (torch.randn(B, H, S, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+    qr, kr = _C.fast_hadamard_transform(q, 0.125, torch.bfloat16), _C.fast_hadamard_transform(k, 0.125, torch.bfloat16)
+    (q8, sq), (k8, sk), (v8, sv) = _C.tokenwise_quant(qr, E4M3), _C.tokenwise_quant(kr, E4M3), _C.tokenwise_quant(v, E4M3)
+    vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
+    flop = 4.0 * B * H * S * S * 64
+    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk,
+                                            v_scales=sv), steps, warmup)
+    out["attn_self_fp8_per_token_scales"] = {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS,
+                                             "shape": "B2 H32 S6144 D64"}
+    s = (1 / 64) ** 0.5 * (0.125 ** 0.5)
+    qd, kd = _C.fast_hadamard_transform(q, s, E4M3), _C.fast_hadamard_transform(k, s, E4M3)
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16), steps, warmup)
+    out["attn_self_fp8_reference_casts"] = {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS,
+                                            "shape": "B2 H32 S6144 D64"}
+    # cross-attention with a padding mask (config 4): HBM-bound
+    N = 128
+    kx, vx = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
+    lens = torch.randint(16, 129, (B,), generator=g, dtype=torch.int32).to(dev)
+    kx8 = _C.fast_hadamard_transform(kx, s, E4M3)
+    vxt = vx.to(E4M3).view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
+    t, _ = _time(lambda: _C.flash_attention(qd, kx8, vxt, 1.0, lens, out_dtype=torch.bfloat16), steps, warmup)
+    byts = B * H * (S * 64 + 2 * N * 64 + S * 64 * 2)
+    out["attn_cross_fp8_masked"] = {"ms": t * 1e3, "gbs": byts / t / 1e9, "frac_of_hbm_peak": byts / t / 1e9 / HBM_PEAK_GBS,
+                                    "tflops": 4.0 * B * H * S * N * 64 / t / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64"}
+    # int8 GEMM (config 2)
+    a = torch.randint(-127, 128, (6144, 2048), generator=g, dtype=torch.int8).to(dev)
+    b = torch.randint(-127, 128, (2048, 2048), generator=g, dtype=torch.int8).to(dev)
+    sa, sb, bias = torch.rand(6144, generator=g).to(dev), torch.rand(2048, generator=g).to(dev), torch.randn(2048, generator=g).to(dev)
+    t, _ = _time(lambda: _C.q8_mm_bias(a, b, bias, sa, sb, False, torch.bfloat16), steps, warmup)
+    out["int8_gemm_6144x2048x2048"] = {"ms": t * 1e3, "tops": 2.0 * 6144 * 2048 * 2048 / t / 1e12}
+    # row kernels on [12288, 2048] tokens
+    x = torch.randn(12288, 2048, generator=g).to(torch.bfloat16).to(dev)
+    n = x.numel()
+    cos, sin = torch.randn(12288, 2048, generator=g).to(dev), torch.randn(12288, 2048, generator=g).to(dev)
+    w = torch.ones(2048, device=dev)
+    for name, fn, bpe in (("quant_fp8", lambda: _C.tokenwise_quant(x, E4M3), 3), ("quant_int8", lambda: _C.tokenwise_quant(x, None), 3),
+                          ("fht_bf16", lambda: _C.fast_hadamard_transform(x, 2048 ** -0.5, None), 4),
+                          ("rmsnorm_bf16", lambda: _C.rms_norm(x, w, None), 4), ("rope_bf16", lambda: _C.rope(x, cos, sin, None), 12)):
+        t, _ = _time(fn, steps, warmup)
+        out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    # the DiT block (config 5)
+    blk = Fp8DiTBlock(device=dev).init_random()
+    hidden = torch.randn(2, 6144, 2048, generator=g).to(torch.bfloat16).to(dev)
+    text = torch.randn(2, 128, 2048, generator=g).to(torch.bfloat16).to(dev)
+    f, hh, ww = 16, 16, 24
+    grid = torch.stack(torch.meshgrid(torch.arange(f), torch.arange(hh), torch.arange(ww), indexing="ij")).reshape(3, -1)
+    cosf, sinf = (t_.to(dev) for t_ in O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), 2048))
+    with torch.no_grad():
+        t, _ = _time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
+    out["dit_block"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12, "shape": "tokens [2,6144,2048], text [2,128,2048]"}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing on this path communicates "
+              "between GPUs)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from q8_kernels_amd import _C, _lib
+    _lib.lib()  # fail loudly if the HIP library has not been built
+    dev = torch.device("cuda:0")
+    M, N, K = 6144, 8192, 2048
+    x, w, bias, xq, sx, wq, sw = _gemm_inputs(dev, M, N, K)
+    bias_d = bias.to(dev)
+    step = lambda: _C.fp8_mm_bias(xq, wq, bias_d, sx, sw, True, torch.bfloat16)  # noqa: E731
+    sec, wall = _time(step, args.steps, args.warmup)
+    flop = 2.0 * M * N * K
+    tflops = flop / sec / 1e12
+    result = {
+        "metric": "fp8 GEMM & fp8 attn TFLOPS at LTX shapes, % of gfx950 MFMA peak; block ms",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {"workload": "fp8 e4m3 GEMM + per-token/per-channel dequant + bias + tanh-GELU -> bf16, M=6144 N=8192 K=2048",
+                   "inputs": "X~N(0,1), W~N(0,0.02), bias~N(0,0.02), per-row absmax e4m3 quantisation, resident in HBM"},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / FP8_PEAK_TFLOPS,
+                     "traffic": None, "kernel": "gemm_kernel<e4m3, bf16, gelu>", "flop_per_launch": flop,
+                     "avg_launch_us": sec * 1e6, "host_wall_us_per_step": wall * 1e6},
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "gemm_fp8_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as fh:
+            result["roofline"]["traffic"] = json.load(fh).get("hbm_bytes_per_launch")
+    if not args.no_cpu:
+        result["cpu_baseline"] = _cpu_baseline_gemm(x, w, bias)
+    else:
+        result["cpu_baseline"] = None
+    if not args.no_extras:
+        result["extras"] = _extras(dev, args.steps, args.warmup)
+        a = result["extras"]["attn_self_fp8_per_token_scales"]
+        result["attn_tflops"] = a["tflops"]
+        result["attn_frac_of_fp8_peak"] = a["frac_of_fp8_peak"]
+        result["block_ms"] = result["extras"]["dit_block"]["ms"]
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

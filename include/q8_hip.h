@@ -136,6 +136,13 @@ int q8_gemm(const void* A, const void* B, const float* bias, const float* sa, co
             q8_stream_t stream);
 
 /*
+ * Tile-shape override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = 256x256 tiles,
+ * 2 = 128x128 tiles. Process-wide; meant for tests and tuning, it has no counterpart in the reference
+ * (whose tile is fixed at 128x128x64, csrc/gemm/fp8_matmul_bias.cu:426-429).
+ */
+int q8_gemm_set_config(int cfg);
+
+/*
  * Raw int32 accumulators of the int8 GEMM, C[m,n] = sum_k A[m,k]*B[n,k], for bit-exact checks.
  * Same mainloop as q8_gemm with in_dtype = Q8_I8 (csrc/gemm/q8_matmul.cu:109-, accumulators
  * before the float conversion at q8_matmul_bias.cu:315-320).
@@ -149,7 +156,8 @@ int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int 
  * flash_attention_cuda_mask.cu:254-535).
  *   s[i,j] = (q_i . k_j) * softmax_scale * (sq[i]*sk[j] if given);  keys j >= kv_len[b] (or >= N) masked
  *   p[i,j] = exp(s[i,j] - max_j s[i,j]);  l_i = sum_j p[i,j]  (fp32, unrounded unless SUM_ROUNDED_P)
- *   o_i = (sum_j e4m3_sat(p[i,j]) * v_j * (sv[j] if given)) / l_i;   rows with l_i == 0 or NaN divide by 1
+ *   o_i = (sum_j e4m3_sat(p[i,j]) * v_j) / l_i;   rows with l_i == 0 or NaN divide by 1
+ *   with sv: o_i = svmax * (sum_j e4m3_sat(p[i,j] * sv[j] / svmax) * v_j) / l_i,  svmax = max_{j valid} sv[j]
  *   O = bf16(o) or e4m3_sat(o)
  * q: [B,H,M,64] e4m3; k: [B,H,N,64] e4m3; v: e4m3 in v_layout; o: [B,H,M,64] of out_dtype.
  * kv_len: int32 [B] or NULL; sq: fp32 [B,H,M], sk, sv: fp32 [B,H,N] per-token dequantisation scales

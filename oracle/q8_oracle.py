@@ -226,17 +226,21 @@ def ref_fp8_linear(a, b, bias=None, scale_a=None, scale_b=None, use_hadamard=Fal
 
 def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                   kv_len: Optional[torch.Tensor] = None, sq=None, sk=None, sv=None,
-                  round_p: bool = True, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+                  round_p: bool = True, out_dtype: Optional[torch.dtype] = None, return_weighted_abs: bool = False):
     """Attention on e4m3 operands as the reference kernel defines it (csrc/flash_attention/
     flash_attention_cuda.cu:171-248,437,487-497; mask: flash_attention_cuda_mask.cu:244,319):
         s_ij = (q_i . k_j) * scale (* sq_i sk_j);  keys j >= kv_len[b] masked;
         p_ij = exp(s_ij - max_j s_ij);  l_i = sum_j p_ij (unrounded);
-        o_i = sum_j e4m3_sat(p_ij (* sv_j)) v_j / l_i;  rows with l_i == 0 are divided by 1.
+        o_i = sum_j e4m3_sat(p_ij) v_j / l_i;  rows with l_i == 0 are divided by 1.
+    Per-token dequantisation scales (an extension, the reference kernel has unit scales): V's scale enters
+    P before its cast as sv_j / max_j sv_j and the common factor is applied to o_i.
     q [B,H,M,D], k, v [B,H,N,D] (v NOT transposed here). With round_p=False this is plain fp32-style
     softmax attention on the dequantised inputs (evaluated in float64), the accuracy target of the
     BASELINE configs. out_dtype None returns float64; bf16 -> RNE; e4m3 -> saturating cast.
     The online kernel rounds p against the running maximum, so its P-hat differs from this one in the
-    last e4m3 bit here and there: comparisons carry a tolerance."""
+    last e4m3 bit here and there: comparisons carry a tolerance. With return_weighted_abs the function also
+    returns sum_j p_ij |v_j| / l_i: any rounding of the weights by a relative eps moves o_i by at most eps
+    times that, which is the rigorous error bound the tests use (eps = 2^-4 for e4m3)."""
     qd, kd, vd = q.to(torch.float64), k.to(torch.float64), v.to(torch.float64)
     s = qd @ kd.transpose(-1, -2) * softmax_scale
     if sq is not None:
@@ -249,11 +253,23 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
     m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
     p = torch.exp(s - m)
     l = p.sum(dim=-1, keepdim=True)
-    pv = p if sv is None else p * sv.to(torch.float64).unsqueeze(-2)
+    pv, sv_ref = p, None
+    if sv is not None:
+        svd = sv.to(torch.float64)
+        if kv_len is not None:
+            svd = torch.where(keep[:, None, :], svd, torch.zeros_like(svd))
+        sv_ref = svd.amax(dim=-1, keepdim=True)
+        pv = p * (svd / torch.where(sv_ref > 0, sv_ref, torch.ones_like(sv_ref))).unsqueeze(-2)
     if round_p:
         pv = e4m3_sat(pv.to(torch.float32)).to(torch.float64)
     o = pv @ vd
-    o = o / torch.where(l == 0, torch.ones_like(l), l)
+    if sv_ref is not None:
+        o = o * sv_ref.unsqueeze(-1)
+    lsafe = torch.where(l == 0, torch.ones_like(l), l)
+    o = o / lsafe
+    if return_weighted_abs:
+        vabs = vd.abs() if sv is None else vd.abs() * sv.to(torch.float64).unsqueeze(-1)
+        return o, (p @ vabs) / lsafe
     if out_dtype is None:
         return o
     if out_dtype == E4M3:
@@ -338,3 +354,39 @@ def ref_freqs_cis(indices_grid: torch.Tensor, dim: int = 2048, theta: float = 10
         cos = torch.cat([torch.ones_like(cos[:, :, : dim % 6]), cos], dim=-1)
         sin = torch.cat([torch.zeros_like(cos[:, :, : dim % 6]), sin], dim=-1)
     return cos.to(torch.float32), sin.to(torch.float32)
+
+
+# ------------------------------------------------------------------------------------------- block composition
+
+
+def ref_dit_block(hidden, text, freqs_cis, text_lens, params, num_heads, head_dim=64):
+    """The simplified LTX-style fp8 block of the benchmark configuration, composed from the functions above
+    (op order as q8_kernels/modules/attention.py:45-106 and q8_kernels/modules/ffn.py:10-17 chain them):
+    RMSNorm -> fp8 QKV -> RoPE(q, k) -> fp8 Hadamard self-attention -> out projection (+res) -> RMSNorm ->
+    fp8 cross-attention with valid lengths (+res) -> RMSNorm -> fp8 FFN with fused bias+GELU (+res).
+    `params[name]` = (e4m3 weight [out, in], fp32 scales [out], fp32 bias [out]); `params['norm*']` = fp32 [dim]."""
+    bf16 = torch.bfloat16
+    b = hidden.shape[0]
+    dim = num_heads * head_dim
+
+    def lin(name, x, gelu=False):
+        w, s, bias = params[name]
+        return ref_fp8_linear(x, w, bias, None, s, False, bf16, fuse_gelu=gelu)
+
+    def heads(t):
+        return t.reshape(b, -1, num_heads, head_dim).transpose(1, 2)
+
+    def merge(t):
+        return t.transpose(1, 2).reshape(b, -1, dim)
+
+    h, _ = ref_rms_norm(hidden, params["norm1"])
+    q, k, v = lin("to_qkv", h).split(dim, dim=-1)
+    q, k = ref_rope(q, *freqs_cis), ref_rope(k, *freqs_cis)
+    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, None, True, out_dtype=bf16)
+    hidden = hidden + lin("to_out", merge(a))
+    h, _ = ref_rms_norm(hidden, params["norm2"])
+    a = ref_flash_attn_func(heads(lin("to_q2", h)), heads(lin("to_k2", text)), heads(lin("to_v2", text)), None, text_lens, True,
+                            out_dtype=bf16)
+    hidden = hidden + lin("to_out2", merge(a))
+    h, _ = ref_rms_norm(hidden, params["norm3"])
+    return hidden + lin("ff_down", lin("ff_up", h, gelu=True))

@@ -1,0 +1,76 @@
+"""An LTX-Video-style DiT block assembled from the fp8 ops of this package:
+
+    RMSNorm -> fp8 QKV linear -> 3-D RoPE on q, k -> fp8 Hadamard self-attention -> out projection (+ residual)
+    -> RMSNorm -> fp8 cross-attention to the text states with a per-batch valid length (+ residual)
+    -> RMSNorm -> fp8 FFN with bias + tanh-GELU fused into the first GEMM (+ residual)
+
+It is the simplified block of the benchmark configuration (hidden 2048, 32 heads x 64, FFN 8192), built
+on the same kernels that the reference's LTXTransformerBlock (q8_kernels/blocks/ltx_transformer_block.py:21-58)
+reaches through its modules; AdaLN modulation and the qk-RMSNorm of that block are not part of it.
+"""
+import torch
+import torch.nn as nn
+
+from .. import functional as Q8F
+from ..modules.linear import FP8Linear
+from ..modules.rms_norm import RMSNorm
+
+
+class Fp8DiTBlock(nn.Module):
+    def __init__(self, dim: int = 2048, num_heads: int = 32, head_dim: int = 64, ffn_dim: int = 8192,
+                 text_dim: int = 2048, device=None):
+        super().__init__()
+        assert num_heads * head_dim == dim
+        self.dim, self.num_heads, self.head_dim = dim, num_heads, head_dim
+        self.norm1, self.norm2, self.norm3 = (RMSNorm(dim, True, device) for _ in range(3))
+        mk = lambda i, o: FP8Linear(i, o, bias=True, device=device)  # noqa: E731
+        self.to_qkv = mk(dim, 3 * dim)
+        self.to_out = mk(dim, dim)
+        self.to_q2, self.to_k2, self.to_v2, self.to_out2 = mk(dim, dim), mk(text_dim, dim), mk(text_dim, dim), mk(dim, dim)
+        self.ff_up, self.ff_down = mk(dim, ffn_dim), mk(ffn_dim, dim)
+
+    @torch.no_grad()
+    def init_random(self, std: float = 0.02, seed: int = 0):
+        """Random weights ~ N(0, std) quantized per output channel to e4m3, biases ~ N(0, std) in fp32."""
+        g = torch.Generator().manual_seed(seed)
+        for m in self.modules():
+            if isinstance(m, FP8Linear):
+                dev = m.weight.device
+                w = (torch.randn(m.weight.shape, generator=g) * std).to(torch.bfloat16).to(dev)
+                m.weight.data, m.scales.data = Q8F.quantizer.quantize_fp8(w)
+                m.bias.data = (torch.randn(m.bias.shape, generator=g) * std).to(torch.bfloat16).float().to(dev)
+        return self
+
+    def _heads(self, t, b):
+        return t.view(b, -1, self.num_heads, self.head_dim).transpose(1, 2)
+
+    def _merge(self, t, b):
+        return t.transpose(1, 2).reshape(b, -1, self.dim)
+
+    def _lin(self, layer, x, fuse_gelu=False):
+        return Q8F.linear.fp8_linear(x, layer.weight.data, layer.bias.data, None, layer.scales, False, x.dtype,
+                                     fuse_gelu=fuse_gelu)
+
+    def forward(self, hidden, text, freqs_cis, text_lens):
+        b = hidden.shape[0]
+        bf16 = torch.bfloat16
+        # self-attention
+        h = self.norm1(hidden)
+        qkv = self._lin(self.to_qkv, h)
+        q, k, v = qkv.split(self.dim, dim=-1)
+        q = Q8F.rope.apply_rope(q.contiguous(), freqs_cis[0], freqs_cis[1])
+        k = Q8F.rope.apply_rope(k.contiguous(), freqs_cis[0], freqs_cis[1])
+        a = Q8F.flash_attention.flash_attn_func(self._heads(q, b), self._heads(k, b), self._heads(v, b),
+                                                apply_qk_hadamard=True, out_dtype=bf16)
+        hidden = hidden + self._lin(self.to_out, self._merge(a, b))
+        # cross-attention to the text states
+        h = self.norm2(hidden)
+        q2 = self._lin(self.to_q2, h)
+        k2, v2 = self._lin(self.to_k2, text), self._lin(self.to_v2, text)
+        a = Q8F.flash_attention.flash_attn_func(self._heads(q2, b), self._heads(k2, b), self._heads(v2, b),
+                                                batch_mask=text_lens, apply_qk_hadamard=True, out_dtype=bf16)
+        hidden = hidden + self._lin(self.to_out2, self._merge(a, b))
+        # feed-forward
+        h = self.norm3(hidden)
+        up = self._lin(self.ff_up, h, fuse_gelu=True)
+        return hidden + self._lin(self.ff_down, up)

@@ -115,6 +115,21 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     for (int t = 0; t < kQT; ++t) { m_run[t] = -INFINITY; l_run[t] = 0.f; }
 
     const int n_tiles = (valid + kKV - 1) / kKV;
+
+    // per-token V scales enter P before its e4m3 cast as sv[j] / max_j sv[j] (<= 1, so the product stays in the
+    // normal range of e4m3); the common factor max_j sv[j] is applied to O at the end.
+    float sv_ref = 1.f, sv_inv = 1.f;
+    if constexpr (SCALED) {
+        __shared__ float red[kWaves];
+        float mx = 0.f;
+        for (int j = tid; j < valid; j += kWaves * 64) mx = fmaxf(mx, p.sv[(size_t)bh * N + j]);
+        mx = group_max<64>(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        sv_ref = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        sv_inv = sv_ref > 0.f ? 1.0f / sv_ref : 0.f;
+    }
+
     if (n_tiles > 0) issue_loads(0, 0);
     for (int it = 0; it < n_tiles; ++it) {
         const int kv0 = it * kKV;
@@ -141,7 +156,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                 int key = kv0 + 32 * h + e;
                 key = key < N ? key : N - 1;
                 skv[e] = p.sk[(size_t)bh * N + key];
-                svv[e] = p.sv[(size_t)bh * N + key];
+                svv[e] = p.sv[(size_t)bh * N + key] * sv_inv;
             }
         }
         const bool partial = kv0 + kKV > valid;
@@ -214,7 +229,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     for (int qt = 0; qt < kQT; ++qt) {
         const int row = q0 + 32 * qt + ql;
         float l = l_run[qt] + lane_xor<32>(l_run[qt]);
-        const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
+        const float inv = ((l == 0.f || l != l) ? 1.f : 1.f / l) * sv_ref;
         if (row >= M) continue;
 #pragma unroll
         for (int d = 0; d < 2; ++d) {

@@ -1,0 +1,146 @@
+"""GPU tests of the Python surface (functional + modules + block) against the oracle's compositions."""
+import pytest
+import torch
+
+from oracle import q8_oracle as O
+from tests.util import E4M3, assert_bit_equal, cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def test_quantize_and_hadamard_functions(dev):
+    import q8_kernels_amd.functional as Q8F
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 17, 2048, generator=g).to(torch.bfloat16)
+    c, s = Q8F.quantizer.quantize(x.to(dev))
+    oc, os_ = O.ref_quant(x)
+    assert c.dtype == torch.int8 and c.shape == x.shape and s.shape == x.shape[:-1]
+    assert_bit_equal(c, oc, "quantize codes")
+    assert_bit_equal(s, os_, "quantize scales")
+    c, s = Q8F.quantizer.quantize_fp8(x.to(dev))
+    oc, os_ = O.ref_quant(x, E4M3)
+    assert_bit_equal(c, oc, "quantize_fp8 codes")
+    assert_bit_equal(s, os_, "quantize_fp8 scales")
+    y = Q8F.fast_hadamard.hadamard_transform(x.to(dev))
+    assert_bit_equal(y, O.ref_fht(x), "hadamard_transform default scale")
+    y = Q8F.fast_hadamard.hadamard_transform(x.to(dev), scale=0.5, out_type=E4M3)
+    assert_bit_equal(y, O.ref_fht(x, 0.5, E4M3), "hadamard_transform -> e4m3")
+    y = Q8F.rms_norm.rms_norm_8bit(x.to(dev), torch.ones(2048, device=dev))
+    assert y.dtype == torch.bfloat16 and cosine(y.cpu(), O.ref_rms_norm(x, torch.ones(2048))[0]) > 0.99999
+    cos, sin = torch.randn(3, 17, 2048, generator=g), torch.randn(3, 17, 2048, generator=g)
+    assert_bit_equal(Q8F.rope.apply_rope(x.to(dev), cos.to(dev), sin.to(dev)), O.ref_rope(x, cos, sin), "apply_rope")
+
+
+def test_q8_linear_matches_oracle_composition(dev):
+    from q8_kernels_amd.functional.linear import q8_linear
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, 50, 512, generator=g).to(torch.bfloat16)
+    w = (torch.randn(320, 512, generator=g) * 0.05).to(torch.bfloat16)
+    bias = torch.randn(320, generator=g) * 0.1
+    for fuse_gelu in (False, True):
+        got = q8_linear(x.to(dev), w.to(dev), bias.to(dev), fuse_gelu=fuse_gelu, out_dtype=torch.bfloat16)
+        want = O.ref_q8_linear(x, w, bias, fuse_gelu=fuse_gelu, out_dtype=torch.bfloat16)
+        assert got.shape == (2, 50, 320)
+        # identical int8 codes and int32 accumulators: only the last bf16 bit may differ (GELU uses exp2/rcp hardware)
+        d = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert d.max() <= 2 and (d > 0).float().mean() < 0.02
+    # pre-quantised operands with scales, default e4m3 output, 2-D activation -> leading batch of 1
+    wq, sw = O.ref_quant(O.ref_fht(w))
+    xq, sx = O.ref_quant(O.ref_fht(x[0]))
+    got = q8_linear(xq.to(dev), wq.to(dev), None, sx.to(dev), sw.to(dev))
+    assert got.dtype == E4M3 and got.shape == (1, 50, 320)
+    want = O.ref_q8_linear(xq, wq, None, sx, sw)
+    assert (got.cpu().view(torch.uint8) != want.view(torch.uint8)).float().mean() < 0.01
+
+
+def test_fp8_linear_matches_oracle_composition(dev):
+    from q8_kernels_amd.functional.linear import fp8_linear
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 33, 256, generator=g).to(torch.bfloat16)
+    w = (torch.randn(192, 256, generator=g) * 0.05).to(torch.bfloat16)
+    bias = torch.randn(192, generator=g) * 0.1
+    for had in (False, True):
+        got = fp8_linear(x.to(dev), w.to(dev), bias.to(dev), use_hadamard=had, out_dtype=torch.bfloat16)
+        want = O.ref_fp8_linear(x, w, bias, use_hadamard=had, out_dtype=torch.bfloat16)
+        assert got.shape == (4, 33, 192) and got.dtype == torch.bfloat16
+        d = (got.cpu().double() - want.double()).abs()
+        assert d.max() <= 2.0 ** -6 * want.double().abs().max()
+        assert cosine(got.cpu(), x.double() @ w.double().T + bias.double()) > 0.998
+
+
+def test_modules_state_dict_and_forward(dev):
+    import torch.nn as nn
+    from q8_kernels_amd.modules import FP8Linear, FeedForward, Q8Linear, RMSNorm
+    torch.manual_seed(0)
+    lin = nn.Linear(256, 128).to(dev).to(torch.bfloat16)
+    q8 = Q8Linear.from_linear(lin)
+    assert set(q8.state_dict().keys()) == {"weight", "bias", "scales"}
+    assert q8.weight.dtype == torch.int8 and q8.scales.dtype == torch.float32 and q8.bias.dtype == torch.float32
+    wq, sw = O.ref_quant(O.ref_fht(lin.weight.data.cpu()))
+    assert_bit_equal(q8.weight.data, wq, "Q8Linear.from_linear weight")
+    assert_bit_equal(q8.scales.data, sw, "Q8Linear.from_linear scales")
+    x = torch.randn(2, 9, 256, device=dev).to(torch.bfloat16)
+    y = q8(x, out_dtype=torch.bfloat16)
+    assert y.shape == (2, 9, 128) and cosine(y.cpu(), lin(x).cpu()) > 0.999
+    assert q8(x).dtype == E4M3  # the reference's default output type
+    f8 = FP8Linear.from_linear(lin, use_hadamard=True)
+    assert f8.weight.dtype == E4M3 and set(f8.state_dict().keys()) == {"weight", "bias", "scales"}
+    y = f8(x)
+    assert y.dtype == torch.bfloat16 and cosine(y.cpu(), lin(x).cpu()) > 0.998
+    # a converted state dict loads into a fresh module
+    fresh = Q8Linear(256, 128, device=dev)
+    fresh.load_state_dict(q8.state_dict())
+    assert torch.equal(fresh(x, out_dtype=torch.bfloat16), q8(x, out_dtype=torch.bfloat16))
+    norm = RMSNorm(256, device=dev)
+    assert norm.weight.dtype == torch.float32 and norm(x).dtype == torch.bfloat16
+    ff = FeedForward(256, mult=2).to(dev)
+    for m in (ff.act.proj, ff.proj_down):
+        src = nn.Linear(m.in_features, m.out_features).to(dev).to(torch.bfloat16)
+        q = Q8Linear.from_linear(src)
+        m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    assert ff(x, out_dtype=torch.bfloat16).shape == (2, 9, 256)
+
+
+def test_attention_module_kernel_path_agrees_with_sdpa_path(dev):
+    import torch.nn as nn
+    from q8_kernels_amd.modules import Attention, Q8Linear
+    torch.manual_seed(1)
+    attn = Attention(256, 4, 64, bias=True, out_bias=True, qk_rms_norm=True, kv_dim=192, use_rope=False).to(dev)
+    for name in ("to_q", "to_k", "to_v", "to_out"):
+        m = getattr(attn, name)
+        src = nn.Linear(m.in_features, m.out_features).to(dev).to(torch.bfloat16)
+        q = Q8Linear.from_linear(src)
+        m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    x = torch.randn(2, 70, 256, device=dev).to(torch.bfloat16)
+    ctx = torch.randn(2, 40, 192, device=dev).to(torch.bfloat16)
+    mask = torch.ones(2, 40, device=dev)
+    mask[0, 25:] = 0
+    mask[1, 39:] = 0
+    y_k = attn(x, encoder_hidden_states=ctx, attention_mask=mask, mm_out_dtype=torch.bfloat16, attn_type="q8_kernels")
+    lens = torch.tensor([25, 39], device=dev, dtype=torch.int32)
+    y_t = attn(x, encoder_hidden_states=ctx, attention_mask=lens, mm_out_dtype=torch.bfloat16, attn_type="torch")
+    assert y_k.shape == (2, 70, 256) and y_k.dtype == torch.bfloat16
+    assert cosine(y_k.cpu(), y_t.cpu()) > 0.99
+
+
+def test_dit_block_matches_oracle_block(dev):
+    from q8_kernels_amd.blocks import Fp8DiTBlock
+    from q8_kernels_amd.modules.linear import FP8Linear
+    dim, heads, ffn, s_tok, s_txt = 256, 4, 512, 96, 24
+    blk = Fp8DiTBlock(dim, heads, 64, ffn, dim, device=dev).init_random(std=0.05, seed=3)
+    g = torch.Generator().manual_seed(4)
+    hidden = torch.randn(2, s_tok, dim, generator=g).to(torch.bfloat16)
+    text = torch.randn(2, s_txt, dim, generator=g).to(torch.bfloat16)
+    grid = torch.stack(torch.meshgrid(torch.arange(4), torch.arange(4), torch.arange(6), indexing="ij")).reshape(3, -1)
+    cos, sin = O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim)
+    lens = torch.tensor([24, 9], dtype=torch.int32)
+    with torch.no_grad():
+        got = blk(hidden.to(dev), text.to(dev), (cos.to(dev), sin.to(dev)), lens.to(dev))
+    params = {n: (m.weight.data.cpu(), m.scales.data.cpu(), m.bias.data.cpu()) for n, m in blk.named_modules() if isinstance(m, FP8Linear)}
+    for n in ("norm1", "norm2", "norm3"):
+        params[n] = getattr(blk, n).weight.data.cpu()
+    want = O.ref_dit_block(hidden, text, (cos, sin), lens, params, heads)
+    assert got.shape == hidden.shape and got.dtype == torch.bfloat16
+    # end to end in bf16 with requantisation between ops: small differences get re-rounded along the way
+    assert cosine(got.cpu(), want) > 0.9995
+    assert (got.cpu().double() - want.double()).abs().max() <= 0.05 * want.double().abs().max()

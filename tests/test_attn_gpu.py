@@ -1,0 +1,186 @@
+"""GPU parity of the fp8 flash-attention forward against the float64 oracle.
+
+Tolerance, stated in _check: the element-wise bound that the e4m3 rounding of P implies (2^-4 of the
+probability-weighted mean of |V|), cosine >= 0.999 against unrounded attention on the dequantised inputs, and
+twice the bound against the oracle that rounds P."""
+import pytest
+import torch
+
+from oracle import q8_oracle as O
+from tests.util import E4M3, cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def _C():
+    from q8_kernels_amd import _C as C
+    return C
+
+
+def _vt(v8):
+    """[B,H,N,D] e4m3 -> the kernel's [B,H,D,Nv] layout, Nv = N rounded up to 16, zero padded."""
+    n = v8.shape[2]
+    nv = (n + 15) // 16 * 16
+    vt = torch.zeros(v8.shape[0], v8.shape[1], v8.shape[3], nv, dtype=torch.uint8)
+    vt[..., :n] = v8.view(torch.uint8).transpose(2, 3)
+    return vt.view(E4M3)
+
+
+def _inputs(seed, b, h, m, n, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = O.e4m3_c10(torch.randn(b, h, m, 64, generator=g) * std)
+    k = O.e4m3_c10(torch.randn(b, h, n, 64, generator=g) * std)
+    v = O.e4m3_c10(torch.randn(b, h, n, 64, generator=g))
+    return q, k, v
+
+
+def _check(got, q, k, v, scale, lens=None, sc=(None, None, None), what=""):
+    """Kernel output against float64 attention on the dequantised inputs.
+    Rigorous part: P is rounded to e4m3 (relative error <= 2^-4 per weight) before it multiplies V, so
+    |o - o_exact| <= 2^-4 * sum_j p_ij |v_j| / l_i, plus the bf16 rounding of the output (2^-8 |o|).
+    Statistical part: the rounding errors average out, cosine >= 0.999 and the mean error stays below a
+    quarter of the mean bound. Against the oracle that rounds P (relative to the final row maximum, the kernel
+    rounds relative to the running one) the distance is at most twice the bound."""
+    g = got.cpu().double()
+    exact, wabs = O.ref_attention(q, k, v, scale, lens, *sc, round_p=False, return_weighted_abs=True)
+    rounded = O.ref_attention(q, k, v, scale, lens, *sc, round_p=True)
+    assert not torch.isnan(g).any(), what
+    bound = 2.0 ** -4 * 1.02 * wabs + 2.0 ** -8 * exact.abs() + 1e-6
+    e_exact, e_round = (g - exact).abs(), (g - rounded).abs()
+    assert (e_exact <= bound).all(), "%s: max-abs vs exact %g exceeds the e4m3 rounding bound (worst ratio %g)" % (
+        what, e_exact.max().item(), (e_exact / bound).max().item())
+    assert (e_round <= 2 * bound).all(), "%s: max-abs vs rounded-P oracle %g" % (what, e_round.max().item())
+    if exact.abs().max() > 0:
+        assert e_exact.mean() <= 0.25 * bound.mean(), "%s: mean error %g vs mean bound %g" % (what, e_exact.mean().item(), bound.mean().item())
+        assert cosine(g, exact) >= 0.999, "%s: cosine %g" % (what, cosine(g, exact))
+
+
+@pytest.mark.parametrize("m,n", [(256, 64), (64, 128), (1, 1), (33, 17), (255, 100), (257, 200), (300, 640), (512, 1000)])
+def test_attention_shapes(dev, m, n):
+    q, k, v = _inputs(m * 1000 + n, 2, 3, m, n)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16)
+    assert got.shape == (2, 3, m, 64) and got.dtype == torch.bfloat16
+    _check(got, q, k, v, 0.125, what="m=%d n=%d" % (m, n))
+
+
+def test_attention_fp8_output_default(dev):
+    q, k, v = _inputs(5, 1, 2, 130, 300)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None)
+    assert got.dtype == E4M3
+    want = O.ref_attention(q, k, v, 0.125, None, out_dtype=E4M3)
+    g, w = got.cpu().float(), want.float()
+    assert not torch.isnan(g).any()
+    assert ((g - w).abs() <= 0.13 * w.abs() + 0.03).all()
+
+
+@pytest.mark.parametrize("lens", [[128, 16], [1, 64], [65, 127], [0, 100], [63, 200]])
+def test_attention_kv_length_mask(dev, lens):
+    n = 128
+    q, k, v = _inputs(sum(lens), 2, 4, 200, n)
+    kv_len = torch.tensor(lens, dtype=torch.int32)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, kv_len.to(dev), out_dtype=torch.bfloat16)
+    _check(got, q, k, v, 0.125, kv_len.clamp(max=n), what="lens=%s" % lens)
+    # masked keys and values have no influence at all
+    k2, v2 = k.clone().view(torch.uint8), v.clone().view(torch.uint8)
+    for b, ln in enumerate(lens):
+        k2[b, :, min(ln, n):] = 0x55
+        v2[b, :, min(ln, n):] = 0x7E
+    got2 = _C().flash_attention(q.to(dev), k2.view(E4M3).to(dev), _vt(v2.view(E4M3)).to(dev), 0.125, kv_len.to(dev),
+                                out_dtype=torch.bfloat16)
+    assert torch.equal(got.cpu().view(torch.int16), got2.cpu().view(torch.int16))
+    for b, ln in enumerate(lens):
+        if ln == 0:
+            assert (got[b].cpu().float() == 0).all()  # nothing to attend to: zeros
+
+
+def test_attention_large_logits_and_scale(dev):
+    q, k, v = _inputs(77, 1, 2, 128, 256, std=4.0)
+    for scale in (0.125, 0.02, 1.0):
+        got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), scale, None, out_dtype=torch.bfloat16)
+        _check(got, q, k, v, scale, what="scale=%g" % scale)
+
+
+def test_attention_per_token_scales(dev):
+    g = torch.Generator().manual_seed(9)
+    b, h, m, n = 2, 2, 150, 333
+    qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)
+    kf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 4 + 0.2)
+    vf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 2 + 0.5)
+    (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+    lens = torch.tensor([333, 77], dtype=torch.int32)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
+                               q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+    _check(got, q, k, v, 0.125, lens, (sq, sk, sv), what="per-token scales")
+    full = torch.nn.functional.scaled_dot_product_attention(
+        qf.double(), kf.double(), vf.double(),
+        attn_mask=torch.zeros(b, 1, 1, n, dtype=torch.float64).masked_fill(
+            ~(torch.arange(n)[None, :] < lens[:, None])[:, None, None, :], float("-inf")))
+    assert cosine(got.cpu(), full) > 0.99
+
+
+def test_attention_config3_self_attention_hadamard(dev):
+    """B=2, H=32, S=6144, D=64, non-causal; Q/K/V bf16 ~ N(0,1) with one head-dim channel scaled x20; Q and K
+    rotated by the normalised 64-point Hadamard transform, everything quantised per token to e4m3, softmax
+    scale 1/8, bf16 output. The whole problem runs on the GPU; the oracle checks four (batch, head) pairs."""
+    C = _C()
+    g = torch.Generator().manual_seed(3)
+    B, H, S = 2, 32, 6144
+    q, k, v = (torch.randn(B, H, S, 64, generator=g).to(torch.bfloat16) for _ in range(3))
+    for t in (q, k, v):
+        t[..., int(torch.randperm(64, generator=g)[0])] *= 20
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    qr, kr = C.fast_hadamard_transform(qd, 0.125, torch.bfloat16), C.fast_hadamard_transform(kd, 0.125, torch.bfloat16)
+    (q8, sq), (k8, sk), (v8, sv) = C.tokenwise_quant(qr, E4M3), C.tokenwise_quant(kr, E4M3), C.tokenwise_quant(vd, E4M3)
+    vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
+    out = C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv)
+    assert out.shape == (B, H, S, 64)
+    for (b, h) in [(0, 0), (0, 17), (1, 5), (1, 31)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        oq, osq = O.ref_quant(O.ref_fht(q[sl], 0.125, torch.bfloat16), E4M3)
+        ok, osk = O.ref_quant(O.ref_fht(k[sl], 0.125, torch.bfloat16), E4M3)
+        ov, osv = O.ref_quant(v[sl], E4M3)
+        assert torch.equal(q8[sl].cpu().view(torch.uint8), oq.view(torch.uint8))
+        assert torch.equal(sk[sl].cpu(), osk)
+        _check(out[sl], oq, ok, ov, 0.125, None, (osq, osk, osv), what="config 3 (b=%d,h=%d)" % (b, h))
+        plain = torch.nn.functional.scaled_dot_product_attention(q[sl].double(), k[sl].double(), v[sl].double())
+        assert cosine(out[sl].cpu(), plain) >= 0.999
+    # size-independent property at full size: every output row is a convex combination of V rows
+    vmax = (v8.float() * sv[..., None]).amax(dim=2, keepdim=True)
+    vmin = (v8.float() * sv[..., None]).amin(dim=2, keepdim=True)
+    o = out.float()
+    slack = 0.02 * (vmax - vmin) + 0.02
+    assert bool(((o <= vmax + slack) & (o >= vmin - slack)).all())
+
+
+def test_attention_config4_cross_attention_mask(dev):
+    """B=2, H=32, 6144 queries, 128 text keys, valid lengths drawn from 16..128, reference-style direct casts with
+    the Hadamard rotation (softmax scale folded into Q and K)."""
+    g = torch.Generator().manual_seed(4)
+    B, H, M, N = 2, 32, 6144, 128
+    q = torch.randn(B, H, M, 64, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16)
+    lens = torch.randint(16, 129, (B,), generator=g, dtype=torch.int32)
+    from q8_kernels_amd.functional.flash_attention import flash_attn_func
+    out = flash_attn_func(q.to(dev), k.to(dev), v.to(dev), None, lens.to(dev), True, out_dtype=torch.bfloat16)
+    assert out.shape == (B, H, M, 64)
+    s = (1 / 64) ** 0.5 * (0.125 ** 0.5)
+    q8, k8, v8 = O.ref_fht(q, s, E4M3), O.ref_fht(k, s, E4M3), O.e4m3_c10(v)
+    hs = slice(0, 32, 11)
+    _check(out[:, hs], q8[:, hs], k8[:, hs], v8[:, hs], 1.0, lens, what="config 4")
+    mask = torch.zeros(B, 1, 1, N, dtype=torch.float64).masked_fill(~(torch.arange(N)[None, :] < lens[:, None])[:, None, None, :], float("-inf"))
+    plain = torch.nn.functional.scaled_dot_product_attention(q[:, hs].double(), k[:, hs].double(), v[:, hs].double(), attn_mask=mask)
+    assert cosine(out[:, hs].cpu(), plain) >= 0.998  # accuracy of the direct e4m3 casts, not of the kernel
+
+
+def test_attention_rejects_bad_arguments(dev):
+    from q8_kernels_amd import Q8Error
+    q, k, v = _inputs(1, 1, 1, 16, 16)
+    vt = _vt(v)
+    with pytest.raises(RuntimeError):
+        _C().flash_attention(q.to(dev), k.to(dev), vt.to(dev), 0.125, torch.tensor([16], device=dev))  # int64 mask
+    with pytest.raises(RuntimeError):
+        _C().flash_attention(q.to(dev).float(), k.to(dev), vt.to(dev), 0.125, None)
+    q32 = O.e4m3_c10(torch.zeros(1, 1, 16, 32))
+    with pytest.raises(Q8Error):
+        _C().flash_attention(q32.to(dev), q32.to(dev), O.e4m3_c10(torch.zeros(1, 1, 32, 16)).to(dev), 0.125, None)

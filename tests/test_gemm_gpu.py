@@ -1,0 +1,185 @@
+"""GPU parity of the 8-bit GEMM: int32 accumulators bit-exact, dequantised outputs within a stated
+tolerance of the float64 oracle."""
+import pytest
+import torch
+
+from oracle import q8_oracle as O
+from tests.util import E4M3, assert_bit_equal, bf16_ulp, cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def _C():
+    from q8_kernels_amd import _C as C
+    return C
+
+
+def _set_cfg(c):
+    from q8_kernels_amd import _lib
+    _lib.check(_lib.lib().q8_gemm_set_config(c))
+
+
+@pytest.fixture(params=[1, 2], ids=["tile256", "tile128"])
+def tile_cfg(request):
+    _set_cfg(request.param)
+    yield request.param
+    _set_cfg(0)
+
+
+def _rand_i8(g, *shape):
+    return torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+
+
+def _check_float_out(got, want64, what):
+    """bf16 outputs: the kernel accumulates in fp32 (MFMA order) and uses the hardware exp2 / rcp for the
+    GELU, the oracle float64: allow 2 bf16 ulp plus 2^-9 of the row scale, and demand cosine >= 0.99999."""
+    g = got.cpu().double()
+    tol = 2 * bf16_ulp(want64) + 2.0 ** -9 * want64.abs().mean()
+    err = (g - want64).abs()
+    assert (err <= tol).all(), "%s: max err %g (tol %g at worst)" % (what, err.max().item(), tol[err.argmax()].item() if tol.dim() else tol)
+    assert cosine(g, want64) >= 0.99999, what
+
+
+# ------------------------------------------------------------------ int8: exact accumulators
+
+@pytest.mark.parametrize("mnk", [(256, 256, 128), (16, 8, 16), (1, 1, 32), (300, 200, 144), (257, 129, 2048), (513, 384, 400)])
+def test_int8_accumulators_bit_exact(dev, tile_cfg, mnk):
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + k)
+    a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+    got = _C().q8_mm_i32(a.to(dev), b.to(dev))
+    assert_bit_equal(got, O.ref_gemm_i32(a, b), "int32 acc %s" % (mnk,))
+
+
+def test_int8_config2_bit_exact_and_dequant(dev):
+    """A int8 [6144, 2048], B int8 [2048, 2048] from per-row absmax quantisation (round to nearest even) of
+    N(0,1) and N(0,0.02) bf16 tensors; int32 accumulators must match exactly, then dequantise with bias."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(6144, 2048, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2048, 2048, generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(2048, generator=g) * 0.02).to(torch.bfloat16).float()
+    a, sa = O.ref_quant(x, torch.int8, round_half_even=True)
+    b, sb = O.ref_quant(w, torch.int8, round_half_even=True)
+    # the quantizer kernel yields the same codes
+    ga, gsa = _C().tokenwise_quant(x.to(dev), torch.int8, round_half_even=True)
+    assert_bit_equal(ga, a, "config-2 A codes")
+    assert_bit_equal(gsa, sa, "config-2 A scales")
+    acc = _C().q8_mm_i32(a.to(dev), b.to(dev))
+    want_acc = O.ref_gemm_i32(a, b)
+    assert_bit_equal(acc, want_acc, "config-2 int32 accumulators")
+    out = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.to(dev), sb.to(dev), False, torch.bfloat16)
+    assert out.shape == (1, 6144, 2048) and out.dtype == torch.bfloat16
+    want = O.ref_epilogue(want_acc[None], sa[None], sb[None], bias, False, torch.bfloat16)
+    # same exact accumulators, one fma and one rounding: at most the last bf16 bit may differ
+    diff = (out.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    assert diff.max() <= 1 and (diff > 0).float().mean() < 1e-3
+    # and it approximates the bf16 linear it stands for
+    ref = x.double() @ w.double().T + bias.double()
+    assert cosine(out.cpu(), ref) > 0.999
+
+
+# ------------------------------------------------------------------ epilogue variants
+
+@pytest.mark.parametrize("in_dtype", ["i8", "fp8"])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_mm_epilogue_vs_oracle(dev, tile_cfg, in_dtype, fuse_gelu, with_bias):
+    g = torch.Generator().manual_seed(100 + fuse_gelu * 2 + with_bias)
+    m, n, k = 200, 264, 384
+    if in_dtype == "i8":
+        a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+        sa, sb = torch.rand(m, generator=g) * 2e-3 + 1e-4, torch.rand(n, generator=g) * 2e-2 + 1e-3
+        mm, mmb, ref = _C().q8_mm, _C().q8_mm_bias, O.ref_q8_mm
+    else:
+        a, b = O.e4m3_c10(torch.randn(m, k, generator=g) * 50), O.e4m3_c10(torch.randn(n, k, generator=g) * 50)
+        sa, sb = torch.rand(m, generator=g) * 1e-2 + 1e-4, torch.rand(n, generator=g) * 1e-2 + 1e-4
+        mm, mmb, ref = _C().fp8_mm, _C().fp8_mm_bias, O.ref_fp8_mm
+    bias = torch.randn(n, generator=g) if with_bias else None
+    args = (a.to(dev), b.to(dev)) + ((bias.to(dev),) if with_bias else ()) + (sa.to(dev), sb.to(dev), fuse_gelu)
+    fn = mmb if with_bias else mm
+    got = fn(*args, torch.bfloat16)
+    assert got.shape == (1, m, n)
+    acc = O.ref_gemm_i32(a, b).double() if in_dtype == "i8" else O.ref_gemm_fp8_acc(a, b)
+    v = acc * (sa[:, None] * sb[None, :]).double() + (bias.double() if with_bias else 0)
+    want64 = torch.nn.functional.gelu(v, approximate="tanh") if fuse_gelu else v
+    _check_float_out(got[0], want64, "%s gelu=%s bias=%s" % (in_dtype, fuse_gelu, with_bias))
+    # e4m3 output (the reference's default out_type): saturating cast of the same value
+    got8 = fn(*args, None)
+    assert got8.dtype == E4M3
+    want8 = ref(a, b, bias, sa, sb, fuse_gelu, None)[0]
+    g8, w8 = got8[0].cpu().float(), want8.float()
+    assert not torch.isnan(g8).any()
+    assert ((g8 - w8).abs() <= 0.126 * w8.abs() + 2 ** -9).all()
+    assert (got8[0].cpu().view(torch.uint8) != want8.view(torch.uint8)).float().mean() < 0.02
+
+
+def test_mm_e4m3_output_saturates(dev):
+    a = torch.full((16, 32), 127, dtype=torch.int8)
+    b = torch.full((16, 32), 127, dtype=torch.int8)
+    b[8:] = -127
+    ones = torch.ones(16)
+    out = _C().q8_mm(a.to(dev), b.to(dev), ones.to(dev), ones.to(dev), False, None)
+    codes = out.cpu().view(torch.uint8)[0]
+    assert (codes[:, :8] == 0x7E).all() and (codes[:, 8:] == 0xFE).all()
+
+
+def test_mm_batch_broadcast(dev, tile_cfg):
+    g = torch.Generator().manual_seed(7)
+    m, n, k = 70, 48, 64
+    a3, b3 = _rand_i8(g, 3, m, k), _rand_i8(g, 3, n, k)
+    sa3, sb3 = torch.rand(3, m, generator=g) * 1e-2, torch.rand(3, n, generator=g) * 1e-2
+    bias = torch.randn(n, generator=g)
+    cases = [(a3, b3[0], sa3, sb3[0]), (a3[0], b3, sa3[0], sb3), (a3, b3, sa3, sb3), (a3[1], b3[2], sa3[1], sb3[2])]
+    for a, b, sa, sb in cases:
+        got = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.contiguous().to(dev), sb.contiguous().to(dev), False, torch.bfloat16)
+        want = O.ref_q8_mm(a, b, bias, sa, sb, False, torch.bfloat16)
+        assert got.shape == want.shape
+        diff = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert diff.max() <= 1, "batch case a%s b%s" % (tuple(a.shape), tuple(b.shape))
+
+
+# ------------------------------------------------------------------ fp8 at the benchmark shapes
+
+@pytest.mark.parametrize("m", [2048, 6144])
+def test_fp8_linear_bias_gelu_config1(dev, m):
+    """X bf16 [m, 2048] ~ N(0,1); W bf16 [8192, 2048] ~ N(0,0.02); bias ~ N(0,0.02); per-row e4m3 quantisation;
+    out = GELU(acc * sx * sw + bias) in bf16. Tolerance: 2 bf16 ulp + 2^-9 mean|out| against float64, cosine
+    >= 0.99999; and cosine >= 0.999 against the unquantised bf16 linear."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, 2048, generator=g).to(torch.bfloat16)
+    w = (torch.randn(8192, 2048, generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(8192, generator=g) * 0.02).to(torch.bfloat16).float()
+    xq, sx = _C().tokenwise_quant(x.to(dev), E4M3)
+    wq, sw = _C().tokenwise_quant(w.to(dev), E4M3)
+    oxq, osx = O.ref_quant(x, E4M3)
+    owq, osw = O.ref_quant(w, E4M3)
+    assert_bit_equal(xq, oxq, "X codes")
+    assert_bit_equal(sx, osx, "X scales")
+    assert_bit_equal(wq, owq, "W codes")
+    assert_bit_equal(sw, osw, "W scales")
+    out = _C().fp8_mm_bias(xq, wq, bias.to(dev), sx, sw, True, torch.bfloat16)
+    assert out.shape == (1, m, 8192)
+    acc = O.ref_gemm_fp8_acc(oxq, owq)
+    v = acc * (osx[:, None] * osw[None, :]).double() + bias.double()
+    want64 = torch.nn.functional.gelu(v, approximate="tanh")
+    _check_float_out(out[0], want64, "config-1 m=%d" % m)
+    full = torch.nn.functional.gelu(x.double() @ w.double().T + bias.double(), approximate="tanh")
+    assert cosine(out[0].cpu(), full) > 0.999
+
+
+def test_mm_rejects_bad_arguments(dev):
+    from q8_kernels_amd import Q8Error
+    a = torch.zeros(16, 24, dtype=torch.int8, device=dev)
+    s = torch.ones(16, device=dev)
+    with pytest.raises(Q8Error):  # K % 16 != 0
+        _C().q8_mm(a, a, s, s, False, torch.bfloat16)
+    a = torch.zeros(16, 32, dtype=torch.int8, device=dev)
+    with pytest.raises(RuntimeError):  # fp16 output is not supported (the reference returns garbage)
+        _C().q8_mm(a, a, s, s, False, torch.float16)
+    with pytest.raises(RuntimeError):
+        _C().q8_mm(a, a.t(), s, s, False, torch.bfloat16)  # not contiguous
+    with pytest.raises(RuntimeError):
+        _C().fp8_mm(a, a, s, s, False, torch.bfloat16)  # wrong operand dtype
+    with pytest.raises(RuntimeError):
+        _C().q8_mm(torch.zeros(2, 16, 32, dtype=torch.int8, device=dev), torch.zeros(3, 16, 32, dtype=torch.int8, device=dev),
+                   torch.ones(32, device=dev), torch.ones(48, device=dev), False, torch.bfloat16)
