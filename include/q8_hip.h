@@ -61,8 +61,11 @@ enum {
     Q8_V_SD = 1  /* V given as [B,H,N,D]                                                                    */
 };
 enum {
-    Q8_ATTN_SUM_ROUNDED_P = 1 /* row sum accumulates the e4m3-rounded probabilities (what multiplies V)
-                                 instead of the unrounded fp32 ones                                        */
+    Q8_ATTN_SUM_ROUNDED_P = 1, /* row sum accumulates the e4m3-rounded probabilities (what multiplies V)
+                                  instead of the unrounded fp32 ones                                        */
+    Q8_ATTN_P_UNIT_RANGE = 2   /* form the probabilities as exp(s - max) <= 1 before their e4m3 cast, like the
+                                  reference; by default they are scaled by 2^8 (the factor cancels in o / l),
+                                  which keeps weights below 2^-10 of the maximum from being flushed to zero  */
 };
 
 const char* q8_strerror(int status);
@@ -155,7 +158,8 @@ int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int 
  * (csrc/flash_attention/flash_attention.cpp:18-48; kernels flash_attention_cuda.cu:254-534 and
  * flash_attention_cuda_mask.cu:254-535).
  *   s[i,j] = (q_i . k_j) * softmax_scale * (sq[i]*sk[j] if given);  keys j >= kv_len[b] (or >= N) masked
- *   p[i,j] = exp(s[i,j] - max_j s[i,j]);  l_i = sum_j p[i,j]  (fp32, unrounded unless SUM_ROUNDED_P)
+ *   p[i,j] = 2^8 exp(s[i,j] - max_j s[i,j])  (without the 2^8 under P_UNIT_RANGE);
+ *   l_i = sum_j p[i,j]  (fp32, unrounded unless SUM_ROUNDED_P)
  *   o_i = (sum_j e4m3_sat(p[i,j]) * v_j) / l_i;   rows with l_i == 0 or NaN divide by 1
  *   with sv: o_i = svmax * (sum_j e4m3_sat(p[i,j] * sv[j] / svmax) * v_j) / l_i,  svmax = max_{j valid} sv[j]
  *   O = bf16(o) or e4m3_sat(o)

@@ -226,7 +226,8 @@ def ref_fp8_linear(a, b, bias=None, scale_a=None, scale_b=None, use_hadamard=Fal
 
 def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                   kv_len: Optional[torch.Tensor] = None, sq=None, sk=None, sv=None,
-                  round_p: bool = True, out_dtype: Optional[torch.dtype] = None, return_weighted_abs: bool = False):
+                  round_p: bool = True, out_dtype: Optional[torch.dtype] = None, return_weighted_abs: bool = False,
+                  p_scale: float = 256.0):
     """Attention on e4m3 operands as the reference kernel defines it (csrc/flash_attention/
     flash_attention_cuda.cu:171-248,437,487-497; mask: flash_attention_cuda_mask.cu:244,319):
         s_ij = (q_i . k_j) * scale (* sq_i sk_j);  keys j >= kv_len[b] masked;
@@ -237,10 +238,13 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
     q [B,H,M,D], k, v [B,H,N,D] (v NOT transposed here). With round_p=False this is plain fp32-style
     softmax attention on the dequantised inputs (evaluated in float64), the accuracy target of the
     BASELINE configs. out_dtype None returns float64; bf16 -> RNE; e4m3 -> saturating cast.
+    p_scale: the probabilities are rounded as e4m3_sat(p_scale * p); the reference has p_scale = 1 (weights
+    below 2^-10 flush to zero), the HIP kernel defaults to 2^8, which cancels in o / l.
     The online kernel rounds p against the running maximum, so its P-hat differs from this one in the
     last e4m3 bit here and there: comparisons carry a tolerance. With return_weighted_abs the function also
-    returns sum_j p_ij |v_j| / l_i: any rounding of the weights by a relative eps moves o_i by at most eps
-    times that, which is the rigorous error bound the tests use (eps = 2^-4 for e4m3)."""
+    returns W = sum_j p_ij |v_j| / l_i and U = sum_j |v_j| / l_i: rounding every weight with relative error eps
+    (2^-4 for normal e4m3 values) or absolute error delta (2^-10 / p_scale in the subnormal range) moves o_i
+    by at most eps W + delta U, the rigorous bound the tests use."""
     qd, kd, vd = q.to(torch.float64), k.to(torch.float64), v.to(torch.float64)
     s = qd @ kd.transpose(-1, -2) * softmax_scale
     if sq is not None:
@@ -261,7 +265,7 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
         sv_ref = svd.amax(dim=-1, keepdim=True)
         pv = p * (svd / torch.where(sv_ref > 0, sv_ref, torch.ones_like(sv_ref))).unsqueeze(-2)
     if round_p:
-        pv = e4m3_sat(pv.to(torch.float32)).to(torch.float64)
+        pv = e4m3_sat((pv * p_scale).to(torch.float32)).to(torch.float64) / p_scale
     o = pv @ vd
     if sv_ref is not None:
         o = o * sv_ref.unsqueeze(-1)
@@ -269,7 +273,9 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
     o = o / lsafe
     if return_weighted_abs:
         vabs = vd.abs() if sv is None else vd.abs() * sv.to(torch.float64).unsqueeze(-1)
-        return o, (p @ vabs) / lsafe
+        if kv_len is not None:
+            vabs = torch.where(keep[:, None, :, None], vabs, torch.zeros_like(vabs))
+        return o, (p @ vabs) / lsafe, vabs.sum(dim=-2, keepdim=True) / lsafe
     if out_dtype is None:
         return o
     if out_dtype == E4M3:

@@ -238,13 +238,15 @@ def q8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                     batch_mask: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
                     q_scales: Optional[torch.Tensor] = None, k_scales: Optional[torch.Tensor] = None,
-                    v_scales: Optional[torch.Tensor] = None, sum_rounded_p: bool = False) -> torch.Tensor:
+                    v_scales: Optional[torch.Tensor] = None, sum_rounded_p: bool = False,
+                    p_unit_range: bool = False) -> torch.Tensor:
     """csrc/flash_attention/flash_attention.cpp:18-48.
 
     q [B,H,M,64], k [B,H,N,64], v [B,H,64,Nv] (pre-transposed, Nv >= N, Nv % 16 == 0), all e4m3 and contiguous;
     batch_mask int32 [B] of valid KV lengths. Returns [B,H,M,64] in out_dtype (None -> e4m3 like the reference).
-    The keyword arguments are extensions: bf16 output and per-token dequantisation scales
-    (q_scales [B,H,M], k_scales / v_scales [B,H,N], fp32).
+    The keyword arguments are extensions: bf16 output, per-token dequantisation scales
+    (q_scales [B,H,M], k_scales / v_scales [B,H,N], fp32), and p_unit_range=True to round the probabilities
+    on the reference's grid (p <= 1) instead of the default 2^8 p, which does not flush small weights.
     """
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
         _check_input(t, name)
@@ -279,5 +281,6 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
         _lib.check(_lib.lib().q8_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(batch_mask),
                                           _ptr(q_scales), _ptr(k_scales), _ptr(v_scales), bs, heads, m, n, d,
                                           _lib.Q8_V_DS, v.shape[3], float(softmax_scale), _DT[out_dtype],
-                                          _lib.Q8_ATTN_SUM_ROUNDED_P if sum_rounded_p else 0, _stream(q)))
+                                          (_lib.Q8_ATTN_SUM_ROUNDED_P if sum_rounded_p else 0) |
+                                          (_lib.Q8_ATTN_P_UNIT_RANGE if p_unit_range else 0), _stream(q)))
     return out

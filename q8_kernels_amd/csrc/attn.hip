@@ -11,9 +11,11 @@
 //                 cast to e4m3, ARE the 32-byte B operand of that lane. For this the K rows are
 //                 placed in LDS in the order in which the S^T accumulator rows come out, such that
 //                 lane half h owns keys 32h .. 32h+31 of the tile in operand byte order.
-// Softmax runs in the log2 domain in fp32: p = exp2(s * c - m), c = softmax_scale * log2(e); the row
+// Softmax runs in the log2 domain in fp32: p = exp2(s * c - m + 8), c = softmax_scale * log2(e); the row
 // sum accumulates the unrounded p while e4m3_sat(p) multiplies V (csrc/flash_attention/
-// flash_attention_cuda.cu:197-221,437). Tiles that lie entirely beyond the valid KV length are
+// flash_attention_cuda.cu:197-221,437). The factor 2^8 cancels in O / l; it places the row maximum at 256 so
+// that probabilities down to 2^-14 of the maximum stay in the normal range of e4m3 (with the reference's p <= 1
+// everything below 2^-10 is flushed to zero, which biases long, flat rows). Q8_ATTN_P_UNIT_RANGE restores p <= 1. Tiles that lie entirely beyond the valid KV length are
 // skipped, the partial tile is masked with -inf (the reference walks backwards and needs -1e6 instead,
 // flash_attention_cuda_mask.cu:244).
 #include "q8_common.h"
@@ -33,6 +35,7 @@ struct AttnParams {
     int B, H, M, N;
     int64_t v_row_stride;  // V^T row stride in bytes-elements (>= N, multiple of 16)
     float scale_log2;      // softmax_scale * log2(e)
+    float p_shift;         // probabilities are formed as 2^(x - max + p_shift)
     int flags;
 };
 
@@ -192,11 +195,12 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
             const float m_new = fmaxf(m_run[qt], mx);
             const float alpha = fast_exp2(m_run[qt] - m_new);
             m_run[qt] = m_new;
+            const float m_sub = m_new - p.p_shift;
             float psum = 0.f;
             float pr[32];
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                const float pe = fast_exp2(x[e] - m_new);
+                const float pe = fast_exp2(x[e] - m_sub);
                 psum += pe;
                 pr[e] = SCALED ? pe * svv[e] : pe;
             }
@@ -266,7 +270,7 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);
     if (out_dtype != Q8_BF16 && out_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_attn_fwd: output dtype %d", out_dtype);
-    if (flags & ~Q8_ATTN_SUM_ROUNDED_P) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
+    if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
     if (v_layout != Q8_V_DS) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V layout %d (only Q8_V_DS [B,H,64,Nv] is implemented)", v_layout);
     if (v_row_stride < N || v_row_stride % 16 != 0)
         return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V row stride %lld must be >= N and a multiple of 16", (long long)v_row_stride);
@@ -275,7 +279,8 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(o) % 8))
         return fail(Q8_ERR_ALIGN, "q8_attn_fwd: q, k, v must be 16-byte and o 8-byte aligned");
     AttnParams p{static_cast<const uint8_t*>(q), static_cast<const uint8_t*>(k), static_cast<const uint8_t*>(v), o, kv_len, sq, sk, sv,
-                 B, H, M, N, v_row_stride, softmax_scale * 1.44269504088896340736f, flags};
+                 B, H, M, N, v_row_stride, softmax_scale * 1.44269504088896340736f,
+                 (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
     const dim3 grid((unsigned)((M + kBlockQ - 1) / kBlockQ), (unsigned)(B * H));
     const dim3 block(kWaves * 64);
     if (out_dtype == Q8_BF16) {

@@ -5,8 +5,12 @@
 // Structure of one workgroup (WAVES_M x WAVES_N waves, one BM x BN tile of C):
 //   * K is walked in steps of 128 bytes. A step's A rows (BM x 128 B) and B rows (BN x 128 B) are
 //     copied HBM -> LDS by `global_load_lds_dwordx4` (no VGPR staging), two LDS stages.
-//   * LDS holds plain 128-byte rows whose 16-byte chunks are XOR-swizzled by ((row >> 1) & 7): the
-//     16 lanes that fetch the same chunk index of 16 consecutive rows hit 16 different bank groups.
+//   * LDS holds plain 128-byte rows whose 16-byte chunks are XOR-swizzled by lds_swizzle(row). A
+//     ds_read_b128 is served in four passes of 16 lanes, and the lanes of one pass are NOT consecutive:
+//     measured on gfx950 they are {0-3, 12-15, 20-23, 24-27}, {4-7, 8-11, 16-19, 28-31} and the same
+//     + 32. With operand lane = (row % 16, k-chunk pair lane / 16) a pass therefore touches all 16 rows,
+//     rows {0-3, 12-15} at one chunk pair and rows {4-11} at the neighbouring one; the swizzle makes
+//     those 16 accesses fall into the 16 different 16-byte bank groups (256 B/clk, no conflicts).
 //   * A wave owns TM x TN MFMA tiles of 16x16. fp8 uses v_mfma_f32_16x16x128_f8f6f4 (one per step),
 //     int8 uses two v_mfma_i32_16x16x64_i8. The B rows feed the MFMA "A" operand and the A rows the
 //     "B" operand, so an accumulator lane holds four consecutive n of one m.
@@ -17,64 +21,10 @@
 //     K are sourced from a 16-byte block of zeros.
 //   * Workgroup ids are re-mapped so that each XCD (ids congruent mod 8 share an L2) owns a
 //     contiguous range of tiles, walked in groups of GROUP_M tile rows for L2 reuse of A and B.
-#include "q8_common.h"
-#include "q8_host.h"
+#include "gemm_common.h"
+#include "gemm_pipe.h"
 
 namespace q8 {
-
-struct GemmParams {
-    const uint8_t* A;
-    const uint8_t* B;
-    const float* bias;
-    const float* sa;
-    const float* sb;
-    void* C;
-    int batch_a, batch_b;
-    int M, N, K;
-};
-
-__device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0};
-
-constexpr int Q8_OUT_I32 = 100;  // raw accumulators (int8 only)
-constexpr int kGroupM = 4;
-
-template <int IN_, int WAVES_M_, int WAVES_N_, int TM_, int TN_>
-struct GemmCfg {
-    static constexpr int IN = IN_;
-    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, TM = TM_, TN = TN_;
-    static constexpr int NW = WAVES_M * WAVES_N;
-    static constexpr int NT = NW * 64;
-    static constexpr int BM = WAVES_M * TM * 16;
-    static constexpr int BN = WAVES_N * TN * 16;
-    static constexpr int BK = 128;
-    static constexpr int STAGE_BYTES = (BM + BN) * BK;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-    static constexpr int RG_A = BM / 8, RG_B = BN / 8;  // 1 KiB row groups per stage
-    static constexpr int PER_A = RG_A / NW, PER_B = RG_B / NW;
-    static_assert(RG_A % NW == 0 && RG_B % NW == 0, "row groups must divide over the waves");
-    static_assert(TN % 2 == 0, "TN must be even (pairs of n tiles form one 16-byte store)");
-};
-
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
-__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70 | 0); }
-
-// column permutation inside a wave's TN*16 columns: LDS row (16 j + s) of the wave's B slab holds
-// local column 32 (j/2) + 8 (s/4) + 4 (j%2) + (s%4).
-__device__ __forceinline__ int bcol_of_slot(int rho) {
-    const int j = rho >> 4, s = rho & 15;
-    return 32 * (j >> 1) + 8 * (s >> 2) + 4 * (j & 1) + (s & 3);
-}
-
-__device__ __forceinline__ float gelu_tanh_fast(float v) {
-    // 0.5 v (1 + tanh(u)) = v / (1 + exp(-2u)),  u = 0.7978845608 (v + 0.044715 v^3)
-    // (csrc/gemm/fp8_matmul_bias.cu:31-35); exp2 and reciprocal on the transcendental unit.
-    const float k1 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
-    const float k3 = k1 * 0.044715f;
-    const float v2 = v * v;
-    const float arg = v * fmaf(v2, k3, k1);
-    const float e = __builtin_amdgcn_exp2f(arg);
-    return v * __builtin_amdgcn_rcpf(1.0f + e);
-}
 
 template <class C, int OUT, bool GELU>
 __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
@@ -84,19 +34,10 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
     const int wave_m = wave / C::WAVES_N, wave_n = wave % C::WAVES_N;
     const int M = p.M, N = p.N, K = p.K;
 
-    // ---- tile of this workgroup (XCD-contiguous, grouped walk)
+    // ---- tile of this workgroup
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    int pid;
-    {
-        const int nb = gridDim.x, bid = blockIdx.x;
-        const int xcd = bid & 7, loc = bid >> 3, per = nb >> 3, rem = nb & 7;
-        pid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-    }
-    const int group_size = kGroupM * tiles_n;
-    const int gid = pid / group_size, first_m = gid * kGroupM;
-    const int gsz = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
-    const int tile_m = first_m + (pid % group_size) % gsz;
-    const int tile_n = (pid % group_size) / gsz;
+    int tile_m, tile_n;
+    tile_of_block(tiles_m, tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int z = blockIdx.y;
@@ -105,7 +46,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
     const uint8_t* Bg = p.B + (size_t)zb * N * K;
 
     // ---- HBM -> LDS copy plan: lane (lane/8, lane%8) of row group q fills LDS row 8q + lane/8,
-    //      physical chunk lane%8, from logical chunk (lane%8) ^ ((row >> 1) & 7)
+    //      physical chunk lane%8, from logical chunk (lane%8) ^ lds_swizzle(row)
     const uint8_t* src[C::PER_A + C::PER_B];
     int kchunk[C::PER_A + C::PER_B];
 #pragma unroll
@@ -113,7 +54,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
         const bool isA = i < C::PER_A;
         const int q = isA ? (wave + i * NW) : (wave + (i - C::PER_A) * NW);
         const int rho = 8 * q + (lane >> 3);
-        const int c = (lane & 7) ^ ((rho >> 1) & 7);
+        const int c = (lane & 7) ^ lds_swizzle(rho);
         kchunk[i] = c * 16;
         if (isA) {
             int m = m0 + rho;
@@ -140,7 +81,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
 
     // ---- operand fetch addresses: lane (s = lane%16, gk = lane/16) reads chunks 2gk, 2gk+1 of row s
     const int s16 = lane & 15, gk = lane >> 4;
-    const int pc0 = ((2 * gk) ^ ((s16 >> 1) & 7)) * 16, pc1 = pc0 ^ 16;
+    const int pc0 = ((2 * gk) ^ lds_swizzle(s16)) * 16, pc1 = pc0 ^ 16;
     const int a_row0 = wave_m * TM * 16 + s16;
     const int b_row0 = BM + wave_n * TN * 16 + s16;
 
@@ -197,64 +138,16 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
         const int n = nw0 + 32 * jj + 8 * g;
         if (n >= N) continue;
         float sbv[8], bv[8];
-        if constexpr (OUT != Q8_OUT_I32) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int nn = (n + e < N) ? n + e : N - 1;
-                sbv[e] = p.sb[(size_t)zb * N + nn];
-                bv[e] = p.bias ? p.bias[nn] : 0.f;
-            }
-        }
+        load_col_params<OUT>(p, zb, n, sbv, bv);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int m = m0 + wave_m * TM * 16 + 16 * i + s16;
             if (m >= M) continue;
-            if constexpr (OUT == Q8_OUT_I32) {
-                int32_t* crow = reinterpret_cast<int32_t*>(p.C) + zc + (size_t)m * N + n;
-                if (n + 8 <= N && ((N & 7) == 0)) {
-                    *reinterpret_cast<v4i*>(crow) = acc[i][2 * jj];
-                    *reinterpret_cast<v4i*>(crow + 4) = acc[i][2 * jj + 1];
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (n + e < N) crow[e] = (e < 4) ? acc[i][2 * jj][e] : acc[i][2 * jj + 1][e - 4];
-                }
-            } else {
-                const float sam = p.sa[(size_t)za * M + m];
-                float v[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float a = (float)((e < 4) ? acc[i][2 * jj][e] : acc[i][2 * jj + 1][e - 4]);
-                    // dequantise as acc * (sa * sb) + bias (csrc/gemm/fp8_matmul_bias.cu:356-365)
-                    float t = fmaf(a, sam * sbv[e], bv[e]);
-                    if constexpr (GELU) t = gelu_tanh_fast(t);
-                    v[e] = t;
-                }
-                if constexpr (OUT == Q8_BF16) {
-                    uint16_t* crow = reinterpret_cast<uint16_t*>(p.C) + zc + (size_t)m * N + n;
-                    if (n + 8 <= N && ((N & 7) == 0)) {
-                        v4u w;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) w[e] = f32_to_bf16_bits(v[2 * e]) | (f32_to_bf16_bits(v[2 * e + 1]) << 16);
-                        *reinterpret_cast<v4u*>(crow) = w;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (n + e < N) crow[e] = (uint16_t)f32_to_bf16_bits(v[e]);
-                    }
-                } else {
-                    uint8_t* crow = reinterpret_cast<uint8_t*>(p.C) + zc + (size_t)m * N + n;
-                    const uint32_t w0 = pack4_e4m3_sat(v[0], v[1], v[2], v[3]);
-                    const uint32_t w1 = pack4_e4m3_sat(v[4], v[5], v[6], v[7]);
-                    if (n + 8 <= N && ((N & 7) == 0)) {
-                        *reinterpret_cast<v2i*>(crow) = v2i{(int)w0, (int)w1};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (n + e < N) crow[e] = (uint8_t)(((e < 4) ? w0 : w1) >> (8 * (e & 3)));
-                    }
-                }
-            }
+            const float sam = (OUT == Q8_OUT_I32) ? 0.f : p.sa[(size_t)za * M + m];
+            using elem_t = typename std::conditional<C::IN == Q8_I8, int, float>::type;
+            const elem_t a8[8] = {acc[i][2 * jj][0], acc[i][2 * jj][1], acc[i][2 * jj][2], acc[i][2 * jj][3],
+                                  acc[i][2 * jj + 1][0], acc[i][2 * jj + 1][1], acc[i][2 * jj + 1][2], acc[i][2 * jj + 1][3]};
+            finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv);
         }
     }
 }
@@ -284,13 +177,32 @@ using CfgBig = GemmCfg<IN, 2, 4, 8, 4>;
 template <int IN>
 using CfgSmall = GemmCfg<IN, 2, 2, 4, 4>;
 
-static int g_force_cfg = 0;  // 0 = auto, 1 = big, 2 = small (test hook, see q8_gemm_set_config)
+static int g_force_cfg = 0;  // 0 = auto, 1 = pipelined 256x256, 2 = 128x128, 3 = plain 256x256 (see q8_gemm_set_config)
+
+template <int IN, int OUT, bool GELU>
+static int launch_pipe(const GemmParams& p, hipStream_t stream) {
+    const int tiles_m = (p.M + kPipeBM - 1) / kPipeBM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
+    const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
+    auto kern = gemm_pipe_kernel<IN, OUT, GELU>;
+    static thread_local bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPipeLds) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", kPipeLds);
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(512), kPipeLds, stream, p);
+    return launch_status("q8_gemm");
+}
 
 template <int IN, int OUT, bool GELU>
 static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
     const long big_tiles = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.batch_a > p.batch_b ? p.batch_a : p.batch_b);
     const bool big = g_force_cfg == 1 || (g_force_cfg == 0 && big_tiles >= 192);
-    if (big) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);
+    if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
+    if (g_force_cfg == 3) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);
     return launch_gemm<CfgSmall<IN>, OUT, GELU>(p, stream);
 }
 
@@ -313,7 +225,7 @@ static int check_gemm(const char* who, const void* A, const void* B, const void*
 using namespace q8;
 
 extern "C" int q8_gemm_set_config(int cfg) {
-    if (cfg < 0 || cfg > 2) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 3) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
     g_force_cfg = cfg;
     return Q8_OK;
 }

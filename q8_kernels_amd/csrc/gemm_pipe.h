@@ -1,0 +1,274 @@
+// Software-pipelined 256x256 GEMM tile for gfx950 (the large-problem path of q8_gemm).
+//
+//   * 8 waves (2 along M x 4 along N), each owning 128 x 64 of the tile as 4 x 2 MFMA tiles of 32x32:
+//     fp8 uses v_mfma_f32_32x32x64_f8f6f4, int8 two v_mfma_i32_32x32x32_i8 per 64-byte K half.
+//   * K advances 128 bytes per stage. A stage is A 256 rows x 128 B + B 256 rows x 128 B = 64 KiB, two stages
+//     in LDS, filled by global_load_lds_dwordx4 with 8 lanes per row: every request to L2 is a full 128-byte
+//     line (measured 61 B/clk/CU against 28 B/clk/CU for 64-byte rows and 40 B/clk/CU through VGPRs).
+//   * One s_barrier per stage. The loads of stage k+1 are issued right after the barrier of stage k, into
+//     the buffer whose reads all waves have completed, and have a whole stage of MFMA time to land.
+//   * Operand fragments are double-buffered in registers over the two 64-byte K halves of a stage: the
+//     ds_read_b128 of the next half are always issued before the MFMAs of the current half. LDS reads and
+//     the counters are inline assembly so that exactly the waits written below are executed.
+//   * LDS rows are 128 bytes = 8 chunks of 16, physical chunk = logical chunk ^ ((row >> 1) & 7); lane
+//     (row % 32, half) reads chunks 4 s + 2 half and 4 s + 2 half + 1 for K half s. A ds_read_b128 is served
+//     in four passes of 16 lanes, {0-3, 12-15, 20-23, 24-27}, {4-11, 16-19, 28-31} and the same + 32
+//     (measured); with this swizzle each pass hits 16 different 16-byte bank groups.
+//   * B rows feed the MFMA A operand, so an accumulator lane (m = lane % 32, h = lane / 32) holds 4 consecutive
+//     n per register quad; LDS row (32 t + 8 w + 4 h + r) of a wave's B slab is loaded with column
+//     32 t + 16 (w / 2) + 8 h + 4 (w % 2) + r so that two quads form 8 consecutive columns (one 16-byte store)
+//     and the two lane halves 32 contiguous bytes.
+#pragma once
+#include "gemm_common.h"
+
+namespace q8 {
+
+constexpr int kPipeBM = 256, kPipeBN = 256, kPipeStages = 2, kPipeStageBytes = 65536;
+constexpr int kPipeLds = kPipeStages * kPipeStageBytes;
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int OFFSET>
+__device__ __forceinline__ v4i lds_read_b128(unsigned addr) {
+    v4i r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET) : "memory");
+    return r;
+}
+
+struct PipeFrags {
+    v4i a[4][2];  // 4 m-tiles x (low, high) 16-byte halves of the lane's 32 K bytes
+    v4i b[2][2];  // 2 n-tiles
+};
+
+// a0/a1 (b0/b1): byte address of the lane's low/high 16-byte chunk in row (lane % 32) of the wave's first A (B)
+// tile; the following 32-row tiles are 4096 bytes apart.
+__device__ __forceinline__ void pipe_read_frags(PipeFrags& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
+    f.b[0][0] = lds_read_b128<0>(b0);
+    f.b[0][1] = lds_read_b128<0>(b1);
+    f.a[0][0] = lds_read_b128<0>(a0);
+    f.a[0][1] = lds_read_b128<0>(a1);
+    f.b[1][0] = lds_read_b128<4096>(b0);
+    f.b[1][1] = lds_read_b128<4096>(b1);
+    f.a[1][0] = lds_read_b128<4096>(a0);
+    f.a[1][1] = lds_read_b128<4096>(a1);
+    f.a[2][0] = lds_read_b128<8192>(a0);
+    f.a[2][1] = lds_read_b128<8192>(a1);
+    f.a[3][0] = lds_read_b128<12288>(a0);
+    f.a[3][1] = lds_read_b128<12288>(a1);
+}
+
+// Wait until every LDS read issued so far has landed; the fragments pass through the statement so that no
+// MFMA consuming them can be scheduled above it.
+__device__ __forceinline__ void pipe_wait_frags(PipeFrags& f) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                   "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1])
+                 :
+                 : "memory");
+}
+
+// Compiler-level fence for the fragments: statements that consume them stay below this point, i.e. below the
+// LDS reads issued before it.
+__device__ __forceinline__ void pipe_pin(PipeFrags& f) {
+    asm volatile(""
+                 : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                   "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1]));
+}
+
+// The 8 (fp8) / 16 (int8) MFMAs of one K half. `between(j)` runs after the j-th of the 8 tiles with scheduling
+// fences around it, so that whatever it issues (one HBM->LDS copy) stays between two MFMAs: a wave that issued
+// all copies of a stage back to back would sit in the full vector-memory queue instead of feeding the matrix pipe.
+template <int IN, typename ACC, typename F>
+__device__ __forceinline__ void pipe_mfma(const PipeFrags& f, ACC (&acc)[4][2], F between) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if constexpr (IN == Q8_I8) {
+                acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[t][0], f.a[i][0], acc[i][t], 0, 0, 0);
+                acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[t][1], f.a[i][1], acc[i][t], 0, 0, 0);
+            } else {
+                const v8i bf = {f.b[t][0][0], f.b[t][0][1], f.b[t][0][2], f.b[t][0][3], f.b[t][1][0], f.b[t][1][1], f.b[t][1][2], f.b[t][1][3]};
+                const v8i af = {f.a[i][0][0], f.a[i][0][1], f.a[i][0][2], f.a[i][0][3], f.a[i][1][0], f.a[i][1][1], f.a[i][1][2], f.a[i][1][3]};
+                acc[i][t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf, af, acc[i][t], 0, 0, 0, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            between(2 * i + t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+// DBG (tuning builds only): bit 0 = no HBM->LDS loads, 1 = no LDS reads, 2 = no MFMA, 3 = no stores, 4 = no barrier
+template <int IN, int OUT, bool GELU, int DBG = 0>
+__global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    constexpr int BM = kPipeBM, BN = kPipeBN;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int wave_m = wave >> 2, wave_n = wave & 3;
+    const int M = p.M, N = p.N, K = p.K;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int tile_m, tile_n;
+    tile_of_block(tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int z = blockIdx.y;
+    const int za = (p.batch_a == 1) ? 0 : z, zb = (p.batch_b == 1) ? 0 : z;
+    const uint8_t* Ag = p.A + (size_t)za * M * K;
+    const uint8_t* Bg = p.B + (size_t)zb * N * K;
+
+    // ---- HBM -> LDS copy plan. A stage is 64 row groups of 1 KiB (8 rows x 128 B): groups 0..31 hold A, 32..63 B.
+    //      Wave w copies groups w, w+8, w+16, w+24 of each; lane (lane/8, lane%8) fills row 8 q + lane/8,
+    //      physical chunk lane%8, from logical chunk (lane%8) ^ ((row >> 1) & 7).
+    const uint8_t* src[8];
+    int kchunk[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int q = wave + 8 * (i & 3);
+        const int rho = 8 * q + (lane >> 3);
+        const int c = (lane & 7) ^ ((rho >> 1) & 7);
+        kchunk[i] = 16 * c;
+        if (i < 4) {
+            int m = m0 + rho;
+            m = m < M ? m : M - 1;
+            src[i] = Ag + (size_t)m * K + 16 * c;
+        } else {
+            const int slab = rho >> 6, t = (rho >> 5) & 1, w = (rho >> 3) & 3, hh = (rho >> 2) & 1, r = rho & 3;
+            int n = n0 + 64 * slab + 32 * t + 16 * (w >> 1) + 8 * hh + 4 * (w & 1) + r;
+            n = n < N ? n : N - 1;
+            src[i] = Bg + (size_t)n * K + 16 * c;
+        }
+    }
+    const int KT = (K + 127) >> 7;
+    auto issue_load = [&](int stage, int i) {  // copy instruction i (0..7) of this wave for `stage`
+        if constexpr (DBG & 1) return;
+        uint8_t* base = lds + (stage & 1) * kPipeStageBytes;
+        const int k0 = stage << 7;
+        const int q = (i < 4 ? 0 : 32) + wave + 8 * (i & 3);
+        // stages past the end of K (and chunks past K in the last stage) read a block of zeros instead
+        const uint8_t* g = (k0 + kchunk[i] < K) ? (src[i] + k0) : reinterpret_cast<const uint8_t*>(g_zero16);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                         (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
+    };
+    auto issue_loads = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) issue_load(stage, i);
+    };
+
+    // ---- operand fetch addresses: [K half s][low / high chunk], byte offsets inside a stage
+    const int r32 = lane & 31, h = lane >> 5;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const unsigned a_row = lds0 + wave_m * 16384 + r32 * 128;
+    const unsigned b_row = lds0 + 32768 + wave_n * 8192 + r32 * 128;
+    unsigned pc[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        pc[s][0] = ((4 * s + 2 * h) ^ ((r32 >> 1) & 7)) * 16;
+        pc[s][1] = pc[s][0] ^ 16;
+    }
+    auto read_half = [&](PipeFrags& f, int stage, int s) {
+        if constexpr (DBG & 2) return;
+        const unsigned so = (stage & 1) * kPipeStageBytes;
+        pipe_read_frags(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+    };
+
+    using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
+    acc_t acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][t][e] = 0;
+
+    // ---- prologue: stage 0 landed, stage 1 in flight, fragments of the first K half on their way
+    PipeFrags f0, f1;
+    issue_loads(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+    issue_loads(1);
+    if constexpr (DBG & 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { f0.a[i][0] = f0.a[i][1] = f1.a[i][0] = f1.a[i][1] = v4i{0x38383838, 0x38383838, 0x38383838, 0x38383838}; }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { f0.b[t][0] = f0.b[t][1] = f1.b[t][0] = f1.b[t][1] = v4i{0x38383838, 0x38383838, 0x38383838, 0x38383838}; }
+    }
+    read_half(f0, 0, 0);
+
+    for (int k = 0; k < KT; ++k) {
+        // f0: first K half of stage k (reads in flight); loads of stage k+1 in flight
+        pipe_wait_frags(f0);
+        read_half(f1, k, 1);
+        pipe_pin(f0);
+        if constexpr (!(DBG & 4)) pipe_mfma<IN>(f0, acc, [](int) {});
+        __builtin_amdgcn_sched_barrier(0);  // all MFMAs of the first half are issued before the wave waits and syncs
+        // the second half of stage k is in registers and stage k+1 has landed: nobody reads buffer k & 1 any more
+        if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        pipe_wait_frags(f1);
+        if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+        read_half(f0, k + 1, 0);
+        pipe_pin(f1);
+        // the copies of stage k+2 (into the buffer just released) trickle out between the MFMAs of the second half
+        if constexpr (DBG & 4) issue_loads(k + 2);
+        else pipe_mfma<IN>(f1, acc, [&](int j) { issue_load(k + 2, j); });
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // drain: the look-ahead loads and fragment reads past the last stage target LDS / registers that nobody uses
+    // (f0 is an operand of a wait so that its registers stay reserved until the last reads have landed)
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    pipe_wait_frags(f0);
+
+    // ---- epilogue: lane (mcol = lane % 32, h) holds for tile (i, t) and register quad w the 4 columns
+    //      32 t + 16 (w / 2) + 8 h + 4 (w % 2) + 0..3 of the wave's 64-column slab, row 32 i + mcol.
+    const size_t zc = (size_t)z * M * N;
+    const int nw0 = n0 + wave_n * 64;
+    // Interior tiles with bf16 output go through LDS: every wave lays its 128 x 64 results out as 128 rows of 128
+    // bytes (16-byte chunks swizzled by (row >> 1) & 7, conflict-free both ways) and then writes 8 full rows of 128
+    // contiguous bytes per instruction, i.e. whole cache lines instead of 32-byte pieces.
+    const bool staged = (OUT == Q8_BF16) && !(DBG & 8) && (m0 + BM <= M) && (n0 + BN <= N) && ((N & 7) == 0);
+    uint8_t* stage_out = lds + wave * 16384;
+    if (staged) __builtin_amdgcn_s_barrier();  // every wave has finished reading the operand stages
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int wp = 0; wp < 2; ++wp) {
+            const int n = nw0 + 32 * t + 16 * wp + 8 * h;
+            if (n >= N) continue;
+            float sbv[8], bv[8];
+            load_col_params<OUT>(p, zb, n, sbv, bv);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + wave_m * 128 + 32 * i + r32;
+                if (m >= M) continue;
+                const float sam = (OUT == Q8_OUT_I32) ? 0.f : p.sa[(size_t)za * M + m];
+                using elem_t = typename std::conditional<IN == Q8_I8, int, float>::type;
+                elem_t a8[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a8[e] = acc[i][t][8 * wp + e];
+                if constexpr (OUT == Q8_BF16) {
+                    if (staged) {
+                        float v[8];
+                        dequant8<GELU>(a8, sam, sbv, bv, v);
+                        const int row = 32 * i + r32, chunk = (4 * t + 2 * wp + h) ^ ((row >> 1) & 7);
+                        *reinterpret_cast<v4u*>(stage_out + row * 128 + chunk * 16) =
+                            v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
+                        continue;
+                    }
+                }
+                if constexpr (DBG & 8) { if (a8[0] == (elem_t)12345.678f) finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv); }
+                else finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv);
+            }
+        }
+    }
+    if constexpr (OUT == Q8_BF16) {
+        if (staged) {
+            uint16_t* cbase = reinterpret_cast<uint16_t*>(p.C) + zc + (size_t)(m0 + wave_m * 128) * N + nw0;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int row = 8 * j + (lane >> 3), chunk = (lane & 7) ^ ((row >> 1) & 7);
+                const v4u w = *reinterpret_cast<const v4u*>(stage_out + row * 128 + chunk * 16);
+                *reinterpret_cast<v4u*>(cbase + (size_t)row * N + (lane & 7) * 8) = w;
+            }
+        }
+    }
+}
+
+}  // namespace q8

@@ -266,9 +266,11 @@ def test_attention_rounded_p_invariants():
     v = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
     lens = torch.tensor([41], dtype=torch.int32)
     o = O.ref_attention(q, k, v, 0.125, lens)
-    exact = O.ref_attention(q, k, v, 0.125, lens, round_p=False)
-    # e4m3 rounding of p is a <= 2^-4 relative perturbation of each weight
-    assert (o - exact).abs().max() < 0.07
+    exact, wabs, uabs = O.ref_attention(q, k, v, 0.125, lens, round_p=False, return_weighted_abs=True)
+    # e4m3 rounding of p is a <= 2^-4 relative (normal range) / 2^-18 absolute (below it) perturbation of each weight
+    assert ((o - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -18 * uabs + 1e-12).all()
+    o1 = O.ref_attention(q, k, v, 0.125, lens, p_scale=1.0)
+    assert ((o1 - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -10 * uabs + 1e-12).all()
     # masked keys carry no weight: changing them changes nothing
     v2 = v.clone().view(torch.uint8)
     v2[:, :, 41:, :] = 0x7E
