@@ -151,6 +151,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain device copy of 512 MiB (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing on this path communicates "
@@ -166,6 +168,12 @@ def main():
     x, w, bias, xq, sx, wq, sw = _gemm_inputs(dev, M, N, K)
     bias_d = bias.to(dev)
     step = lambda: _C.fp8_mm_bias(xq, wq, bias_d, sx, sw, True, torch.bfloat16)  # noqa: E731
+    if args.copy_calibration:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 512 MiB, writes 512 MiB
+        torch.cuda.synchronize()
+        del src, dst
     sec, wall = _time(step, args.steps, args.warmup)
     flop = 2.0 * M * N * K
     tflops = flop / sec / 1e12
@@ -185,7 +193,7 @@ def main():
         "config": {"workload": "fp8 e4m3 GEMM + per-token/per-channel dequant + bias + tanh-GELU -> bf16, M=6144 N=8192 K=2048",
                    "inputs": "X~N(0,1), W~N(0,0.02), bias~N(0,0.02), per-row absmax e4m3 quantisation, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / FP8_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "gemm_kernel<e4m3, bf16, gelu>", "flop_per_launch": flop,
+                     "traffic": None, "kernel": "gemm_pipe_kernel<e4m3, bf16, gelu>", "flop_per_launch": flop,
                      "avg_launch_us": sec * 1e6, "host_wall_us_per_step": wall * 1e6},
     }
     traffic_file = os.path.join(ROOT, "profiles", "gemm_fp8_traffic.json")

@@ -172,6 +172,13 @@ int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int3
                 int B, int H, int M, int N, int D, int v_layout, int64_t v_row_stride,
                 float softmax_scale, int out_dtype, int flags, q8_stream_t stream);
 
+/*
+ * Workgroup-shape override for q8_attn_fwd: 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries,
+ * 2 = 4 waves x 32 queries. Process-wide; meant for tests and tuning, no counterpart in the reference (whose
+ * workgroup is fixed at 4 warps x 16 queries, csrc/flash_attention/flash_attention_cuda.cu:279-287).
+ */
+int q8_attn_set_config(int cfg);
+
 #ifdef __cplusplus
 }
 #endif

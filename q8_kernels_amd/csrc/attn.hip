@@ -41,17 +41,17 @@ struct AttnParams {
 
 __device__ __attribute__((aligned(16))) const uint32_t g_attn_zero16[4] = {0, 0, 0, 0};
 
-constexpr int kQT = 2;          // 32-query tiles per wave
-constexpr int kWaves = 4;
-constexpr int kBlockQ = kWaves * kQT * 32;  // 256 queries per workgroup
 constexpr int kKV = 64;         // keys per tile
 constexpr int kStage = 8192;    // K tile 4 KiB + V^T tile 4 KiB
+constexpr int kStages = 4;      // LDS ring: one tile being read, up to three in flight
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int OUT, bool SCALED>
+// kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
+template <int OUT, bool SCALED, int kQT, int kWaves>
 __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams p) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStage];
+    constexpr int kBlockQ = kWaves * kQT * 32;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int ql = lane & 31, h = lane >> 5;
     const int bh = blockIdx.y, b = bh / p.H;
@@ -81,30 +81,38 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
 
     // copy plan: wave w fills LDS rows 16w .. 16w+15 of both tiles (64-byte rows, 4 chunks of 16 bytes,
     // physical chunk = logical chunk ^ ((row >> 2) & 3)).
-    const int crow = 16 * wave + (lane >> 2);
+    // (with 8 waves, waves 0..3 copy the K tile and waves 4..7 the V^T tile; with 4 waves every wave copies both)
+    const int cw = wave & 3;
+    const bool copy_k = (kWaves == 4) || wave < 4, copy_v = (kWaves == 4) || wave >= 4;
+    const int crow = 16 * cw + (lane >> 2);
     const int cchunk = (lane & 3) ^ ((crow >> 2) & 3);
     int k_src_row;  // key index inside the tile held by LDS row `crow`
     {
         const int t = crow >> 5, i = crow & 31;
         k_src_row = 32 * ((i >> 2) & 1) + 16 * t + 4 * (i >> 3) + (i & 3);
     }
-    auto issue_loads = [&](int stage, int kv0) {
-        uint8_t* base = lds + stage * kStage;
+    // Every wave issues exactly one (4 waves: two) copy per tile, also for tiles past the end (from a block of
+    // zeros into a free stage), so that "s_waitcnt vmcnt(n)" always means "all but the n youngest tiles".
+    auto issue_loads = [&](int tile, bool real) {
+        uint8_t* base = lds + (tile & (kStages - 1)) * kStage;
+        const int kv0 = tile * kKV;
         int kr = kv0 + k_src_row;
         kr = kr < N ? kr : N - 1;
-        const uint8_t* ks = Kg + (size_t)kr * 64 + cchunk * 16;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
-                                         (__attribute__((address_space(3))) void*)(base + wave * 1024), 16, 0, 0);
+        const uint8_t* zero = reinterpret_cast<const uint8_t*>(g_attn_zero16);
+        const uint8_t* ks = real ? Kg + (size_t)kr * 64 + cchunk * 16 : zero;
+        if (copy_k)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
+                                             (__attribute__((address_space(3))) void*)(base + cw * 1024), 16, 0, 0);
         const int col = kv0 + cchunk * 16;
-        const uint8_t* vs = (col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col)
-                                                   : reinterpret_cast<const uint8_t*>(g_attn_zero16);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
-                                         (__attribute__((address_space(3))) void*)(base + 4096 + wave * 1024), 16, 0, 0);
+        const uint8_t* vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
+        if (copy_v)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
+                                             (__attribute__((address_space(3))) void*)(base + 4096 + cw * 1024), 16, 0, 0);
     };
 
     // operand fetch: lane (i = lane%32, h) reads chunks 2h, 2h+1 of row (32 t + i)
-    const int frow = ql * 64;
-    const int fpc0 = ((2 * h) ^ ((ql >> 2) & 3)) * 16, fpc1 = fpc0 ^ 16;
+    const unsigned fbase = lds_addr(lds) + ql * 64;
+    const unsigned fpc0 = ((2 * h) ^ ((ql >> 2) & 3)) * 16, fpc1 = fpc0 ^ 16;
 
     v16f o_acc[kQT][2];
 #pragma unroll
@@ -129,27 +137,47 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         mx = group_max<64>(mx);
         if (lane == 0) red[wave] = mx;
         __syncthreads();
-        sv_ref = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        sv_ref = red[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) sv_ref = fmaxf(sv_ref, red[w]);
         sv_inv = sv_ref > 0.f ? 1.0f / sv_ref : 0.f;
     }
 
-    if (n_tiles > 0) issue_loads(0, 0);
+    if (n_tiles > 0) {
+        issue_loads(0, true);
+        issue_loads(1, 1 < n_tiles);
+        issue_loads(2, 2 < n_tiles);
+    }
     for (int it = 0; it < n_tiles; ++it) {
         const int kv0 = it * kKV;
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        const uint8_t* st = lds + (it & 1) * kStage;
+        // tile `it` has landed (the two younger tiles may still be in flight) - for every wave after the barrier,
+        // which also says that all waves are done reading tile it-1, whose stage the next copy overwrites
+        if constexpr (kWaves == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        issue_loads(it + 3, it + 3 < n_tiles);
+        const unsigned st = fbase + (it & (kStages - 1)) * kStage;
+        v4i kl[2], kh[2], vl[2], vh[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            kl[t] = t ? lds_read_b128<2048>(st + fpc0) : lds_read_b128<0>(st + fpc0);
+            kh[t] = t ? lds_read_b128<2048>(st + fpc1) : lds_read_b128<0>(st + fpc1);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            vl[t] = t ? lds_read_b128<4096 + 2048>(st + fpc0) : lds_read_b128<4096>(st + fpc0);
+            vh[t] = t ? lds_read_b128<4096 + 2048>(st + fpc1) : lds_read_b128<4096>(st + fpc1);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1])
+                     :
+                     : "memory");
         v8i kf[2], vf[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const uint8_t* r = st + t * 2048 + frow;
-            const v4i a = *reinterpret_cast<const v4i*>(r + fpc0), c = *reinterpret_cast<const v4i*>(r + fpc1);
-            kf[t] = v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
-            const uint8_t* rv = st + 4096 + t * 2048 + frow;
-            const v4i av = *reinterpret_cast<const v4i*>(rv + fpc0), cv = *reinterpret_cast<const v4i*>(rv + fpc1);
-            vf[t] = v8i{av[0], av[1], av[2], av[3], cv[0], cv[1], cv[2], cv[3]};
+            kf[t] = v8i{kl[t][0], kl[t][1], kl[t][2], kl[t][3], kh[t][0], kh[t][1], kh[t][2], kh[t][3]};
+            vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
         }
-        if (it + 1 < n_tiles) issue_loads((it + 1) & 1, kv0 + kKV);
 
         // per-key scales of this lane's 32 keys (key = kv0 + 32h + 16t + e)
         float skv[SCALED ? 32 : 1], svv[SCALED ? 32 : 1];
@@ -174,41 +202,47 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                 for (int e = 0; e < 16; ++e) z[e] = 0.f;
                 s[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[t], qf[qt], z, 0, 0, 0, 0, 0, 0);
             }
+            // logits in units of log2: x = s * c (c > 0); the maximum is taken on the raw accumulators
             float x[32];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float val = s[t][e];
-                    if constexpr (SCALED) val *= skv[16 * t + e];
-                    x[16 * t + e] = val * sqc[qt];
-                }
+                for (int e = 0; e < 16; ++e) x[16 * t + e] = SCALED ? s[t][e] * skv[16 * t + e] : s[t][e];
             if (partial) {
 #pragma unroll
                 for (int e = 0; e < 32; ++e)
                     if (kv0 + 32 * h + e >= valid) x[e] = -INFINITY;
             }
-            float mx = x[0];
+            float mx = fmaxf(x[0], x[1]);
 #pragma unroll
-            for (int e = 1; e < 32; ++e) mx = fmaxf(mx, x[e]);
+            for (int e = 2; e < 32; e += 2) mx = fmaxf(fmaxf(mx, x[e]), x[e + 1]);
             mx = fmaxf(mx, lane_xor<32>(mx));
-            const float m_new = fmaxf(m_run[qt], mx);
-            const float alpha = fast_exp2(m_run[qt] - m_new);
+            const float c = sqc[qt];
+            const float m_new = fmaxf(m_run[qt], mx * c);
+            // rescale only when some row of the wave saw a new maximum (alpha is exactly 1 otherwise)
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
+                const float alpha = fast_exp2(m_run[qt] - m_new);
+                l_run[qt] *= alpha;
+#pragma unroll
+                for (int d = 0; d < 2; ++d)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[qt][d][e] *= alpha;
+            }
             m_run[qt] = m_new;
             const float m_sub = m_new - p.p_shift;
             float psum = 0.f;
             float pr[32];
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                const float pe = fast_exp2(x[e] - m_sub);
+                const float pe = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^p_shift: inside the e4m3 range
                 psum += pe;
                 pr[e] = SCALED ? pe * svv[e] : pe;
             }
             v8i pf;
 #pragma unroll
             for (int w = 0; w < 8; ++w) {
-                uint32_t u = cvt_pk_e4m3(clamp448(pr[4 * w]), clamp448(pr[4 * w + 1]), 0u, false);
-                u = cvt_pk_e4m3(clamp448(pr[4 * w + 2]), clamp448(pr[4 * w + 3]), u, true);
+                uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
+                u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
                 pf[w] = (int)u;
             }
             if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {
@@ -218,15 +252,14 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                     psum += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
                 }
             }
-            l_run[qt] = l_run[qt] * alpha + psum;
+            l_run[qt] += psum;
 #pragma unroll
-            for (int d = 0; d < 2; ++d) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o_acc[qt][d][e] *= alpha;
+            for (int d = 0; d < 2; ++d)
                 o_acc[qt][d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[d], pf, o_acc[qt][d], 0, 0, 0, 0, 0, 0);
-            }
         }
     }
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // look-ahead copies of the last tiles
 
     // ---- finalize: O^T lane (q, h), tile d, register e holds dim 32 d + 8 (e/4) + 4 h + (e%4)
 #pragma unroll
@@ -245,8 +278,8 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                 if constexpr (OUT == Q8_BF16) {
                     uint16_t* dst = reinterpret_cast<uint16_t*>(p.o) + ((size_t)bh * M + row) * 64 + dim;
                     v2i wv;
-                    wv[0] = (int)(f32_to_bf16_bits(a0) | (f32_to_bf16_bits(a1) << 16));
-                    wv[1] = (int)(f32_to_bf16_bits(a2) | (f32_to_bf16_bits(a3) << 16));
+                    wv[0] = (int)pack2_bf16(a0, a1);
+                    wv[1] = (int)pack2_bf16(a2, a3);
                     *reinterpret_cast<v2i*>(dst) = wv;
                 } else {
                     uint8_t* dst = reinterpret_cast<uint8_t*>(p.o) + ((size_t)bh * M + row) * 64 + dim;
@@ -260,6 +293,14 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
 }  // namespace q8
 
 using namespace q8;
+
+static int g_attn_cfg = 0;  // 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries
+
+extern "C" int q8_attn_set_config(int cfg) {
+    if (cfg < 0 || cfg > 2) return fail(Q8_ERR_FLAGS, "q8_attn_set_config: %d", cfg);
+    g_attn_cfg = cfg;
+    return Q8_OK;
+}
 
 extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int32_t* kv_len, const float* sq,
                            const float* sk, const float* sv, int B, int H, int M, int N, int D, int v_layout,
@@ -281,14 +322,21 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     AttnParams p{static_cast<const uint8_t*>(q), static_cast<const uint8_t*>(k), static_cast<const uint8_t*>(v), o, kv_len, sq, sk, sv,
                  B, H, M, N, v_row_stride, softmax_scale * 1.44269504088896340736f,
                  (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
-    const dim3 grid((unsigned)((M + kBlockQ - 1) / kBlockQ), (unsigned)(B * H));
-    const dim3 block(kWaves * 64);
+    if (!(softmax_scale > 0.f)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: softmax_scale must be positive");
+    const int cfg = g_attn_cfg;
+#define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV)                                                                         \
+    hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
+                                                                  (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
+#define Q8_ATTN_CFG(OUTT, SC)                                  \
+    if (cfg == 1) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4);               \
+    else if (cfg == 2) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4);          \
+    else Q8_ATTN_LAUNCH(OUTT, SC, 1, 8)
     if (out_dtype == Q8_BF16) {
-        if (scaled) hipLaunchKernelGGL((attn_fwd_kernel<Q8_BF16, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((attn_fwd_kernel<Q8_BF16, false>), grid, block, 0, stream, p);
+        if (scaled) { Q8_ATTN_CFG(Q8_BF16, true); } else { Q8_ATTN_CFG(Q8_BF16, false); }
     } else {
-        if (scaled) hipLaunchKernelGGL((attn_fwd_kernel<Q8_E4M3, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((attn_fwd_kernel<Q8_E4M3, false>), grid, block, 0, stream, p);
+        if (scaled) { Q8_ATTN_CFG(Q8_E4M3, true); } else { Q8_ATTN_CFG(Q8_E4M3, false); }
     }
+#undef Q8_ATTN_CFG
+#undef Q8_ATTN_LAUNCH
     return launch_status("q8_attn_fwd");
 }

@@ -27,13 +27,6 @@ constexpr int kPipeBM = 256, kPipeBN = 256, kPipeStages = 2, kPipeStageBytes = 6
 constexpr int kPipeLds = kPipeStages * kPipeStageBytes;
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-template <int OFFSET>
-__device__ __forceinline__ v4i lds_read_b128(unsigned addr) {
-    v4i r;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET) : "memory");
-    return r;
-}
-
 struct PipeFrags {
     v4i a[4][2];  // 4 m-tiles x (low, high) 16-byte halves of the lane's 32 K bytes
     v4i b[2][2];  // 2 n-tiles

@@ -131,6 +131,23 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// ---------------------------------------------------------------- LDS access with explicit waits
+
+// ds_read_b128 as inline assembly: invisible to the compiler's wait-count insertion, which would otherwise put
+// a full s_waitcnt vmcnt(0) in front of every LDS read that follows a global_load_lds. The caller must execute
+// an s_waitcnt lgkmcnt that names the result as an operand (lds_wait) before using it.
+template <int OFFSET>
+__device__ __forceinline__ v4i lds_read_b128(unsigned addr) {
+    v4i r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET) : "memory");
+    return r;
+}
+
+// LDS byte address of a pointer into __shared__ memory
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
 // ---------------------------------------------------------------- 8-element row chunks
 
 // Load 8 consecutive elements of `DT` starting at element index `e` of row pointer `p` into fp32.
