@@ -52,6 +52,7 @@ template <int OUT, bool SCALED, int kQT, int kWaves>
 __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams p) {
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
+    __shared__ __attribute__((aligned(256))) float lds_sc[SCALED ? kStages * 128 : 4];  // per stage: sk[64], sv[64]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int ql = lane & 31, h = lane >> 5;
     const int bh = blockIdx.y, b = bh / p.H;
@@ -108,6 +109,18 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         if (copy_v)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
                                              (__attribute__((address_space(3))) void*)(base + 4096 + cw * 1024), 16, 0, 0);
+        if constexpr (SCALED) {
+            if (wave == 0) {  // the 64 key scales and value scales of the tile, one dword per lane
+                int key = kv0 + lane;
+                key = key < N ? key : N - 1;
+                const float* zf = reinterpret_cast<const float*>(g_attn_zero16);
+                float* dst = lds_sc + (tile & (kStages - 1)) * 128;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sk + (size_t)bh * N + key : zf),
+                                                 (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sv + (size_t)bh * N + key : zf),
+                                                 (__attribute__((address_space(3))) void*)(dst + 64), 4, 0, 0);
+            }
+        }
     };
 
     // operand fetch: lane (i = lane%32, h) reads chunks 2h, 2h+1 of row (32 t + i)
@@ -140,8 +153,12 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         sv_ref = red[0];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) sv_ref = fmaxf(sv_ref, red[w]);
-        sv_inv = sv_ref > 0.f ? 1.0f / sv_ref : 0.f;
+        sv_inv = sv_ref > 0.f ? 1.0f / sv_ref : 1.f;
     }
+    // 2^p_shift / max_j sv_j, as an exponent: p' = 2^(x - m + p_shift) / svmax, P = e4m3(p' sv_j) <= 2^p_shift, l' = sum p';
+    // the factor svmax then comes out of O / l' by itself.
+    const float exp_bias = p.p_shift + (SCALED ? __builtin_log2f(sv_inv) : 0.f);
+    (void)sv_ref;
 
     if (n_tiles > 0) {
         issue_loads(0, true);
@@ -152,8 +169,13 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         const int kv0 = it * kKV;
         // tile `it` has landed (the two younger tiles may still be in flight) - for every wave after the barrier,
         // which also says that all waves are done reading tile it-1, whose stage the next copy overwrites
-        if constexpr (kWaves == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        {
+            const int per_tile = (kWaves == 4 ? 2 : 1) + ((SCALED && wave == 0) ? 2 : 0);  // copies this wave issues per tile
+            if (per_tile == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+            else if (per_tile == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else if (per_tile == 3) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        }
         __builtin_amdgcn_s_barrier();
         issue_loads(it + 3, it + 3 < n_tiles);
         const unsigned st = fbase + (it & (kStages - 1)) * kStage;
@@ -179,15 +201,24 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
             vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
         }
 
-        // per-key scales of this lane's 32 keys (key = kv0 + 32h + 16t + e)
+        // per-key scales of this lane's 32 keys (key = kv0 + 32h + e): broadcast reads from the stage's scale rows
         float skv[SCALED ? 32 : 1], svv[SCALED ? 32 : 1];
         if constexpr (SCALED) {
+            const unsigned sc = lds_addr(lds_sc) + (it & (kStages - 1)) * 512 + 128 * h;
+            v4i r[16];
+            r[0] = lds_read_b128<0>(sc); r[1] = lds_read_b128<16>(sc); r[2] = lds_read_b128<32>(sc); r[3] = lds_read_b128<48>(sc);
+            r[4] = lds_read_b128<64>(sc); r[5] = lds_read_b128<80>(sc); r[6] = lds_read_b128<96>(sc); r[7] = lds_read_b128<112>(sc);
+            r[8] = lds_read_b128<256>(sc); r[9] = lds_read_b128<272>(sc); r[10] = lds_read_b128<288>(sc); r[11] = lds_read_b128<304>(sc);
+            r[12] = lds_read_b128<320>(sc); r[13] = lds_read_b128<336>(sc); r[14] = lds_read_b128<352>(sc); r[15] = lds_read_b128<368>(sc);
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]), "+v"(r[8]),
+                           "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]), "+v"(r[15])
+                         :
+                         : "memory");
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                int key = kv0 + 32 * h + e;
-                key = key < N ? key : N - 1;
-                skv[e] = p.sk[(size_t)bh * N + key];
-                svv[e] = p.sv[(size_t)bh * N + key] * sv_inv;
+                skv[e] = __int_as_float(r[e >> 2][e & 3]);
+                svv[e] = __int_as_float(r[8 + (e >> 2)][e & 3]);
             }
         }
         const bool partial = kv0 + kKV > valid;
@@ -229,7 +260,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                     for (int e = 0; e < 16; ++e) o_acc[qt][d][e] *= alpha;
             }
             m_run[qt] = m_new;
-            const float m_sub = m_new - p.p_shift;
+            const float m_sub = m_new - exp_bias;
             float psum = 0.f;
             float pr[32];
 #pragma unroll
@@ -266,7 +297,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     for (int qt = 0; qt < kQT; ++qt) {
         const int row = q0 + 32 * qt + ql;
         float l = l_run[qt] + lane_xor<32>(l_run[qt]);
-        const float inv = ((l == 0.f || l != l) ? 1.f : 1.f / l) * sv_ref;
+        const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
         if (row >= M) continue;
 #pragma unroll
         for (int d = 0; d < 2; ++d) {
