@@ -63,9 +63,12 @@ enum {
 enum {
     Q8_ATTN_SUM_ROUNDED_P = 1, /* row sum accumulates the e4m3-rounded probabilities (what multiplies V)
                                   instead of the unrounded fp32 ones                                        */
-    Q8_ATTN_P_UNIT_RANGE = 2   /* form the probabilities as exp(s - max) <= 1 before their e4m3 cast, like the
+    Q8_ATTN_P_UNIT_RANGE = 2,  /* form the probabilities as exp(s - max) <= 1 before their e4m3 cast, like the
                                   reference; by default they are scaled by 2^8 (the factor cancels in o / l),
                                   which keeps weights below 2^-10 of the maximum from being flushed to zero  */
+    Q8_ATTN_O_TOKEN_MAJOR = 4  /* write o as [B, M, H, D] (the layout the output projection reads, which the
+                                  reference reaches by transpose(1, 2).reshape, modules/attention.py:105)
+                                  instead of [B, H, M, D]                                                     */
 };
 
 const char* q8_strerror(int status);
@@ -120,6 +123,42 @@ int q8_rmsnorm(const void* x, int x_dtype, const float* w, void* y, int y_dtype,
  */
 int q8_rope(const void* x, int x_dtype, const float* cos_t, const float* sin_t, void* y, int y_dtype,
             int64_t rows, int dim, q8_stream_t stream);
+
+/*
+ * Fused row kernels: launch sequences of the reference with the 16-bit tensor between two kernels kept in
+ * registers. Each intermediate value is rounded to `mid_dtype` exactly where the unfused sequence stores it
+ * (mid_dtype = Q8_BF16 gives the same bits as the separate calls; Q8_F32 skips that rounding).
+ *
+ * q8_fht_quant_rows: codes, scales = quant(FHT(x) * fht_scale). The prologue of the int8 linear layer,
+ *   hadamard_transform followed by quantize (q8_kernels/functional/linear.py:30-31), = q8_fht then q8_quant_rows.
+ * q8_rmsnorm_quant_rows: codes, scales = quant(rmsnorm(x, w)); rstd (nullable) as q8_rmsnorm. The norm in front
+ *   of an 8-bit projection (q8_kernels/modules/attention.py:67-77) = q8_rmsnorm then q8_quant_rows.
+ * x_dtype in {BF16, E4M3}; code_dtype in {I8, E4M3}; flags as q8_quant_rows; rows contiguous; dim as the row kernels.
+ */
+int q8_fht_quant_rows(const void* x, int x_dtype, void* codes, int code_dtype, float* scales, int64_t rows,
+                      int dim, float fht_scale, int mid_dtype, int flags, q8_stream_t stream);
+int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* codes, int code_dtype, float* scales,
+                          float* rstd, int64_t rows, int dim, float eps, int mid_dtype, int flags,
+                          q8_stream_t stream);
+
+/*
+ * Attention prologues: from token-major 16-bit projections [B, S, H*D] (row stride in elements, so a slice of a
+ * fused QKV projection can be passed without a copy) to the e4m3 operands of q8_attn_fwd.
+ * Replaces the torch glue of flash_attn_func (q8_kernels/functional/flash_attention.py:38-55: transpose, pad,
+ * cast, hadamard_transform) and the RoPE in front of it (q8_kernels/modules/attention.py:84-87).
+ *
+ * q8_attn_prep_qk: per token and head: [RoPE with tables cos, sin fp32 [B*S, H*D], both NULL = none] ->
+ *   [D-point FHT * scale if apply_fht] -> e4m3 codes [B, H, S, D]. scales == NULL: direct c10 cast (the
+ *   reference's cast); otherwise one absmax scale per (token, head) to scales [B, H, S].
+ *   D in {64, 128}; H * D in {64, 128, 256} or a multiple of 512 up to 4096.
+ * q8_attn_prep_v: e4m3 codes [B, H, D, S_pad] (Q8_V_DS), columns S..S_pad-1 zero, S_pad % 16 == 0;
+ *   scales as above. D == 64.
+ */
+int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
+                    float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                    q8_stream_t stream);
+int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
+                   int S_pad, q8_stream_t stream);
 
 /*
  * 8-bit GEMM with fused dequantisation, bias and tanh-GELU.

@@ -239,14 +239,15 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
                     batch_mask: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
                     q_scales: Optional[torch.Tensor] = None, k_scales: Optional[torch.Tensor] = None,
                     v_scales: Optional[torch.Tensor] = None, sum_rounded_p: bool = False,
-                    p_unit_range: bool = False) -> torch.Tensor:
+                    p_unit_range: bool = False, token_major_out: bool = False) -> torch.Tensor:
     """csrc/flash_attention/flash_attention.cpp:18-48.
 
     q [B,H,M,64], k [B,H,N,64], v [B,H,64,Nv] (pre-transposed, Nv >= N, Nv % 16 == 0), all e4m3 and contiguous;
     batch_mask int32 [B] of valid KV lengths. Returns [B,H,M,64] in out_dtype (None -> e4m3 like the reference).
     The keyword arguments are extensions: bf16 output, per-token dequantisation scales
     (q_scales [B,H,M], k_scales / v_scales [B,H,N], fp32), and p_unit_range=True to round the probabilities
-    on the reference's grid (p <= 1) instead of the default 2^8 p, which does not flush small weights.
+    on the reference's grid (p <= 1) instead of the default 2^8 p, which does not flush small weights;
+    token_major_out=True returns [B,M,H*64], the transpose(1, 2).reshape the callers apply next.
     """
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
         _check_input(t, name)
@@ -276,11 +277,117 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
     out_dtype = torch.float8_e4m3fn if out_dtype is None else out_dtype
     if out_dtype not in (torch.bfloat16, torch.float8_e4m3fn):
         raise RuntimeError("flash_attention: out_dtype must be bfloat16 or float8_e4m3fn")
-    out = torch.empty((bs, heads, m, d), dtype=out_dtype, device=q.device)
+    out = torch.empty((bs, m, heads * d) if token_major_out else (bs, heads, m, d), dtype=out_dtype, device=q.device)
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().q8_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(batch_mask),
                                           _ptr(q_scales), _ptr(k_scales), _ptr(v_scales), bs, heads, m, n, d,
                                           _lib.Q8_V_DS, v.shape[3], float(softmax_scale), _DT[out_dtype],
                                           (_lib.Q8_ATTN_SUM_ROUNDED_P if sum_rounded_p else 0) |
-                                          (_lib.Q8_ATTN_P_UNIT_RANGE if p_unit_range else 0), _stream(q)))
+                                          (_lib.Q8_ATTN_P_UNIT_RANGE if p_unit_range else 0) |
+                                          (_lib.Q8_ATTN_O_TOKEN_MAJOR if token_major_out else 0), _stream(q)))
     return out
+
+
+# ----------------------------------------------------------------------------- fused row kernels
+# No counterpart among the reference's bindings: each replaces a sequence of two or more of the calls above and
+# returns the same bits (intermediate values are rounded to bfloat16 where the sequence stores a bfloat16 tensor).
+
+def _quant_out(x2, out_type, who):
+    out_type = torch.int8 if out_type is None else out_type
+    if out_type not in (torch.int8, torch.float8_e4m3fn):
+        raise RuntimeError("%s not implemented for output type '%s'" % (who, out_type))
+    rows, dim = x2.shape
+    return (out_type, torch.empty((rows, dim), dtype=out_type, device=x2.device),
+            torch.empty((rows,), dtype=torch.float32, device=x2.device))
+
+
+def fht_quant(x: torch.Tensor, scale: float, out_type: Optional[torch.dtype] = None, *,
+              round_intermediate: bool = True) -> List[torch.Tensor]:
+    """tokenwise_quant(fast_hadamard_transform(x, scale, bfloat16), out_type) in one pass over x.
+    x bfloat16 or e4m3 with last dim a multiple of 8. Returns [codes(x.shape), scales(x.shape[:-1])]."""
+    _require_gpu(x, "x")
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("fht_quant: input must be bfloat16 or float8_e4m3fn")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).contiguous()
+    out_type, out, scales = _quant_out(x2, out_type, "fht_quant")
+    rows, dim = x2.shape
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_fht_quant_rows(x2.data_ptr(), _DT[x2.dtype], out.data_ptr(), _DT[out_type],
+                                                scales.data_ptr(), rows, dim, float(scale),
+                                                Q8_BF16 if round_intermediate else Q8_F32, 0, _stream(x)))
+    return [out.reshape(shape), scales.reshape(shape[:-1])]
+
+
+def rms_norm_quant(x: torch.Tensor, weights: Optional[torch.Tensor] = None, out_type: Optional[torch.dtype] = None, *,
+                   eps: float = 0.0, round_intermediate: bool = True) -> List[torch.Tensor]:
+    """tokenwise_quant(rms_norm(x, weights, bfloat16)[0], out_type) in one pass over x.
+    Returns [codes(x.shape), scales(x.shape[:-1]), rstd(x.shape[:-1])]."""
+    _require_gpu(x, "x")
+    if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise RuntimeError("rms_norm_quant: input must be bfloat16 or float8_e4m3fn")
+    if weights is not None and (weights.dtype != torch.float32 or not weights.is_cuda):
+        raise RuntimeError("rms_norm_quant: weights must be a float32 CUDA tensor")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).contiguous()
+    out_type, out, scales = _quant_out(x2, out_type, "rms_norm_quant")
+    rows, dim = x2.shape
+    if weights is not None and weights.numel() != dim:
+        raise RuntimeError("rms_norm_quant: weights must have %d elements" % dim)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_rmsnorm_quant_rows(x2.data_ptr(), _DT[x2.dtype], _ptr(weights), out.data_ptr(),
+                                                    _DT[out_type], scales.data_ptr(), rstd.data_ptr(), rows, dim,
+                                                    float(eps), Q8_BF16 if round_intermediate else Q8_F32, 0,
+                                                    _stream(x)))
+    return [out.reshape(shape), scales.reshape(shape[:-1]), rstd.reshape(shape[:-1])]
+
+
+def _token_major(x, num_heads, who):
+    """x [B, S, H*D] bfloat16 with unit last stride and one row stride over (B, S)."""
+    _require_gpu(x, "x")
+    if x.dtype != torch.bfloat16 or x.dim() != 3:
+        raise RuntimeError("%s: x must be a bfloat16 tensor [B, S, H*D]" % who)
+    b, s, dim = x.shape
+    if dim % num_heads != 0:
+        raise RuntimeError("%s: last dim %d is not divisible by %d heads" % (who, dim, num_heads))
+    if x.stride(2) != 1 or (b > 1 and x.stride(0) != s * x.stride(1)) or x.data_ptr() % 16 != 0 or x.stride(1) % 8 != 0:
+        x = x.contiguous()
+    return x, b, s, dim // num_heads
+
+
+def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
+                 sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
+                 per_token_scales: bool = False, *, round_intermediate: bool = True):
+    """x [B, S, H*D] bfloat16 (a strided slice of a fused projection is fine) -> e4m3 [B, H, S, D]:
+    optional RoPE (tables fp32 [B, S, H*D]), head split, optional D-point Hadamard transform times `scale`,
+    then the direct e4m3 cast, or per-(token, head) absmax quantization when per_token_scales
+    (returns (codes, scales [B, H, S]) in that case)."""
+    x, b, s, d = _token_major(x, num_heads, "attn_prep_qk")
+    if (cos is None) != (sin is None):
+        raise RuntimeError("attn_prep_qk: cos and sin come together")
+    if cos is not None:
+        for t in (cos, sin):
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != x.numel():
+                raise RuntimeError("attn_prep_qk: tables must be float32 CUDA tensors of x's shape")
+        cos, sin = cos.contiguous(), sin.contiguous()
+    codes = torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((b, num_heads, s), dtype=torch.float32, device=x.device) if per_token_scales else None
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_attn_prep_qk(x.data_ptr(), x.stride(1), _ptr(cos), _ptr(sin), codes.data_ptr(),
+                                              _ptr(scales), b, s, num_heads, d, int(apply_fht), float(scale),
+                                              Q8_BF16 if round_intermediate else Q8_F32, _stream(x)))
+    return (codes, scales) if per_token_scales else codes
+
+
+def attn_prep_v(x: torch.Tensor, num_heads: int, per_token_scales: bool = False):
+    """x [B, S, H*64] bfloat16 -> e4m3 [B, H, 64, S_pad] (S_pad = S rounded up to 16, zero filled), the V operand
+    of flash_attention; with per_token_scales also scales [B, H, S]."""
+    x, b, s, d = _token_major(x, num_heads, "attn_prep_v")
+    s_pad = (s + 15) // 16 * 16
+    codes = torch.empty((b, num_heads, d, s_pad), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((b, num_heads, s), dtype=torch.float32, device=x.device) if per_token_scales else None
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_attn_prep_v(x.data_ptr(), x.stride(1), codes.data_ptr(), _ptr(scales), b, s,
+                                             num_heads, d, s_pad, _stream(x)))
+    return (codes, scales) if per_token_scales else codes

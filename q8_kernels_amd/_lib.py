@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libq8_hip.so")
 Q8_I8, Q8_E4M3, Q8_BF16, Q8_F16, Q8_F32 = 0, 1, 2, 3, 4
 Q8_QUANT_RNE, Q8_QUANT_SCALE_DIV = 1, 2
 Q8_V_DS, Q8_V_SD = 0, 1
-Q8_ATTN_SUM_ROUNDED_P, Q8_ATTN_P_UNIT_RANGE = 1, 2
+Q8_ATTN_SUM_ROUNDED_P, Q8_ATTN_P_UNIT_RANGE, Q8_ATTN_O_TOKEN_MAJOR = 1, 2, 4
 
 _c = ctypes
 _vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
@@ -27,6 +27,10 @@ SIGNATURES = {
     "q8_fht": (_i, [_vp, _i, _vp, _i, _i64, _i, _f, _vp]),
     "q8_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i64, _i, _f, _vp]),
     "q8_rope": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i64, _i, _vp]),
+    "q8_fht_quant_rows": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _f, _i, _i, _vp]),
+    "q8_rmsnorm_quant_rows": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i64, _i, _f, _i, _i, _vp]),
+    "q8_attn_prep_qk": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "q8_attn_prep_v": (_i, [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "q8_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "q8_gemm_i32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "q8_gemm_set_config": (_i, [_i]),

@@ -41,36 +41,30 @@ class Fp8DiTBlock(nn.Module):
                 m.bias.data = (torch.randn(m.bias.shape, generator=g) * std).to(torch.bfloat16).float().to(dev)
         return self
 
-    def _heads(self, t, b):
-        return t.view(b, -1, self.num_heads, self.head_dim).transpose(1, 2)
-
-    def _merge(self, t, b):
-        return t.transpose(1, 2).reshape(b, -1, self.dim)
-
     def _lin(self, layer, x, fuse_gelu=False):
         return Q8F.linear.fp8_linear(x, layer.weight.data, layer.bias.data, None, layer.scales, False, x.dtype,
                                      fuse_gelu=fuse_gelu)
 
+    def _norm_lin(self, norm, layer, x, fuse_gelu=False):
+        """layer(norm(x)) with the norm and the e4m3 quantizer of the layer's input in one kernel."""
+        codes, scales = Q8F.fused.rms_norm_quantize(x, norm.weight, torch.float8_e4m3fn)
+        return Q8F.linear.fp8_linear(codes, layer.weight.data, layer.bias.data, scales, layer.scales, False, x.dtype,
+                                     fuse_gelu=fuse_gelu)
+
     def forward(self, hidden, text, freqs_cis, text_lens):
-        b = hidden.shape[0]
         bf16 = torch.bfloat16
-        # self-attention
-        h = self.norm1(hidden)
-        qkv = self._lin(self.to_qkv, h)
-        q, k, v = qkv.split(self.dim, dim=-1)
-        q = Q8F.rope.apply_rope(q.contiguous(), freqs_cis[0], freqs_cis[1])
-        k = Q8F.rope.apply_rope(k.contiguous(), freqs_cis[0], freqs_cis[1])
-        a = Q8F.flash_attention.flash_attn_func(self._heads(q, b), self._heads(k, b), self._heads(v, b),
-                                                apply_qk_hadamard=True, out_dtype=bf16)
-        hidden = hidden + self._lin(self.to_out, self._merge(a, b))
+        d, h = self.dim, self.num_heads
+        # self-attention: q, k, v are read in place from the fused projection by the attention prologue kernels
+        qkv = self._norm_lin(self.norm1, self.to_qkv, hidden)
+        a = Q8F.fused.flash_attn_token_major(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], h,
+                                             apply_qk_hadamard=True, freqs_cis=freqs_cis, out_dtype=bf16)
+        hidden = hidden + self._lin(self.to_out, a)
         # cross-attention to the text states
-        h = self.norm2(hidden)
-        q2 = self._lin(self.to_q2, h)
+        q2 = self._norm_lin(self.norm2, self.to_q2, hidden)
         k2, v2 = self._lin(self.to_k2, text), self._lin(self.to_v2, text)
-        a = Q8F.flash_attention.flash_attn_func(self._heads(q2, b), self._heads(k2, b), self._heads(v2, b),
-                                                batch_mask=text_lens, apply_qk_hadamard=True, out_dtype=bf16)
-        hidden = hidden + self._lin(self.to_out2, self._merge(a, b))
+        a = Q8F.fused.flash_attn_token_major(q2, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
+                                             out_dtype=bf16)
+        hidden = hidden + self._lin(self.to_out2, a)
         # feed-forward
-        h = self.norm3(hidden)
-        up = self._lin(self.ff_up, h, fuse_gelu=True)
+        up = self._norm_lin(self.norm3, self.ff_up, hidden, fuse_gelu=True)
         return hidden + self._lin(self.ff_down, up)

@@ -66,6 +66,10 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     const uint8_t* Kg = p.k + (size_t)bh * N * 64;
     const uint8_t* Vg = p.v + (size_t)bh * 64 * p.v_row_stride;
     const int q0 = blockIdx.x * kBlockQ + wave * (kQT * 32);
+    // output row r of this (batch, head): element offset o_base + r * o_rs
+    const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
+    const size_t o_base = o_tok ? ((size_t)b * M * p.H + (size_t)(bh - b * p.H)) * 64 : (size_t)bh * M * 64;
+    const size_t o_rs = o_tok ? (size_t)p.H * 64 : 64;
 
     // Q^T operand: lane (q, h) holds bytes 32h .. 32h+31 of query row q
     v8i qf[kQT];
@@ -307,13 +311,13 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                 const float a0 = o_acc[qt][d][4 * w] * inv, a1 = o_acc[qt][d][4 * w + 1] * inv;
                 const float a2 = o_acc[qt][d][4 * w + 2] * inv, a3 = o_acc[qt][d][4 * w + 3] * inv;
                 if constexpr (OUT == Q8_BF16) {
-                    uint16_t* dst = reinterpret_cast<uint16_t*>(p.o) + ((size_t)bh * M + row) * 64 + dim;
+                    uint16_t* dst = reinterpret_cast<uint16_t*>(p.o) + o_base + (size_t)row * o_rs + dim;
                     v2i wv;
                     wv[0] = (int)pack2_bf16(a0, a1);
                     wv[1] = (int)pack2_bf16(a2, a3);
                     *reinterpret_cast<v2i*>(dst) = wv;
                 } else {
-                    uint8_t* dst = reinterpret_cast<uint8_t*>(p.o) + ((size_t)bh * M + row) * 64 + dim;
+                    uint8_t* dst = reinterpret_cast<uint8_t*>(p.o) + o_base + (size_t)row * o_rs + dim;
                     *reinterpret_cast<uint32_t*>(dst) = pack4_e4m3_sat(a0, a1, a2, a3);
                 }
             }
@@ -342,7 +346,7 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);
     if (out_dtype != Q8_BF16 && out_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_attn_fwd: output dtype %d", out_dtype);
-    if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
+    if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE | Q8_ATTN_O_TOKEN_MAJOR)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
     if (v_layout != Q8_V_DS) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V layout %d (only Q8_V_DS [B,H,64,Nv] is implemented)", v_layout);
     if (v_row_stride < N || v_row_stride % 16 != 0)
         return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V row stride %lld must be >= N and a multiple of 16", (long long)v_row_stride);

@@ -1,0 +1,399 @@
+// Row kernels that fuse what the reference runs as separate launches with a 16-bit tensor in HBM between them:
+//   FHT -> token-wise quantizer            (the Q8Linear prologue, q8_kernels/functional/linear.py:30-31)
+//   RMSNorm -> token-wise quantizer        (norm followed by an 8-bit linear, q8_kernels/modules/attention.py:67-77)
+//   RoPE -> head split -> FHT -> e4m3      (the Q / K side of q8_kernels/functional/flash_attention.py:47-55)
+//   head split -> e4m3 -> transpose        (the V side, flash_attention.py:38-45)
+// Every intermediate value is rounded to the dtype the unfused sequence would have stored (template MID), so the
+// results are the same bits as the separate kernels give.
+#include "rows_common.h"
+
+namespace q8 {
+
+// ---- FHT -> quantizer ------------------------------------------------------------------------------
+
+template <int LANES, int CH, int IN, int OUT, int MID>
+__global__ __launch_bounds__(kBlock) void fht_quant_kernel(const void* __restrict__ x, void* __restrict__ codes,
+                                                           float* __restrict__ scales, int64_t rows, int dim,
+                                                           float fht_scale, int flags) {
+    constexpr int RPB = kBlock / LANES;
+    constexpr int IN_B = (IN == Q8_E4M3) ? 1 : 2;
+    __shared__ float red[4];
+    const int t = threadIdx.x % LANES;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
+    const bool row_ok = row < rows;
+    const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
+
+    float v[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (row_ok && e < dim) {
+            load8<IN>(xr, e, v[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+        }
+    }
+    fht_row<LANES, CH>(v, t);
+
+    float amax[1] = {0.f};
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[c][i] = round_mid<MID>(v[c][i] * fht_scale);
+            if (e < dim) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));  // outputs beyond dim are dropped
+        }
+    }
+    row_reduce<LANES, true, 1>(amax, red);
+    if (!row_ok) return;
+    const float ratio = quant_ratio<OUT>(amax[0]);
+    if (t == 0) scales[row] = quant_scale<OUT>(amax[0], ratio, flags);
+    uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
+    }
+}
+
+// ---- RMSNorm -> quantizer ----------------------------------------------------------------------------
+
+template <int LANES, int CH, int IN, int OUT, int MID>
+__global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __restrict__ x, const float* __restrict__ w,
+                                                               void* __restrict__ codes, float* __restrict__ scales,
+                                                               float* __restrict__ rstd_out, int64_t rows, int dim,
+                                                               float eps, int flags) {
+    constexpr int RPB = kBlock / LANES;
+    constexpr int IN_B = (IN == Q8_E4M3) ? 1 : 2;
+    __shared__ float red[4];
+    const int t = threadIdx.x % LANES;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
+    const bool row_ok = row < rows;
+    const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
+
+    float v[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (row_ok && e < dim) {
+            load8<IN>(xr, e, v[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+        }
+    }
+    float ss[1] = {0.f};
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss[0] += v[c][i] * v[c][i];
+    row_reduce<LANES, false, 1>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss[0] * (1.0f / (float)dim) + eps);
+
+    float amax[1] = {0.f};
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (e >= dim) continue;  // the padding stays zero
+        if (w != nullptr) {
+            float wv[8];
+            load8<Q8_F32>(w, e, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = round_mid<MID>((v[c][i] * rstd) * wv[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = round_mid<MID>(v[c][i] * rstd);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));
+    }
+    row_reduce<LANES, true, 1>(amax, red);
+    if (!row_ok) return;
+    const float ratio = quant_ratio<OUT>(amax[0]);
+    if (t == 0) {
+        scales[row] = quant_scale<OUT>(amax[0], ratio, flags);
+        if (rstd_out != nullptr) rstd_out[row] = rstd;
+    }
+    uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
+    }
+}
+
+// ---- attention prologue for Q and K ---------------------------------------------------------------------
+//
+// LANES threads per token: the row of H * D = 8 * LANES * CH elements (H heads of D = 8 * LH) uses the row mapping,
+// so a head is one group of LH consecutive lanes of one chunk and the D-point Hadamard transform is the register
+// stages plus log2(LH) lane stages. Codes go to the head-major layout [B, H, S, D] the attention kernel reads.
+// The options are uniform branches: cs != NULL rotates, scales != NULL quantizes per (token, head).
+template <int LANES, int CH, int LH>
+__global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
+                                                              const float* __restrict__ cs, const float* __restrict__ sn,
+                                                              uint8_t* __restrict__ codes, float* __restrict__ scales,
+                                                              int64_t tokens, int S, int apply_fht, float scale,
+                                                              int mid_bf16) {
+    static_assert(LH <= LANES, "a head may not span tokens");
+    constexpr int DIM = LANES * CH * 8, D = LH * 8, H = DIM / D;
+    const int t = threadIdx.x % LANES;
+    const int64_t tok = (int64_t)blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES;
+    if (tok >= tokens) return;  // no barrier below; the lane exchanges stay inside a head, i.e. inside a token
+    const int64_t b = tok / S, s = tok - b * S;
+    const uint16_t* xr = x + tok * x_row_stride;
+    auto mid = [&](float f) { return mid_bf16 ? round_mid<Q8_BF16>(f) : f; };
+
+    float v[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) load8<Q8_BF16>(xr, (c * LANES + t) * 8, v[c]);
+    if (cs != nullptr) {
+        // interleaved pairs with per-element tables (csrc/ops/rope_cuda.cu:99-103)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int64_t e = tok * DIM + (c * LANES + t) * 8;
+            float cv[8], sv[8], o[8];
+            load8<Q8_F32>(cs, e, cv);
+            load8<Q8_F32>(sn, e, sv);
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                o[i] = v[c][i] * cv[i] - v[c][i + 1] * sv[i];
+                o[i + 1] = v[c][i + 1] * cv[i + 1] + v[c][i] * sv[i + 1];
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = mid(o[i]);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if (apply_fht) {
+#pragma unroll
+            for (int st = 1; st < 8; st <<= 1) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if ((i & st) == 0) {
+                        const float a0 = v[c][i], b0 = v[c][i + st];
+                        v[c][i] = a0 + b0;
+                        v[c][i + st] = a0 - b0;
+                    }
+                }
+            }
+            fht_lane_stage<1>(v[c], (unsigned)(t & 1) << 31);
+            fht_lane_stage<2>(v[c], (unsigned)(t & 2) << 30);
+            fht_lane_stage<4>(v[c], 0u);
+            if constexpr (LH > 8) fht_lane_stage<8>(v[c], 0u);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] *= scale;
+        }
+        const int h = (c * LANES + t) / LH;
+        const int64_t orow = (b * H + h) * S + s;
+        v2i w;
+        if (scales != nullptr) {
+            float amax = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[c][i] = mid(v[c][i]);
+                amax = fmaxf(amax, fabsf(v[c][i]));
+            }
+            amax = group_max<LH>(amax);
+            const float ratio = quant_ratio<Q8_E4M3>(amax);
+            if ((t % LH) == 0) scales[orow] = quant_scale<Q8_E4M3>(amax, ratio, 0);
+            w = quant_codes8<Q8_E4M3>(v[c], ratio, 0);
+        } else {
+            w[0] = (int)pack4_e4m3_c10(v[c][0], v[c][1], v[c][2], v[c][3]);
+            w[1] = (int)pack4_e4m3_c10(v[c][4], v[c][5], v[c][6], v[c][7]);
+        }
+        *reinterpret_cast<v2i*>(codes + orow * D + (t % LH) * 8) = w;
+    }
+}
+
+// ---- attention prologue for V ---------------------------------------------------------------------------
+//
+// x [B, S, H * 64] (token-major, bf16) -> e4m3 codes [B, H, 64, S_pad] (channel-major per head, the layout of the
+// attention kernel's V operand), columns S..S_pad-1 zero. One block transposes 64 tokens x 64 channels of one head
+// through LDS. SCALED: one absmax scale per (token, head), written to scales [B, H, S].
+template <bool SCALED>
+__global__ __launch_bounds__(kBlock) void attn_prep_v_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
+                                                             uint8_t* __restrict__ codes, float* __restrict__ scales,
+                                                             int S, int S_pad, int H) {
+    __shared__ uint32_t tile[64][17];  // [token][channel / 4], one pad word per row
+    const int b = blockIdx.z, h = blockIdx.y, s0 = blockIdx.x * 64;
+    {
+        const int tok = threadIdx.x >> 2, part = threadIdx.x & 3;  // 16 channels per thread
+        const int s = s0 + tok;
+        float v[2][8];
+        if (s < S) {
+            const uint16_t* xr = x + ((int64_t)b * S + s) * x_row_stride + h * 64 + part * 16;
+            load8<Q8_BF16>(xr, 0, v[0]);
+            load8<Q8_BF16>(xr, 8, v[1]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[0][i] = v[1][i] = 0.f;
+        }
+        uint32_t w[4];
+        if constexpr (SCALED) {
+            float amax = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fmaxf(fabsf(v[0][i]), fabsf(v[1][i])));
+            amax = group_max<4>(amax);
+            const float ratio = quant_ratio<Q8_E4M3>(amax);
+            if (part == 0 && s < S) scales[((int64_t)b * H + h) * S + s] = quant_scale<Q8_E4M3>(amax, ratio, 0);
+            const v2i c0 = quant_codes8<Q8_E4M3>(v[0], ratio, 0), c1 = quant_codes8<Q8_E4M3>(v[1], ratio, 0);
+            w[0] = (uint32_t)c0[0]; w[1] = (uint32_t)c0[1]; w[2] = (uint32_t)c1[0]; w[3] = (uint32_t)c1[1];
+        } else {
+            w[0] = pack4_e4m3_c10(v[0][0], v[0][1], v[0][2], v[0][3]);
+            w[1] = pack4_e4m3_c10(v[0][4], v[0][5], v[0][6], v[0][7]);
+            w[2] = pack4_e4m3_c10(v[1][0], v[1][1], v[1][2], v[1][3]);
+            w[3] = pack4_e4m3_c10(v[1][4], v[1][5], v[1][6], v[1][7]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tile[tok][part * 4 + i] = w[i];
+    }
+    __syncthreads();
+    {
+        const int d = threadIdx.x >> 2, part = threadIdx.x & 3;  // channel d, tokens part * 16 .. + 15
+        if (s0 + part * 16 >= S_pad) return;
+        const uint8_t* tb = reinterpret_cast<const uint8_t*>(&tile[0][0]);
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t acc = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc |= (uint32_t)tb[(part * 16 + i * 4 + j) * 68 + d] << (8 * j);
+            w[i] = acc;
+        }
+        uint8_t* out = codes + (((int64_t)b * H + h) * 64 + d) * S_pad + s0 + part * 16;
+        *reinterpret_cast<v4u*>(out) = v4u{w[0], w[1], w[2], w[3]};
+    }
+}
+
+}  // namespace q8
+
+using namespace q8;
+
+static int check_quant_args(const char* who, const void* x, int x_dtype, const void* codes, int code_dtype,
+                            const float* scales, int mid_dtype, int flags) {
+    if (!x || !codes || !scales) return fail(Q8_ERR_NULL, "%s: null pointer", who);
+    if (flags & ~(Q8_QUANT_RNE | Q8_QUANT_SCALE_DIV)) return fail(Q8_ERR_FLAGS, "%s: flags 0x%x", who, flags);
+    if (code_dtype != Q8_I8 && code_dtype != Q8_E4M3)
+        return fail(Q8_ERR_DTYPE, "%s: code dtype %d (want I8 or E4M3)", who, code_dtype);
+    if (x_dtype != Q8_BF16 && x_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "%s: input dtype %d (want BF16 or E4M3)", who, x_dtype);
+    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32)
+        return fail(Q8_ERR_DTYPE, "%s: intermediate dtype %d (want BF16 or F32)", who, mid_dtype);
+    if ((reinterpret_cast<uintptr_t>(x) % (x_dtype == Q8_BF16 ? 16 : 8)) || (reinterpret_cast<uintptr_t>(codes) % 8) ||
+        (reinterpret_cast<uintptr_t>(scales) % 4))
+        return fail(Q8_ERR_ALIGN, "%s: x must be 16-byte (bf16) or 8-byte (e4m3) aligned, codes 8-byte aligned", who);
+    return Q8_OK;
+}
+
+#define Q8_FUSED_SWITCH(XD, CD, MD, ...)                                                              \
+    if (XD == Q8_BF16 && CD == Q8_I8 && MD == Q8_BF16) { constexpr int IN = Q8_BF16, OUT = Q8_I8, MID = Q8_BF16; __VA_ARGS__; } \
+    else if (XD == Q8_BF16 && CD == Q8_E4M3 && MD == Q8_BF16) { constexpr int IN = Q8_BF16, OUT = Q8_E4M3, MID = Q8_BF16; __VA_ARGS__; } \
+    else if (XD == Q8_BF16 && CD == Q8_I8) { constexpr int IN = Q8_BF16, OUT = Q8_I8, MID = Q8_F32; __VA_ARGS__; } \
+    else if (XD == Q8_BF16) { constexpr int IN = Q8_BF16, OUT = Q8_E4M3, MID = Q8_F32; __VA_ARGS__; } \
+    else if (CD == Q8_I8 && MD == Q8_BF16) { constexpr int IN = Q8_E4M3, OUT = Q8_I8, MID = Q8_BF16; __VA_ARGS__; } \
+    else if (CD == Q8_E4M3 && MD == Q8_BF16) { constexpr int IN = Q8_E4M3, OUT = Q8_E4M3, MID = Q8_BF16; __VA_ARGS__; } \
+    else if (CD == Q8_I8) { constexpr int IN = Q8_E4M3, OUT = Q8_I8, MID = Q8_F32; __VA_ARGS__; } \
+    else { constexpr int IN = Q8_E4M3, OUT = Q8_E4M3, MID = Q8_F32; __VA_ARGS__; }
+
+extern "C" int q8_fht_quant_rows(const void* x, int x_dtype, void* codes, int code_dtype, float* scales, int64_t rows,
+                                 int dim, float fht_scale, int mid_dtype, int flags, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int st = check_rows("q8_fht_quant_rows", rows, dim)) return st;
+    if (rows == 0) return Q8_OK;
+    if (int st = check_quant_args("q8_fht_quant_rows", x, x_dtype, codes, code_dtype, scales, mid_dtype, flags)) return st;
+    const int N = pow2_ceil(dim);
+    Q8_FUSED_SWITCH(x_dtype, code_dtype, mid_dtype, {
+        Q8_ROW_SHAPE_SWITCH(N, {
+            const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            hipLaunchKernelGGL((fht_quant_kernel<LANES, CH, IN, OUT, MID>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+                               x, codes, scales, rows, dim, fht_scale, flags);
+        })
+    })
+    return launch_status("q8_fht_quant_rows");
+}
+
+extern "C" int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* codes, int code_dtype,
+                                     float* scales, float* rstd, int64_t rows, int dim, float eps, int mid_dtype,
+                                     int flags, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int st = check_rows("q8_rmsnorm_quant_rows", rows, dim)) return st;
+    if (rows == 0) return Q8_OK;
+    if (int st = check_quant_args("q8_rmsnorm_quant_rows", x, x_dtype, codes, code_dtype, scales, mid_dtype, flags)) return st;
+    if (w && !aligned16(w)) return fail(Q8_ERR_ALIGN, "q8_rmsnorm_quant_rows: weights must be 16-byte aligned");
+    const int N = pow2_ceil(dim);
+    Q8_FUSED_SWITCH(x_dtype, code_dtype, mid_dtype, {
+        Q8_ROW_SHAPE_SWITCH(N, {
+            const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            hipLaunchKernelGGL((rmsnorm_quant_kernel<LANES, CH, IN, OUT, MID>), dim3((unsigned)grid), dim3(kBlock), 0,
+                               stream, x, w, codes, scales, rstd, rows, dim, eps, flags);
+        })
+    })
+    return launch_status("q8_rmsnorm_quant_rows");
+}
+
+extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
+                               float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                               q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (B < 0 || S < 0 || H <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: B %d S %d H %d", B, S, H);
+    if (D != 64 && D != 128) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: head dim %d (want 64 or 128)", D);
+    const int64_t dim = (int64_t)H * D;
+    const bool small = dim == 64 || dim == 128 || dim == 256;
+    if (!small && (dim % 512 != 0 || dim > 4096))
+        return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: H * D = %lld must be 64, 128, 256 or a multiple of 512 up to 4096", (long long)dim);
+    if ((int64_t)B * S == 0) return Q8_OK;
+    if (!x || !codes) return fail(Q8_ERR_NULL, "q8_attn_prep_qk: null pointer");
+    if ((cos_t == nullptr) != (sin_t == nullptr)) return fail(Q8_ERR_NULL, "q8_attn_prep_qk: cos and sin come together");
+    if (x_row_stride < dim || x_row_stride % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: row stride %lld", (long long)x_row_stride);
+    if (!aligned16(x) || (cos_t && (!aligned16(cos_t) || !aligned16(sin_t))) || (reinterpret_cast<uintptr_t>(codes) % 8))
+        return fail(Q8_ERR_ALIGN, "q8_attn_prep_qk: x and tables must be 16-byte aligned, codes 8-byte aligned");
+    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32) return fail(Q8_ERR_DTYPE, "q8_attn_prep_qk: intermediate dtype %d", mid_dtype);
+    const int64_t tokens = (int64_t)B * S;
+    const int lanes = small ? (int)(dim / 8) : 64;
+    const int64_t grid = (tokens + (kBlock / lanes) - 1) / (kBlock / lanes);
+    if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: too many tokens");
+#define PREP_LAUNCH(LANES, CH, LH)                                                                                  \
+    hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH>), dim3((unsigned)grid), dim3(kBlock), 0, stream,         \
+                       static_cast<const uint16_t*>(x), x_row_stride, cos_t, sin_t, static_cast<uint8_t*>(codes), \
+                       scales, tokens, S, apply_fht, scale, mid_dtype == Q8_BF16 ? 1 : 0)
+#define PREP_D(LANES, CH) \
+    if (D == 64) PREP_LAUNCH(LANES, CH, 8); else PREP_LAUNCH(LANES, CH, 16)
+    switch (dim) {
+        case 64: PREP_LAUNCH(8, 1, 8); break;
+        case 128: PREP_D(16, 1); break;
+        case 256: PREP_D(32, 1); break;
+        case 512: PREP_D(64, 1); break;
+        case 1024: PREP_D(64, 2); break;
+        case 1536: PREP_D(64, 3); break;
+        case 2048: PREP_D(64, 4); break;
+        case 2560: PREP_D(64, 5); break;
+        case 3072: PREP_D(64, 6); break;
+        case 3584: PREP_D(64, 7); break;
+        default: PREP_D(64, 8); break;
+    }
+#undef PREP_D
+#undef PREP_LAUNCH
+    return launch_status("q8_attn_prep_qk");
+}
+
+extern "C" int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
+                              int S_pad, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (B < 0 || S < 0 || H <= 0 || H > 65535 || B > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: B %d S %d H %d", B, S, H);
+    if (D != 64) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: head dim %d (want 64)", D);
+    if (S_pad < S || S_pad % 16 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: S_pad %d must be a multiple of 16 >= S %d", S_pad, S);
+    if (B == 0 || S_pad == 0) return Q8_OK;
+    if (!x || !codes) return fail(Q8_ERR_NULL, "q8_attn_prep_v: null pointer");
+    if (x_row_stride < (int64_t)H * D || x_row_stride % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: row stride %lld", (long long)x_row_stride);
+    if (!aligned16(x) || !aligned16(codes)) return fail(Q8_ERR_ALIGN, "q8_attn_prep_v: x and codes must be 16-byte aligned");
+    const dim3 grid((unsigned)((S_pad + 63) / 64), (unsigned)H, (unsigned)B);
+    if (scales)
+        hipLaunchKernelGGL((attn_prep_v_kernel<true>), grid, dim3(kBlock), 0, stream, static_cast<const uint16_t*>(x),
+                           x_row_stride, static_cast<uint8_t*>(codes), scales, S, S_pad, H);
+    else
+        hipLaunchKernelGGL((attn_prep_v_kernel<false>), grid, dim3(kBlock), 0, stream, static_cast<const uint16_t*>(x),
+                           x_row_stride, static_cast<uint8_t*>(codes), scales, S, S_pad, H);
+    return launch_status("q8_attn_prep_v");
+}

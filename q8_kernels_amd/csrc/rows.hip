@@ -1,45 +1,8 @@
 // Memory-bound row kernels for gfx950: token-wise absmax quantizer, fast Walsh-Hadamard transform,
-// RMSNorm and RoPE.
-//
-// Row mapping shared by the three reducing kernels: a row of `dim` elements is padded to
-// N = 8 * LANES * CH (a power of two). LANES consecutive threads own a row, thread t of the row holds
-// the elements (c * LANES + t) * 8 + 0..7 for c = 0..CH-1, i.e. one 128-bit bf16 load per chunk.
-// A block is 256 threads = 256 / LANES rows. Element-index bits therefore map, low to high, to
-// (register index, lane, wave, chunk), which is also the order in which the Hadamard butterflies
-// run, so that every output is produced by the same sequence of fp32 additions as the ascending-stride
-// butterfly network of the reference (csrc/fast_hadamard/fast_hadamard_transform_cuda.cu:84-108).
-//
-// fp contraction is off in this file: products and sums round separately, like the element-wise fp32
-// arithmetic they are checked against.
-#include "q8_common.h"
-#include "q8_host.h"
-
-#pragma clang fp contract(off)
+// RMSNorm and RoPE. The thread-to-element mapping and the shared arithmetic are in rows_common.h.
+#include "rows_common.h"
 
 namespace q8 {
-
-constexpr int kBlock = 256;
-
-// ---- reductions over the LANES threads of a row (LANES <= 256) -------------------------------
-
-template <int LANES, bool IS_MAX>
-__device__ __forceinline__ float row_reduce(float v, float* red) {
-    constexpr int WL = LANES < 64 ? LANES : 64;
-    v = IS_MAX ? group_max<WL>(v) : group_sum<WL>(v);
-    if constexpr (LANES > 64) {
-        constexpr int WPR = LANES / 64;  // waves per row
-        const int wave = threadIdx.x >> 6;
-        if ((threadIdx.x & 63) == 0) red[wave] = v;
-        __syncthreads();
-        const int w0 = (wave / WPR) * WPR;
-        float r = red[w0];
-#pragma unroll
-        for (int i = 1; i < WPR; ++i) r = IS_MAX ? fmaxf(r, red[w0 + i]) : (r + red[w0 + i]);
-        __syncthreads();
-        v = r;
-    }
-    return v;
-}
 
 // ---- token-wise quantizer -----------------------------------------------------------------------
 
@@ -47,78 +10,55 @@ template <int LANES, int CH, int IN, int OUT>
 __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const void* __restrict__ x, void* __restrict__ codes,
                                                             float* __restrict__ scales, int64_t rows, int dim,
                                                             int64_t x_row_stride, int flags) {
-    constexpr int RPB = kBlock / LANES;
-    __shared__ float red[4];
+    constexpr int RPB = kBlock / LANES, RPT = RowsPerThread<LANES, CH>::value;
+    constexpr int ESZ = (IN == Q8_F32 ? 4 : (IN == Q8_E4M3 ? 1 : 2));
+    __shared__ float red[RPT * 4];
     const int t = threadIdx.x % LANES;
-    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
-    const bool row_ok = row < rows;
-    const char* xr = reinterpret_cast<const char*>(x) + row * x_row_stride * (IN == Q8_F32 ? 4 : (IN == Q8_E4M3 ? 1 : 2));
-
-    float v[CH][8];
-    float amax = 0.f;
+    int64_t row[RPT];
+    bool row_ok[RPT];
+    float v[RPT][CH][8];
+    float amax[RPT];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<IN>(xr, e, v[c]);
-        } else {
+    for (int r = 0; r < RPT; ++r) {
+        row[r] = ((int64_t)blockIdx.x * RPT + r) * RPB + threadIdx.x / LANES;
+        row_ok[r] = row[r] < rows;
+        const char* xr = reinterpret_cast<const char*>(x) + row[r] * x_row_stride * ESZ;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
-        }
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (row_ok[r] && e < dim) {
+                load8<IN>(xr, e, v[r][c]);
+            } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[c][i]));
-    }
-    amax = row_reduce<LANES, true>(amax, red);
-
-    constexpr float QMAX = (OUT == Q8_I8) ? 127.f : 448.f;
-    // reference order: r = QMAX / absmax, code = x * r, stored scale = 1 / r
-    // (csrc/quantizer/tokenwise_quant_cuda.cu:135-147), in IEEE fp32.
-    const float r = (amax > 0.f) ? QMAX / amax : 0.f;
-    if (row_ok && t == 0) {
-        float s = 0.f;
-        if (amax > 0.f) s = (flags & Q8_QUANT_SCALE_DIV) ? amax / QMAX : 1.0f / r;
-        scales[row] = s;
-    }
-    if (!row_ok) return;
-    uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (e >= dim) continue;
-        v2i w;
-        if constexpr (OUT == Q8_I8) {
-            uint32_t b[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float q = v[c][i] * r;
-                const float qr = (flags & Q8_QUANT_RNE) ? rintf(q) : roundf(q);
-                b[i] = (uint32_t)(int)qr & 0xffu;
+                for (int i = 0; i < 8; ++i) v[r][c][i] = 0.f;
             }
-            w[0] = (int)(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24));
-            w[1] = (int)(b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
-        } else {
-            // |x * r| <= 448 (1 + 2^-23): never reaches the NaN range of the c10 cast
-            uint32_t p0 = cvt_pk_e4m3(v[c][0] * r, v[c][1] * r, 0u, false);
-            p0 = cvt_pk_e4m3(v[c][2] * r, v[c][3] * r, p0, true);
-            uint32_t p1 = cvt_pk_e4m3(v[c][4] * r, v[c][5] * r, 0u, false);
-            p1 = cvt_pk_e4m3(v[c][6] * r, v[c][7] * r, p1, true);
-            w[0] = (int)p0;
-            w[1] = (int)p1;
         }
-        *reinterpret_cast<v2i*>(out + e) = w;
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        amax[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax[r] = fmaxf(amax[r], fabsf(v[r][c][i]));
+    }
+    row_reduce<LANES, true, RPT>(amax, red);
+
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        if (!row_ok[r]) continue;
+        const float ratio = quant_ratio<OUT>(amax[r]);
+        if (t == 0) scales[row[r]] = quant_scale<OUT>(amax[r], ratio, flags);
+        uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row[r] * (int64_t)dim;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[r][c], ratio, flags);
+        }
     }
 }
 
 // ---- fast Walsh-Hadamard transform --------------------------------------------------------------
-
-template <int MASK>
-__device__ __forceinline__ void fht_lane_stage(float (&v)[8], int lane_bit_set) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float o = lane_xor<MASK>(v[i]);
-        v[i] = lane_bit_set ? (o - v[i]) : (v[i] + o);
-    }
-}
 
 template <int LANES, int CH, int IN, int OUT>
 __global__ __launch_bounds__(kBlock) void fht_kernel(const void* __restrict__ x, void* __restrict__ y, int64_t rows,
@@ -143,79 +83,7 @@ __global__ __launch_bounds__(kBlock) void fht_kernel(const void* __restrict__ x,
         }
     }
 
-    // element bits 0..2: inside the 8 registers of a chunk
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-#pragma unroll
-        for (int s = 1; s < 8; s <<= 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if ((i & s) == 0) {
-                    const float a = v[c][i], b = v[c][i + s];
-                    v[c][i] = a + b;
-                    v[c][i + s] = a - b;
-                }
-            }
-        }
-    }
-    // lane bits
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if constexpr (LANES > 1) fht_lane_stage<1>(v[c], t & 1);
-        if constexpr (LANES > 2) fht_lane_stage<2>(v[c], t & 2);
-        if constexpr (LANES > 4) fht_lane_stage<4>(v[c], t & 4);
-        if constexpr (LANES > 8) fht_lane_stage<8>(v[c], t & 8);
-        if constexpr (LANES > 16) fht_lane_stage<16>(v[c], t & 16);
-        if constexpr (LANES > 32) fht_lane_stage<32>(v[c], t & 32);
-    }
-    // wave bits: one exchange through LDS per chunk, both stages evaluated from the 2 or 4 wave values
-    if constexpr (LANES > 64) {
-        __shared__ v4f xch[2][kBlock];
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            xch[0][threadIdx.x] = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
-            xch[1][threadIdx.x] = v4f{v[c][4], v[c][5], v[c][6], v[c][7]};
-            __syncthreads();
-            auto peer = [&](int w, float (&o)[8]) {
-                const v4f a = xch[0][w * 64 + lane], b = xch[1][w * 64 + lane];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
-            };
-            float p1[8];
-            peer(wave ^ 1, p1);
-            if constexpr (LANES == 128) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[c][i] = (wave & 1) ? (p1[i] - v[c][i]) : (v[c][i] + p1[i]);
-            } else {
-                float p2[8], p3[8];
-                peer(wave ^ 2, p2);
-                peer(wave ^ 3, p3);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float ya = (wave & 1) ? (p1[i] - v[c][i]) : (v[c][i] + p1[i]);
-                    const float yb = (wave & 1) ? (p3[i] - p2[i]) : (p2[i] + p3[i]);
-                    v[c][i] = (wave & 2) ? (yb - ya) : (ya + yb);
-                }
-            }
-            __syncthreads();
-        }
-    }
-    // chunk bits
-#pragma unroll
-    for (int s = 1; s < CH; s <<= 1) {
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            if ((c & s) == 0) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float a = v[c][i], b = v[c + s][i];
-                    v[c][i] = a + b;
-                    v[c + s][i] = a - b;
-                }
-            }
-        }
-    }
+    fht_row<LANES, CH>(v, t);
 
     if (!row_ok) return;
     char* yr = reinterpret_cast<char*>(y) + row * (int64_t)dim * OUT_B;
@@ -235,49 +103,62 @@ template <int LANES, int CH, int IN, int OUT>
 __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const void* __restrict__ x, const float* __restrict__ w,
                                                          void* __restrict__ y, float* __restrict__ rstd_out,
                                                          int64_t rows, int dim, float eps) {
-    constexpr int RPB = kBlock / LANES;
+    constexpr int RPB = kBlock / LANES, RPT = RowsPerThread<LANES, CH>::value;
     constexpr int IN_B = (IN == Q8_E4M3) ? 1 : 2;
     constexpr int OUT_B = (OUT == Q8_E4M3) ? 1 : 2;
-    __shared__ float red[4];
+    __shared__ float red[RPT * 4];
     const int t = threadIdx.x % LANES;
-    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
-    const bool row_ok = row < rows;
-    const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
-
-    float v[CH][8];
-    float ss = 0.f;
+    int64_t row[RPT];
+    bool row_ok[RPT];
+    float v[RPT][CH][8];
+    float ss[RPT];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<IN>(xr, e, v[c]);
-        } else {
+    for (int r = 0; r < RPT; ++r) {
+        row[r] = ((int64_t)blockIdx.x * RPT + r) * RPB + threadIdx.x / LANES;
+        row_ok[r] = row[r] < rows;
+        const char* xr = reinterpret_cast<const char*>(x) + row[r] * (int64_t)dim * IN_B;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (row_ok[r] && e < dim) {
+                load8<IN>(xr, e, v[r][c]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[r][c][i] = 0.f;
+            }
         }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) ss += v[c][i] * v[c][i];
     }
-    ss = row_reduce<LANES, false>(ss, red);
-    // rstd = rsqrt(mean(x^2)) with no epsilon in the reference (csrc/ops/rms_norm_cuda.cu:127-156)
-    const float rstd = 1.0f / sqrtf(ss * (1.0f / (float)dim) + eps);
-    if (!row_ok) return;
-    if (rstd_out != nullptr && t == 0) rstd_out[row] = rstd;
-    char* yr = reinterpret_cast<char*>(y) + row * (int64_t)dim * OUT_B;
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (e >= dim) continue;
-        if (w != nullptr) {
-            float wv[8];
-            load8<Q8_F32>(w, e, wv);
+    for (int r = 0; r < RPT; ++r) {
+        ss[r] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = (v[c][i] * rstd) * wv[i];
-        } else {
+        for (int c = 0; c < CH; ++c)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = v[c][i] * rstd;
+            for (int i = 0; i < 8; ++i) ss[r] += v[r][c][i] * v[r][c][i];
+    }
+    row_reduce<LANES, false, RPT>(ss, red);
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        if (!row_ok[r]) continue;
+        // rstd = rsqrt(mean(x^2)) with no epsilon in the reference (csrc/ops/rms_norm_cuda.cu:127-156)
+        const float rstd = 1.0f / sqrtf(ss[r] * (1.0f / (float)dim) + eps);
+        if (rstd_out != nullptr && t == 0) rstd_out[row[r]] = rstd;
+        char* yr = reinterpret_cast<char*>(y) + row[r] * (int64_t)dim * OUT_B;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (e >= dim) continue;
+            if (w != nullptr) {
+                float wv[8];
+                load8<Q8_F32>(w, e, wv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[r][c][i] = (v[r][c][i] * rstd) * wv[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[r][c][i] = v[r][c][i] * rstd;
+            }
+            store8<OUT>(yr, e, v[r][c]);
         }
-        store8<OUT>(yr, e, v[c]);
     }
 }
 
@@ -303,40 +184,6 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(const void* __restrict__ x
     store8<OUT>(y, e, o);
 }
 
-// ---- dispatch ------------------------------------------------------------------------------------
-
-// N = padded row length (power of two, 8..32768): LANES = min(N / 8, 256), CH = N / (8 * LANES).
-#define Q8_ROW_SHAPE_SWITCH(N, ...)                                                       \
-    switch (N) {                                                                          \
-        case 8:     { constexpr int LANES = 1,   CH = 1;  __VA_ARGS__; } break;           \
-        case 16:    { constexpr int LANES = 2,   CH = 1;  __VA_ARGS__; } break;           \
-        case 32:    { constexpr int LANES = 4,   CH = 1;  __VA_ARGS__; } break;           \
-        case 64:    { constexpr int LANES = 8,   CH = 1;  __VA_ARGS__; } break;           \
-        case 128:   { constexpr int LANES = 16,  CH = 1;  __VA_ARGS__; } break;           \
-        case 256:   { constexpr int LANES = 32,  CH = 1;  __VA_ARGS__; } break;           \
-        case 512:   { constexpr int LANES = 64,  CH = 1;  __VA_ARGS__; } break;           \
-        case 1024:  { constexpr int LANES = 128, CH = 1;  __VA_ARGS__; } break;           \
-        case 2048:  { constexpr int LANES = 256, CH = 1;  __VA_ARGS__; } break;           \
-        case 4096:  { constexpr int LANES = 256, CH = 2;  __VA_ARGS__; } break;           \
-        case 8192:  { constexpr int LANES = 256, CH = 4;  __VA_ARGS__; } break;           \
-        case 16384: { constexpr int LANES = 256, CH = 8;  __VA_ARGS__; } break;           \
-        case 32768: { constexpr int LANES = 256, CH = 16; __VA_ARGS__; } break;           \
-        default: return fail(Q8_ERR_SHAPE, "row length %d not supported", (int)(N));      \
-    }
-
-static int pow2_ceil(int d) {
-    int n = 8;
-    while (n < d) n <<= 1;
-    return n;
-}
-
-static int check_rows(const char* who, int64_t rows, int dim) {
-    if (rows < 0) return fail(Q8_ERR_SHAPE, "%s: rows = %lld", who, (long long)rows);
-    if (dim <= 0 || dim % 8 != 0 || dim > 32768)
-        return fail(Q8_ERR_SHAPE, "%s: dim = %d must be a multiple of 8 in [8, 32768]", who, dim);
-    return Q8_OK;
-}
-
 }  // namespace q8
 
 using namespace q8;
@@ -360,7 +207,8 @@ extern "C" int q8_quant_rows(const void* x, int x_dtype, void* codes, int code_d
     const int N = pow2_ceil(dim);
 #define LAUNCH_Q(IN, OUT)                                                                              \
     Q8_ROW_SHAPE_SWITCH(N, {                                                                           \
-        const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);                         \
+        constexpr int RB = (kBlock / LANES) * RowsPerThread<LANES, CH>::value;                         \
+        const int64_t grid = (rows + RB - 1) / RB;                                                     \
         hipLaunchKernelGGL((quant_rows_kernel<LANES, CH, IN, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, \
                            codes, scales, rows, dim, x_row_stride, flags);                             \
     })
@@ -419,7 +267,8 @@ extern "C" int q8_rmsnorm(const void* x, int x_dtype, const float* w, void* y, i
     const int N = pow2_ceil(dim);
     Q8_IO_SWITCH(x_dtype, y_dtype, {
         Q8_ROW_SHAPE_SWITCH(N, {
-            const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            constexpr int RB = (kBlock / LANES) * RowsPerThread<LANES, CH>::value;
+            const int64_t grid = (rows + RB - 1) / RB;
             hipLaunchKernelGGL((rmsnorm_kernel<LANES, CH, IN, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, w, y,
                                rstd, rows, dim, eps);
         })

@@ -1,0 +1,65 @@
+"""Fused forms of operator sequences that the reference runs as separate launches. Every function returns the
+same bits as the sequence it names; none has a counterpart of its own in the reference.
+
+    hadamard_quantize      = quantize(hadamard_transform(x))              (q8_kernels/functional/linear.py:30-31)
+    rms_norm_quantize      = quantize(rms_norm_8bit(x, w)[0])             (q8_kernels/modules/attention.py:67-77)
+    flash_attn_token_major = apply_rope -> split heads -> flash_attn_func -> merge heads
+                                                                          (q8_kernels/modules/attention.py:84-105)
+"""
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _C
+
+_FP8 = torch.float8_e4m3fn
+
+
+def hadamard_quantize(x: torch.Tensor, out_type: Optional[torch.dtype] = None,
+                      scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bfloat16 x (..., dim) -> (codes, scales) of the Hadamard-rotated rows; out_type None -> int8."""
+    if scale is None:
+        scale = 1.0 / math.sqrt(x.shape[-1])
+    codes, scales = _C.fht_quant(x, scale, out_type)
+    return codes, scales
+
+
+def can_fuse_hadamard_quantize(x: torch.Tensor) -> bool:
+    """The fused kernel reproduces the two-kernel sequence for bfloat16 inputs whose rows need no padding."""
+    return x.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 and x.shape[-1] <= 32768
+
+
+def rms_norm_quantize(x: torch.Tensor, weights: Optional[torch.Tensor] = None,
+                      out_type: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bfloat16 x -> (codes, scales) of rms_norm(x) * weights; out_type None -> int8."""
+    codes, scales, _ = _C.rms_norm_quant(x, weights, out_type)
+    return codes, scales
+
+
+def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int,
+                           softmax_scale: Optional[float] = None, batch_mask: Optional[torch.Tensor] = None,
+                           apply_qk_hadamard: bool = False, freqs_cis=None, out_dtype: Optional[torch.dtype] = None,
+                           per_token_scales: bool = False) -> torch.Tensor:
+    """q [B, M, H*64], k, v [B, N, H*64] bfloat16 projections (strided slices of a fused projection are read in
+    place) -> attention output [B, M, H*64].
+
+    freqs_cis = (cos, sin) fp32 tables of q's shape rotates q and k first (k must then have q's shape).
+    Without per_token_scales the operands are cast to e4m3 exactly as flash_attn_func does; with it each
+    (token, head) row of q, k and v gets its own absmax scale."""
+    d = q.shape[-1] // num_heads
+    if softmax_scale is None:
+        softmax_scale = d ** (-0.5)
+    cos, sin = (None, None) if freqs_cis is None else freqs_cis
+    if apply_qk_hadamard:
+        qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
+    else:
+        qk_scale, kernel_scale = 1.0, softmax_scale
+    qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+    kc = _C.attn_prep_qk(k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+    vc = _C.attn_prep_v(v, num_heads, per_token_scales)
+    if per_token_scales:
+        (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
+        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
+                                  v_scales=vs, token_major_out=True)
+    return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True)

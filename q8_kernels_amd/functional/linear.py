@@ -9,6 +9,7 @@ import torch
 
 from .. import _C
 from .fast_hadamard import hadamard_transform
+from .fused import can_fuse_hadamard_quantize, hadamard_quantize
 from .quantizer import quantize, quantize_fp8
 
 _FP8 = torch.float8_e4m3fn
@@ -31,10 +32,13 @@ def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = N
         "Q8LinearFunc: b dtype missmatch"
     assert a.shape[-1] == b.shape[-1], "Q8LinearFunc: mnk missmatch"
     assert bias is None or bias.dtype == torch.float, "Q8LinearFunc: bias must be in fp32"
+    def rotate_quant(t):  # one kernel where it gives the bits of the two
+        return hadamard_quantize(t) if can_fuse_hadamard_quantize(t) else quantize(hadamard_transform(t))
+
     if a_needs_q:
-        a, scale_a = quantize(hadamard_transform(a))
+        a, scale_a = rotate_quant(a)
     if b_needs_q:
-        b, scale_b = quantize(hadamard_transform(b))
+        b, scale_b = rotate_quant(b)
     if bias is not None:
         return _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
     return _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
@@ -56,7 +60,11 @@ def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = 
     assert out_dtype is not None and is_16bit(out_dtype), "FP8LinearFunc: out_dtype must be in 16bit"
 
     def quant(t):
-        return quantize_fp8(hadamard_transform(t)) if use_hadamard else quantize_fp8(t)
+        if use_hadamard:
+            if can_fuse_hadamard_quantize(t):
+                return hadamard_quantize(t, _FP8)
+            return quantize_fp8(hadamard_transform(t))
+        return quantize_fp8(t)
 
     if is_16bit(a):
         a, scale_a = quant(a)

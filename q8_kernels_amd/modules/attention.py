@@ -13,6 +13,10 @@ from .rms_norm import RMSNorm
 
 
 class Attention(nn.Module):
+    # False runs the reference's operator sequence (rope, split heads, flash_attn_func, merge) kernel by kernel;
+    # True (default) takes the fused prologue kernels where they apply. Both give the same bits.
+    fuse_prologue = True
+
     def __init__(self, query_dim: int, num_heads: int, head_dim: int, bias: bool = False, out_bias: bool = False,
                  out_dim: Optional[int] = None, qk_rms_norm: bool = False, kv_dim: Optional[int] = None,
                  use_rope: bool = False):
@@ -51,11 +55,20 @@ class Attention(nn.Module):
         if self.qk_rms_norm:
             query = self.q_norm(query, non_mm_precision)
             key = self.k_norm(key, non_mm_precision)
-        if encoder_hidden_states is None and self.use_rope:
+        rope = encoder_hidden_states is None and self.use_rope
+        batch = query.shape[0]
+        if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64 and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
+                and non_mm_precision == torch.bfloat16 and query.dim() == 3
+                and all(t.dtype == torch.bfloat16 for t in (query, key, value))):
+            # one prologue kernel per operand and head-merged output: the same bits as the sequence below
+            hidden_states = Q8F.fused.flash_attn_token_major(
+                query, key, value, self.num_heads, batch_mask=attention_mask, apply_qk_hadamard=apply_qk_hadamard,
+                freqs_cis=freqs_cis if rope else None)
+            return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
+        if rope:
             query = Q8F.rope.apply_rope(query, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)
             key = Q8F.rope.apply_rope(key, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)
 
-        batch = query.shape[0]
         query, key, value = (self._split_heads(t, batch) for t in (query, key, value))
 
         if attn_type == "q8_kernels":

@@ -33,7 +33,7 @@ def test_header_enums_match_python_constants():
     from q8_kernels_amd import _lib
     text = open(HEADER).read()
     for name in ("Q8_I8", "Q8_E4M3", "Q8_BF16", "Q8_F16", "Q8_F32", "Q8_QUANT_RNE", "Q8_QUANT_SCALE_DIV",
-                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE"):
+                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR"):
         m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
         assert m, name
         assert int(m.group(1)) == getattr(_lib, name), name

@@ -1,0 +1,201 @@
+"""GPU parity of the fused row kernels (FHT+quantizer, RMSNorm+quantizer, attention prologues) through
+q8_kernels_amd._C -> libq8_hip.so. Each fused kernel must return the same bits as the CPU oracle's composition
+of the separate operators (and therefore as the separate HIP kernels, which are checked on their own)."""
+import pytest
+import torch
+
+from oracle import q8_oracle as O
+from tests.util import E4M3, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+def _C():
+    from q8_kernels_amd import _C as C
+    return C
+
+
+# ------------------------------------------------------------------ FHT -> quantizer
+
+@pytest.mark.parametrize("dim", [64, 512, 1000, 2048, 4096, 8192])
+@pytest.mark.parametrize("out_type", [torch.int8, E4M3])
+def test_fht_quant_bit_exact(dev, dim, out_type):
+    g = torch.Generator().manual_seed(dim + 1)
+    for rows in (1, 33, 130):
+        x = (torch.randn(rows, dim, generator=g) * 2).to(BF16)
+        x[rows // 2] = 0
+        scale = dim ** -0.5
+        codes, scales = _C().fht_quant(x.to(dev), scale, out_type)
+        wc, ws = O.ref_quant(O.ref_fht(x, scale, BF16), out_type)
+        assert_bit_equal(codes, wc, "codes dim=%d rows=%d" % (dim, rows))
+        assert_bit_equal(scales, ws, "scales dim=%d rows=%d" % (dim, rows))
+
+
+def test_fht_quant_fp8_input_and_unrounded_intermediate(dev):
+    g = torch.Generator().manual_seed(5)
+    x = O.e4m3_c10(torch.randn(3, 7, 256, generator=g) * 4)
+    codes, scales = _C().fht_quant(x.to(dev), 1.0 / 16, None)
+    wc, ws = O.ref_quant(O.ref_fht(x, 1.0 / 16, BF16), None)
+    assert codes.shape == x.shape and scales.shape == x.shape[:-1]
+    assert_bit_equal(codes, wc, "codes")
+    assert_bit_equal(scales, ws, "scales")
+    # without the bf16 rounding of the transform: quantizer applied to the fp32 transform
+    xb = (torch.randn(9, 512, generator=g)).to(BF16)
+    codes, scales = _C().fht_quant(xb.to(dev), 512 ** -0.5, E4M3, round_intermediate=False)
+    y32 = O.ref_fht(xb, 512 ** -0.5, torch.float32) if _accepts_f32() else None
+    if y32 is not None:
+        wc, ws = O.ref_quant(y32, E4M3)
+        assert_bit_equal(codes, wc, "codes (fp32 intermediate)")
+        assert_bit_equal(scales, ws, "scales (fp32 intermediate)")
+
+
+def _accepts_f32():
+    try:
+        return O.ref_fht(torch.zeros(1, 8, dtype=BF16), 1.0, torch.float32).dtype == torch.float32
+    except Exception:
+        return False
+
+
+def test_fht_quant_equals_separate_kernels_full_size(dev):
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(12288, 2048, generator=g).to(BF16).to(dev)
+    codes, scales = _C().fht_quant(x, 2048 ** -0.5, None)
+    wc, ws = _C().tokenwise_quant(_C().fast_hadamard_transform(x, 2048 ** -0.5, None), None)
+    assert_bit_equal(codes, wc, "codes")
+    assert_bit_equal(scales, ws, "scales")
+
+
+# ------------------------------------------------------------------ RMSNorm -> quantizer
+
+@pytest.mark.parametrize("dim", [64, 1000, 2048, 8192])
+@pytest.mark.parametrize("out_type", [torch.int8, E4M3])
+def test_rmsnorm_quant(dev, dim, out_type):
+    g = torch.Generator().manual_seed(dim + 2)
+    for rows, with_w in ((1, True), (37, True), (130, False)):
+        x = (torch.randn(rows, dim, generator=g) * 1.7).to(BF16)
+        w = (1 + 0.1 * torch.randn(dim, generator=g)) if with_w else None
+        codes, scales, rstd = _C().rms_norm_quant(x.to(dev), None if w is None else w.to(dev), out_type)
+        # the separate kernels use the same summation order: bit for bit
+        y, rstd_sep = _C().rms_norm(x.to(dev), None if w is None else w.to(dev), BF16)
+        wc, ws = _C().tokenwise_quant(y, out_type)
+        assert_bit_equal(codes, wc, "codes vs separate kernels")
+        assert_bit_equal(scales, ws, "scales vs separate kernels")
+        assert_bit_equal(rstd, rstd_sep, "rstd vs separate kernels")
+        # against the oracle: the row sum of squares is accumulated in another order, so rstd may differ in its
+        # last bits and a code may move by one step where x * rstd * w falls on a rounding boundary
+        yo, ro = O.ref_rms_norm(x, w, BF16)
+        oc, os_ = O.ref_quant(yo, out_type)
+        assert torch.allclose(rstd.cpu(), ro, rtol=2e-6, atol=0)
+        deq = codes.cpu().float() * scales.cpu()[:, None]
+        want = oc.float() * os_[:, None]
+        step = os_[:, None] * (1.0 if out_type == torch.int8 else 32.0)
+        assert bool(((deq - want).abs() <= step * 1.001).all())
+        assert float((codes.cpu().view(torch.uint8) != oc.view(torch.uint8)).float().mean()) < 0.01
+
+
+# ------------------------------------------------------------------ attention prologues
+
+def _heads(t, h):
+    b, s, dim = t.shape
+    return t.view(b, s, h, dim // h).transpose(1, 2).contiguous()
+
+
+@pytest.mark.parametrize("shape", [(2, 70, 8, 64), (1, 33, 32, 64), (2, 19, 8, 128), (1, 5, 64, 64), (2, 37, 4, 64),
+                                   (3, 5, 1, 64), (1, 9, 24, 64), (2, 7, 2, 128)])
+@pytest.mark.parametrize("rope", [False, True])
+@pytest.mark.parametrize("fht", [False, True])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_qk(dev, shape, rope, fht, scaled):
+    b, s, h, d = shape
+    dim = h * d
+    g = torch.Generator().manual_seed(b * 1000 + s + dim)
+    x = (torch.randn(b, s, dim, generator=g) * 1.5).to(BF16)
+    x[0, s // 2] = 0
+    cos = sin = None
+    if rope:
+        ang = torch.rand(b, s, dim // 2, generator=g) * 6.28
+        cos, sin = torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1)
+    scale = (d ** -0.5) * (0.125 ** 0.5)
+    got = _C().attn_prep_qk(x.to(dev), h, None if cos is None else cos.to(dev), None if sin is None else sin.to(dev),
+                            fht, scale, scaled)
+    y = O.ref_rope(x, cos, sin, BF16) if rope else x
+    y = _heads(y, h)
+    if scaled:
+        y = O.ref_fht(y, scale, BF16) if fht else y
+        wc, ws = O.ref_quant(y, E4M3)
+        assert_bit_equal(got[0], wc, "codes")
+        assert_bit_equal(got[1], ws, "scales")
+    else:
+        want = O.ref_fht(y, scale, E4M3) if fht else O.e4m3_c10(y)
+        assert_bit_equal(got, want, "codes")
+
+
+def test_attn_prep_qk_strided_slice_of_fused_projection(dev):
+    g = torch.Generator().manual_seed(77)
+    qkv = torch.randn(2, 50, 3 * 2048, generator=g).to(BF16)
+    qkv_d = qkv.to(dev)
+    for i in range(3):
+        got = _C().attn_prep_qk(qkv_d[..., i * 2048:(i + 1) * 2048], 32, None, None, True, 0.125, False)
+        want = O.ref_fht(_heads(qkv[..., i * 2048:(i + 1) * 2048].contiguous(), 32), 0.125, E4M3)
+        assert_bit_equal(got, want, "slice %d" % i)
+
+
+@pytest.mark.parametrize("shape", [(2, 70, 8), (1, 128, 32), (2, 16, 3), (1, 6144, 2)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_v(dev, shape, scaled):
+    b, s, h = shape
+    g = torch.Generator().manual_seed(s + h)
+    x = (torch.randn(b, s, h * 64, generator=g) * 2).to(BF16)
+    got = _C().attn_prep_v(x.to(dev), h, scaled)
+    s_pad = (s + 15) // 16 * 16
+    v = _heads(x, h)  # [b, h, s, 64]
+    if scaled:
+        wc, ws = O.ref_quant(v, E4M3)
+        assert_bit_equal(got[1], ws, "scales")
+        got = got[0]
+    else:
+        wc = O.e4m3_c10(v)
+    want = torch.zeros(b, h, 64, s_pad, dtype=torch.uint8)
+    want[..., :s] = wc.view(torch.uint8).transpose(2, 3)
+    assert got.shape == (b, h, 64, s_pad)
+    assert torch.equal(got.cpu().view(torch.uint8), want)
+
+
+def test_prologues_feed_attention_like_the_functional_path(dev):
+    """flash_attn_func on [B,H,S,D] tensors == prologue kernels on the token-major projections + the kernel."""
+    import q8_kernels_amd.functional as Q8F
+    g = torch.Generator().manual_seed(91)
+    b, s, h, d = 2, 200, 8, 64
+    q, k, v = ((torch.randn(b, s, h * d, generator=g)).to(BF16).to(dev) for _ in range(3))
+    want = Q8F.flash_attention.flash_attn_func(_heads(q, h), _heads(k, h), _heads(v, h), apply_qk_hadamard=True,
+                                               out_dtype=BF16)
+    sc = (d ** -0.5) * ((d ** -0.5) ** 0.5)
+    qc = _C().attn_prep_qk(q, h, None, None, True, sc)
+    kc = _C().attn_prep_qk(k, h, None, None, True, sc)
+    vc = _C().attn_prep_v(v, h)
+    got = _C().flash_attention(qc, kc, vc, 1.0, None, out_dtype=BF16)
+    assert_bit_equal(got, want, "attention output")
+
+
+def test_attention_module_fused_path_equals_operator_sequence(dev):
+    import torch.nn as nn
+    from q8_kernels_amd.modules import Attention, Q8Linear
+    torch.manual_seed(2)
+    attn = Attention(256, 8, 64, bias=True, out_bias=True, qk_rms_norm=True, use_rope=True).to(dev)
+    for name in ("to_q", "to_k", "to_v", "to_out"):
+        m = getattr(attn, name)
+        src = nn.Linear(m.in_features, m.out_features).to(dev).to(BF16)
+        q = Q8Linear.from_linear(src)
+        m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    x = torch.randn(2, 77, 256, device=dev).to(BF16)
+    ang = torch.rand(2, 77, 256, device=dev) * 6.28
+    freqs = (torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1))
+    kw = dict(freqs_cis=freqs, mm_out_dtype=BF16, attn_type="q8_kernels")
+    fused = attn(x, **kw)
+    try:
+        Attention.fuse_prologue = False
+        seq = attn(x, **kw)
+    finally:
+        Attention.fuse_prologue = True
+    assert_bit_equal(fused, seq, "attention module output")
