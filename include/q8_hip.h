@@ -125,6 +125,37 @@ int q8_rope(const void* x, int x_dtype, const float* cos_t, const float* sin_t, 
             int64_t rows, int dim, q8_stream_t stream);
 
 /*
+ * out = x * (y + scale_add) + z, the AdaLN modulation.
+ * Replaces ops._C.fma_8bit  (csrc/ops/fma.cpp:63-112, kernel csrc/ops/fma_cuda.cu:61-98).
+ * x, out [rows, dim]; y and z are broadcast over groups of consecutive rows: row r reads row r / y_rows_every of y
+ * (the reference: one row of y per batch entry or per token, fma.cpp:85-86). The product and the sum round once
+ * (a fused multiply-add, which is what the reference's expression compiles to).
+ * x_dtype, out_dtype in {E4M3 (the reference), BF16}; y_dtype, z_dtype in {F32, BF16, E4M3} (the reference has the
+ * pairs F32/F32, F32/E4M3, BF16/BF16); dim % 8 == 0 (the reference: 2048 or 8192 only, fma_cuda.cu:117-122).
+ */
+int q8_fma(const void* x, int x_dtype, const void* y, int y_dtype, const void* z, int z_dtype, void* out,
+           int out_dtype, int64_t rows, int dim, int64_t y_rows_every, int64_t z_rows_every, float scale_add,
+           q8_stream_t stream);
+
+/*
+ * tanh-GELU and the operators of the backward pass (the LoRA fine-tuning path of the reference).
+ *   q8_gelu             replaces ops._C.gelu_forward      (csrc/ops/gelu_act.cpp, kernel gelu_forward_cuda.cu:12-16,73-100)
+ *   q8_gelu_backward    replaces ops._C.gelu_backward     (kernel gelu_backward_cuda.cu:67-105): out = grad * dGELU(x)
+ *   q8_rope_backward    replaces ops._C.rope_backward     (csrc/ops/rope.cpp:150-200, kernel rope_backward_cuda.cu:68-118):
+ *                       out[2i] = g[2i] cos[2i] + g[2i+1] sin[2i+1]; out[2i+1] = -g[2i] sin[2i] + g[2i+1] cos[2i+1]
+ *   q8_rmsnorm_backward replaces ops._C.rms_norm_backward (kernel rms_norm_backward_cuda.cu:101-206):
+ *                       out = rstd / dim * (dim * g * w - y / w * sum_j g_j y_j), y the forward output, w NULL = 1
+ * All element dtypes in {BF16, E4M3} independently (the reference ties grad's dtype to out's); n, dim % 8 == 0.
+ */
+int q8_gelu(const void* x, int x_dtype, void* out, int out_dtype, int64_t n, q8_stream_t stream);
+int q8_gelu_backward(const void* x, int x_dtype, const void* grad, int grad_dtype, void* out, int out_dtype,
+                     int64_t n, q8_stream_t stream);
+int q8_rope_backward(const void* grad, int grad_dtype, const float* cos_t, const float* sin_t, void* out,
+                     int out_dtype, int64_t rows, int dim, q8_stream_t stream);
+int q8_rmsnorm_backward(const void* y, int y_dtype, const float* rstd, const void* grad, int grad_dtype,
+                        const float* w, void* out, int out_dtype, int64_t rows, int dim, q8_stream_t stream);
+
+/*
  * Fused row kernels: launch sequences of the reference with the 16-bit tensor between two kernels kept in
  * registers. Each intermediate value is rounded to `mid_dtype` exactly where the unfused sequence stores it
  * (mid_dtype = Q8_BF16 gives the same bits as the separate calls; Q8_F32 skips that rounding).

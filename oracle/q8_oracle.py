@@ -11,7 +11,9 @@ float64 softmax, complex-number rotation ...).
 
 Pinning status (also listed in DESIGN.md):
   pinned by closed forms ....... e4m3 casts, ref_fht, ref_quant, ref_gemm_i32, ref_gemm_fp8_acc,
-                                 ref_epilogue, ref_rms_norm, ref_rope, ref_attention, ref_freqs_cis
+                                 ref_epilogue, ref_rms_norm, ref_rope, ref_attention, ref_freqs_cis,
+                                 ref_fma (exact rational arithmetic), ref_gelu_backward, ref_rms_norm_backward,
+                                 ref_rope_backward (float64 autograd of the forward formulas, adjoint identity)
   parity unpinned (bit level) .. the low-order bits the reference gets from nvcc --use_fast_math
                                  (approximate division in the quantizer, tanhf / exp2f / rsqrtf) and the
                                  accumulation order inside mma.sync; unobservable without an sm_89 GPU.
@@ -362,6 +364,67 @@ def ref_freqs_cis(indices_grid: torch.Tensor, dim: int = 2048, theta: float = 10
     return cos.to(torch.float32), sin.to(torch.float32)
 
 
+# ------------------------------------------------------------------------------------------- fma, GELU, backward ops
+
+
+def ref_fma(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, scale_add: float = 0.0,
+            out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out = x * (y + scale_add) + z with y, z [B, T or 1, dim] broadcast over tokens, csrc/ops/fma_cuda.cu:94 and
+    csrc/ops/fma.cpp:85-86; output in x's dtype (fma.cpp:99). y + scale_add rounds to fp32; the product and the
+    sum round once (the expression contracts to a fused multiply-add), evaluated here in float64 where the
+    product of an 8- or 16-bit x with an fp32 factor is exact."""
+    out_type = x.dtype if out_type is None else out_type
+    ys = (y.to(torch.float32) + torch.tensor(scale_add, dtype=torch.float32)).to(torch.float64)
+    v = x.to(torch.float32).to(torch.float64) * ys + z.to(torch.float32).to(torch.float64)
+    return cast(v.to(torch.float32), out_type)
+
+
+def ref_gelu_forward(x: torch.Tensor, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """tanh-GELU, csrc/ops/gelu_forward_cuda.cu:12-16; out_type None -> input dtype. Evaluated in float64."""
+    out_type = x.dtype if out_type is None else out_type
+    return cast(gelu_tanh(x.to(torch.float32).to(torch.float64)).to(torch.float32), out_type)
+
+
+def ref_gelu_backward(x: torch.Tensor, grad_output: torch.Tensor, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """grad * (0.5 (1 + phi) + 0.5 x phi'), phi = tanh(tau), tau = k (x + c x^3),
+    phi' = (1 - phi^2) k (1 + 3 c x^2): csrc/ops/gelu_backward_cuda.cu:94-100. Evaluated in float64."""
+    out_type = x.dtype if out_type is None else out_type
+    k, c = 0.7978845608028654, 0.044715
+    xv = x.to(torch.float32).to(torch.float64)
+    g = grad_output.to(torch.float32).to(torch.float64)
+    phi = torch.tanh(k * (xv + c * xv ** 3))
+    dphi = (1.0 - phi * phi) * (k * (1.0 + 3.0 * c * xv * xv))
+    return cast((g * (0.5 * (1.0 + phi) + 0.5 * xv * dphi)).to(torch.float32), out_type)
+
+
+def ref_rope_backward(grad_out: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                      out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """The transpose of ref_rope's rotation, csrc/ops/rope_backward_cuda.cu:106-107:
+        o[2i] = g[2i] cos[2i] + g[2i+1] sin[2i+1];   o[2i+1] = -g[2i] sin[2i] + g[2i+1] cos[2i+1]."""
+    out_type = grad_out.dtype if out_type is None else out_type
+    g = grad_out.to(torch.float32)
+    g0, g1 = g[..., 0::2], g[..., 1::2]
+    c0, c1 = cos[..., 0::2], cos[..., 1::2]
+    s0, s1 = sin[..., 0::2], sin[..., 1::2]
+    o0 = g0 * c0 + g1 * s1
+    o1 = -g0 * s0 + g1 * c1
+    return cast(torch.stack((o0, o1), dim=-1).reshape(g.shape), out_type)
+
+
+def ref_rms_norm_backward(x_normed: torch.Tensor, x_norms: torch.Tensor, grad_out: torch.Tensor,
+                          weights: Optional[torch.Tensor] = None, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """dx = rstd / dim * (dim * g * w - y / w * sum_j g_j y_j) from the forward's outputs y = x_normed and
+    rstd = x_norms: csrc/ops/rms_norm_backward_cuda.cu:140-160. Evaluated in float64."""
+    out_type = x_normed.dtype if out_type is None else out_type
+    y = x_normed.to(torch.float32).to(torch.float64)
+    g = grad_out.to(torch.float32).to(torch.float64)
+    w = torch.ones(y.shape[-1], dtype=torch.float64) if weights is None else weights.to(torch.float64)
+    dim = y.shape[-1]
+    dot = (g * y).sum(dim=-1, keepdim=True)
+    r = x_norms.to(torch.float64).reshape(y.shape[:-1] + (1,))
+    return cast((r / dim * (dim * g * w - y / w * dot)).to(torch.float32), out_type)
+
+
 # ------------------------------------------------------------------------------------------- block composition
 
 
@@ -396,3 +459,52 @@ def ref_dit_block(hidden, text, freqs_cis, text_lens, params, num_heads, head_di
     hidden = hidden + lin("to_out2", merge(a))
     h, _ = ref_rms_norm(hidden, params["norm3"])
     return hidden + lin("ff_down", lin("ff_up", h, gelu=True))
+
+
+def ref_attention_module(p, prefix, x, num_heads, head_dim, freqs_cis=None, context=None, lens=None,
+                         non_mm=torch.bfloat16, mm_out=torch.bfloat16):
+    """q8_kernels/modules/attention.py:45-106 with attn_type 'q8_kernels': int8 projections, qk-RMSNorm over the
+    full inner dim, RoPE on self-attention, fp8 flash attention with Hadamard (e4m3 output), output projection.
+    p[prefix + name] = (int8 weight, fp32 scales, fp32 bias or None); p[prefix + 'q_norm' / 'k_norm'] = fp32 [inner]."""
+    b = x.shape[0]
+
+    def lin(name, t):
+        w, s, bias = p[prefix + name]
+        return ref_q8_linear(t, w, bias, None, s, False, mm_out)
+
+    def heads(t):
+        return t.reshape(b, -1, num_heads, head_dim).transpose(1, 2)
+
+    src = x if context is None else context
+    q, k, v = lin("to_q", x), lin("to_k", src), lin("to_v", src)
+    q, _ = ref_rms_norm(q, p[prefix + "q_norm"], non_mm)
+    k, _ = ref_rms_norm(k, p[prefix + "k_norm"], non_mm)
+    if context is None and freqs_cis is not None:
+        q, k = ref_rope(q, freqs_cis[0], freqs_cis[1], non_mm), ref_rope(k, freqs_cis[0], freqs_cis[1], non_mm)
+    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, lens, True)
+    a = a.transpose(1, 2).reshape(b, -1, num_heads * head_dim)
+    return lin("to_out", a).to(non_mm)
+
+
+def ref_ltx_block(p, hidden, freqs_cis, context, context_lens, timestep, num_heads, head_dim):
+    """q8_kernels/blocks/ltx_transformer_block.py:21-58 with bfloat16 activations; the modulations and gated
+    residuals are evaluated as fused multiply-adds (ref_fma). p['scale_shift_table'] fp32 [6, dim],
+    p['norm1'] / p['norm2'] = fp32 [dim] or None, attention parameters under 'attn1.' / 'attn2.',
+    feed-forward under 'ff.up' / 'ff.down'."""
+    bf16 = torch.bfloat16
+    b = hidden.shape[0]
+    ada = p["scale_shift_table"][None, None] + timestep.reshape(b, timestep.shape[1], 6, -1)
+    shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (t.to(bf16) for t in ada.unbind(dim=2))
+    h, _ = ref_rms_norm(hidden, p["norm1"], bf16)
+    h = ref_fma(h, scale_msa, shift_msa, 1.0)
+    a = ref_attention_module(p, "attn1.", h, num_heads, head_dim, freqs_cis)
+    hidden = ref_fma(a, gate_msa, hidden, 0.0)
+    a = ref_attention_module(p, "attn2.", hidden, num_heads, head_dim, None, context, context_lens)
+    hidden = a + hidden
+    h, _ = ref_rms_norm(hidden, p["norm2"], bf16)
+    h = ref_fma(h, scale_mlp, shift_mlp, 1.0)
+    w, s, bias = p["ff.up"]
+    up = ref_q8_linear(h, w, bias, None, s, True, bf16)
+    w, s, bias = p["ff.down"]
+    ff = ref_q8_linear(up, w, bias, None, s, False, bf16).to(bf16)
+    return ref_fma(ff.reshape(hidden.shape), gate_mlp, hidden, 0.0)

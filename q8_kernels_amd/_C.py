@@ -391,3 +391,113 @@ def attn_prep_v(x: torch.Tensor, num_heads: int, per_token_scales: bool = False)
         _lib.check(_lib.lib().q8_attn_prep_v(x.data_ptr(), x.stride(1), codes.data_ptr(), _ptr(scales), b, s,
                                              num_heads, d, s_pad, _stream(x)))
     return (codes, scales) if per_token_scales else codes
+
+
+# ----------------------------------------------------------------------------- ops._C: fma and the backward operators
+
+_EW = (torch.bfloat16, torch.float8_e4m3fn)
+
+
+def _rows2d(t, name):
+    _require_gpu(t, name)
+    t2 = t.reshape(-1, t.shape[-1])
+    return t2 if t2.is_contiguous() else t2.contiguous()
+
+
+def fma_8bit(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, scale_add: float = 0.0, *,
+             out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/fma.cpp:63-112: x * (y + scale_add) + z for x [B, T, dim] e4m3, y and z [B, T or 1, dim]
+    (fp32/fp32, fp32/e4m3 or bf16/bf16 in the reference; any mix of the three here). Returns x's shape in x's
+    dtype; bfloat16 x and `out_type` are extensions."""
+    if x.dtype not in _EW:
+        raise RuntimeError("fma_8bit: x must be float8_e4m3fn (or bfloat16)")
+    if x.dim() != 3:
+        raise RuntimeError("fma_8bit: x must be 3-D")
+    for t, name in ((y, "y"), (z, "z")):
+        if t.dtype not in (torch.float32, torch.bfloat16, torch.float8_e4m3fn):
+            raise RuntimeError("fma not implemented for input type '%s'" % t.dtype)
+        if t.shape[-1] != x.shape[-1]:
+            raise RuntimeError("fma: channels missmatch")
+        if t.dim() != 3 or t.shape[0] != x.shape[0] or t.shape[-2] not in (1, x.shape[-2]):
+            raise RuntimeError("fma: token missmatch")
+    out_type = x.dtype if out_type is None else out_type
+    if out_type not in _EW:
+        raise RuntimeError("fma_8bit: output must be bfloat16 or float8_e4m3fn")
+    shape = x.shape
+    x2, y2, z2 = _rows2d(x, "x"), _rows2d(y, "y"), _rows2d(z, "z")
+    rows, dim = x2.shape
+    out = torch.empty((rows, dim), dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_fma(x2.data_ptr(), _DT[x2.dtype], y2.data_ptr(), _DT[y2.dtype], z2.data_ptr(),
+                                     _DT[z2.dtype], out.data_ptr(), _DT[out_type], rows, dim,
+                                     shape[-2] // y.shape[-2], shape[-2] // z.shape[-2], float(scale_add), _stream(x)))
+    return out.reshape(shape)
+
+
+def _ew_out(x, out_type, who):
+    out_type = x.dtype if out_type is None else out_type
+    if x.dtype not in _EW or out_type not in _EW:
+        raise RuntimeError("%s: input and output must be bfloat16 or float8_e4m3fn" % who)
+    if x.shape[-1] % 8 != 0:
+        raise RuntimeError("%s: last dim must be a multiple of 8" % who)
+    return out_type
+
+
+def gelu_forward(x: torch.Tensor, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/gelu_act.cpp (gelu_forward): tanh-GELU, out_type None -> x.dtype."""
+    out_type = _ew_out(x, out_type, "gelu_forward")
+    x2 = _rows2d(x, "x")
+    out = torch.empty(x2.shape, dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_gelu(x2.data_ptr(), _DT[x2.dtype], out.data_ptr(), _DT[out_type], x2.numel(), _stream(x)))
+    return out.reshape(x.shape)
+
+
+def gelu_backward(x: torch.Tensor, grad_output: torch.Tensor, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/gelu_act.cpp (gelu_backward): grad_output * dGELU/dx at x, out_type None -> x.dtype."""
+    out_type = _ew_out(x, out_type, "gelu_backward")
+    if grad_output.shape != x.shape or grad_output.dtype not in _EW:
+        raise RuntimeError("gelu_backward: grad_output must have x's shape and be bfloat16 or float8_e4m3fn")
+    x2, g2 = _rows2d(x, "x"), _rows2d(grad_output, "grad_output")
+    out = torch.empty(x2.shape, dtype=out_type, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_gelu_backward(x2.data_ptr(), _DT[x2.dtype], g2.data_ptr(), _DT[g2.dtype], out.data_ptr(),
+                                               _DT[out_type], x2.numel(), _stream(x)))
+    return out.reshape(x.shape)
+
+
+def rope_backward(grad_out: torch.Tensor, cos_freqs: torch.Tensor, sin_freqs: torch.Tensor,
+                  out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/rope.cpp:150-200: the transposed rotation applied to grad_out."""
+    if cos_freqs.dtype != torch.float32 or sin_freqs.dtype != torch.float32:
+        raise RuntimeError("rope_backward: cos/sin tables must be float32")
+    if cos_freqs.shape != grad_out.shape or sin_freqs.shape != grad_out.shape:
+        raise RuntimeError("rope_backward: cos/sin tables must have the shape of grad_out")
+    out_type = _ew_out(grad_out, out_type, "rope_backward")
+    g2, c2, s2 = _rows2d(grad_out, "grad_out"), _rows2d(cos_freqs, "cos_freqs"), _rows2d(sin_freqs, "sin_freqs")
+    out = torch.empty(g2.shape, dtype=out_type, device=grad_out.device)
+    with torch.cuda.device(grad_out.device):
+        _lib.check(_lib.lib().q8_rope_backward(g2.data_ptr(), _DT[g2.dtype], c2.data_ptr(), s2.data_ptr(), out.data_ptr(),
+                                               _DT[out_type], g2.shape[0], g2.shape[1], _stream(grad_out)))
+    return out.reshape(grad_out.shape)
+
+
+def rms_norm_backward(x_normed: torch.Tensor, x_norms: torch.Tensor, grad_out: torch.Tensor,
+                      weights: Optional[torch.Tensor] = None, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+    """csrc/ops/rms_norm.cpp (rms_norm_backward): dx from the forward's outputs (x_normed, x_norms = rstd per row)."""
+    out_type = _ew_out(x_normed, out_type, "rms_norm_backward")
+    if grad_out.shape != x_normed.shape or grad_out.dtype not in _EW:
+        raise RuntimeError("rms_norm_backward: grad_out must have x_normed's shape and be bfloat16 or float8_e4m3fn")
+    y2, g2 = _rows2d(x_normed, "x_normed"), _rows2d(grad_out, "grad_out")
+    rows, dim = y2.shape
+    _require_gpu(x_norms, "x_norms")
+    if x_norms.dtype != torch.float32 or x_norms.numel() != rows:
+        raise RuntimeError("rms_norm_backward: x_norms must be float32 with one value per row")
+    if weights is not None and (weights.dtype != torch.float32 or not weights.is_cuda or weights.numel() != dim):
+        raise RuntimeError("rms_norm_backward: weights error")
+    out = torch.empty((rows, dim), dtype=out_type, device=x_normed.device)
+    with torch.cuda.device(x_normed.device):
+        _lib.check(_lib.lib().q8_rmsnorm_backward(y2.data_ptr(), _DT[y2.dtype], x_norms.contiguous().data_ptr(), g2.data_ptr(),
+                                                  _DT[g2.dtype], _ptr(None if weights is None else weights.contiguous()),
+                                                  out.data_ptr(), _DT[out_type], rows, dim, _stream(x_normed)))
+    return out.reshape(x_normed.shape)

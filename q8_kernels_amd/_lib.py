@@ -27,6 +27,11 @@ SIGNATURES = {
     "q8_fht": (_i, [_vp, _i, _vp, _i, _i64, _i, _f, _vp]),
     "q8_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i64, _i, _f, _vp]),
     "q8_rope": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i64, _i, _vp]),
+    "q8_fma": (_i, [_vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i, _i64, _i64, _f, _vp]),
+    "q8_gelu": (_i, [_vp, _i, _vp, _i, _i64, _vp]),
+    "q8_gelu_backward": (_i, [_vp, _i, _vp, _i, _vp, _i, _i64, _vp]),
+    "q8_rope_backward": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i64, _i, _vp]),
+    "q8_rmsnorm_backward": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i, _vp]),
     "q8_fht_quant_rows": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _f, _i, _i, _vp]),
     "q8_rmsnorm_quant_rows": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i64, _i, _f, _i, _i, _vp]),
     "q8_attn_prep_qk": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp]),

@@ -1,0 +1,56 @@
+"""The AdaLN-modulated LTX-Video transformer block (reference: q8_kernels/blocks/ltx_transformer_block.py:9-58):
+RMSNorm -> scale/shift -> self-attention (qk-RMSNorm, RoPE) -> gated residual -> cross-attention -> residual ->
+RMSNorm -> scale/shift -> feed-forward -> gated residual, on int8 (Q8Linear) projections.
+
+The modulations `norm(x) * (1 + scale) + shift` and the gated residuals `gate * y + x` run as one fused
+multiply-add kernel each (multiply_add, fp32 arithmetic, one rounding to bfloat16); the reference evaluates
+them with torch element-wise kernels that round to bfloat16 after every operation."""
+import torch
+import torch.nn as nn
+
+from .. import functional as Q8F
+from ..modules.attention import Attention
+from ..modules.ffn import FeedForward
+from ..modules.rms_norm import RMSNorm
+
+
+class LTXTransformerBlock(nn.Module):
+    def __init__(self, dim, num_heads, head_dim, kv_dim, bias=True, use_rope=True, norm_affine=False):
+        super().__init__()
+        self.norm1 = RMSNorm(dim, norm_affine)
+        self.attn1 = Attention(dim, num_heads, head_dim, bias, bias, qk_rms_norm=True, kv_dim=None, use_rope=use_rope)
+        self.attn2 = Attention(dim, num_heads, head_dim, bias, bias, qk_rms_norm=True, kv_dim=kv_dim, use_rope=False)
+        self.norm2 = RMSNorm(dim, norm_affine)
+        self.ff = FeedForward(dim, bias=bias)
+        self.scale_shift_table = nn.Parameter(torch.randn(6, dim) / dim ** 0.5)
+
+    @staticmethod
+    def _fma(x, y, z, add):
+        """x * (y + add) + z with y, z [B, 1 or T, dim]: one kernel for bfloat16 activations on the GPU."""
+        if (x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 3 and x.shape[-1] % 8 == 0
+                and not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad or z.requires_grad))):
+            bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
+            return Q8F.fma.multiply_add(x.contiguous(), bf(y), bf(z), add)
+        return x * (y + add) + z
+
+    def forward(self, hidden_states, freqs_cis, attention_mask, encoder_hidden_states, encoder_attention_mask,
+                timestep, mm_out_dtype=torch.bfloat16, non_mm_precision=torch.bfloat16, attn_type="torch"):
+        num_ada_params = self.scale_shift_table.shape[0]
+        ada_values = self.scale_shift_table[None, None] + timestep.reshape(
+            hidden_states.shape[0], timestep.shape[1], num_ada_params, -1)
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada_values.unbind(dim=2)
+
+        norm_hidden_states = self._fma(self.norm1(hidden_states, non_mm_precision), scale_msa, shift_msa, 1.0)
+        attn_output = self.attn1(norm_hidden_states, freqs_cis, None, attention_mask, non_mm_precision, mm_out_dtype,
+                                 attn_type=attn_type)
+        hidden_states = self._fma(attn_output, gate_msa, hidden_states, 0.0)
+
+        attn_output = self.attn2(hidden_states, freqs_cis=freqs_cis, encoder_hidden_states=encoder_hidden_states,
+                                 attention_mask=encoder_attention_mask, non_mm_precision=non_mm_precision,
+                                 mm_out_dtype=mm_out_dtype, attn_type=attn_type)
+        hidden_states = attn_output + hidden_states
+
+        norm_hidden_states = self._fma(self.norm2(hidden_states, non_mm_precision), scale_mlp, shift_mlp, 1.0)
+        ff_output = self.ff(norm_hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
+        hidden_states = self._fma(ff_output, gate_mlp, hidden_states, 0.0)
+        return hidden_states

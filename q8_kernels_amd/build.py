@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libq8_hip.so")
-SOURCES = ["api.hip", "rows.hip", "fused.hip", "gemm.hip", "attn.hip"]
+SOURCES = ["api.hip", "rows.hip", "fused.hip", "elementwise.hip", "gemm.hip", "attn.hip"]
 # packed fp32 VALU forms are disabled on purpose (they have miscomputed on this hardware pool)
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -1,1 +1,1 @@
-from . import fast_hadamard, flash_attention, fused, linear, quantizer, rms_norm, rope  # noqa: F401
+from . import fast_hadamard, flash_attention, fma, fused, linear, quantizer, rms_norm, rope  # noqa: F401

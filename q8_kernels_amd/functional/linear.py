@@ -1,7 +1,9 @@
-"""int8 / fp8 linear layers on the 8-bit GEMM (reference: q8_kernels/functional/linear.py:24-42,138-196).
+"""int8 / fp8 linear layers on the 8-bit GEMM (reference: q8_kernels/functional/linear.py:22-196).
 
-Forward (inference) only. Operands that arrive in 16-bit (or fp8 for the int8 path) are quantized on
-the fly: int8 path = FHT rotation then per-row int8; fp8 path = optional FHT then per-row e4m3.
+Operands that arrive in 16-bit (or fp8 for the int8 path) are quantized on the fly: int8 path = FHT rotation
+then per-row int8; fp8 path = optional FHT then per-row e4m3. The backward functions return the gradient of
+the activation only (the 8-bit weights are frozen), computed like the reference's with an fp8 GEMM on the
+re-quantized, dequantized weight; the LoRA variant also returns the gradients of the two adapter matrices.
 """
 from typing import Optional
 
@@ -20,10 +22,20 @@ def is_16bit(x) -> bool:
     return dtype in (torch.float16, torch.bfloat16)
 
 
-def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
-              scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
-              fuse_gelu: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """a [..., K] x b [N, K] -> [batch, M, N] through the int8 GEMM; out_dtype None -> e4m3 (as the reference)."""
+def _rotate_quant(t, out_type=None):
+    """quantize(hadamard_transform(t)); one kernel where that gives the bits of the two."""
+    if can_fuse_hadamard_quantize(t):
+        return hadamard_quantize(t, out_type)
+    return (quantize if out_type is None else quantize_fp8)(hadamard_transform(t))
+
+
+def _needs_grad(t) -> bool:
+    return torch.is_grad_enabled() and isinstance(t, torch.Tensor) and t.requires_grad
+
+
+# ----------------------------------------------------------------------------- int8
+
+def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype):
     a_needs_q = a.dtype == _FP8 or is_16bit(a)
     b_needs_q = b.dtype == _FP8 or is_16bit(b)
     assert (a_needs_q and scale_a is None) or (a.dtype == torch.int8 and scale_a is not None), \
@@ -32,25 +44,55 @@ def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = N
         "Q8LinearFunc: b dtype missmatch"
     assert a.shape[-1] == b.shape[-1], "Q8LinearFunc: mnk missmatch"
     assert bias is None or bias.dtype == torch.float, "Q8LinearFunc: bias must be in fp32"
-    def rotate_quant(t):  # one kernel where it gives the bits of the two
-        return hadamard_quantize(t) if can_fuse_hadamard_quantize(t) else quantize(hadamard_transform(t))
-
     if a_needs_q:
-        a, scale_a = rotate_quant(a)
+        a, scale_a = _rotate_quant(a)
     if b_needs_q:
-        b, scale_b = rotate_quant(b)
+        b, scale_b = _rotate_quant(b)
     if bias is not None:
-        return _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
-    return _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+    else:
+        out = _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+    return out, b, scale_b
 
 
-def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
-               use_hadamard: bool = False, out_dtype: Optional[torch.dtype] = None, *,
-               fuse_gelu: bool = False) -> torch.Tensor:
-    """a [..., K] x b [N, K] -> [batch, M, N] through the fp8 GEMM; out_dtype must be 16-bit.
+def _grad_through_weight(grad_output, w, out_dtype):
+    """grad_output [.., N] @ w [N, K] on the fp8 GEMM: both operands re-quantized per row to e4m3
+    (q8_kernels/functional/linear.py:49-52)."""
+    g8, gs = quantize_fp8(grad_output)
+    w8, ws = quantize_fp8(w.T.contiguous())
+    return _C.fp8_mm(g8, w8, gs, ws, False, out_dtype)
 
-    `fuse_gelu` (keyword only, default False = the reference's behaviour) applies tanh-GELU in the epilogue."""
+
+class Q8LinearFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype):
+        out, bq, sb = _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+        ctx.save_for_backward(bq, sb)
+        ctx.out_dtype = out_dtype
+        ctx.a_shape = a.shape
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        # y = (a H) W'^T with W' the rotated, dequantized weight, so da = (dy W') H (H is symmetric)
+        b, scale_b = ctx.saved_tensors
+        w = b.to(ctx.out_dtype) * scale_b[:, None].to(ctx.out_dtype)
+        grad_x = hadamard_transform(_grad_through_weight(grad_output, w, ctx.out_dtype))
+        return grad_x.reshape(ctx.a_shape), None, None, None, None, None, None
+
+
+def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
+              fuse_gelu: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """a [..., K] x b [N, K] -> [batch, M, N] through the int8 GEMM; out_dtype None -> e4m3 (as the reference)."""
+    if _needs_grad(a):
+        return Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+    return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)[0]
+
+
+# ----------------------------------------------------------------------------- fp8
+
+def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu):
     assert (is_16bit(a) and scale_a is None) or (a.dtype == _FP8 and scale_a is not None), \
         "FP8LinearFunc: a dtype missmatch"
     assert (is_16bit(b) and scale_b is None) or (b.dtype == _FP8 and scale_b is not None), \
@@ -60,16 +102,109 @@ def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = 
     assert out_dtype is not None and is_16bit(out_dtype), "FP8LinearFunc: out_dtype must be in 16bit"
 
     def quant(t):
-        if use_hadamard:
-            if can_fuse_hadamard_quantize(t):
-                return hadamard_quantize(t, _FP8)
-            return quantize_fp8(hadamard_transform(t))
-        return quantize_fp8(t)
+        return _rotate_quant(t, _FP8) if use_hadamard else quantize_fp8(t)
 
     if is_16bit(a):
         a, scale_a = quant(a)
     if is_16bit(b):
         b, scale_b = quant(b)
     if bias is not None:
-        return _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
-    return _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+    else:
+        out = _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+    return out, b, scale_b
+
+
+class FP8LinearFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, bias, scale_a, scale_b, out_dtype, use_hadamard):
+        out, bq, sb = _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, False)
+        ctx.save_for_backward(bq, sb)
+        ctx.out_dtype = out_dtype
+        ctx.use_hadamard = use_hadamard
+        ctx.a_shape = a.shape
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        b, scale_b = ctx.saved_tensors
+        w = b.to(ctx.out_dtype) * scale_b[:, None].to(ctx.out_dtype)
+        grad_x = _grad_through_weight(grad_output, w, ctx.out_dtype)
+        if ctx.use_hadamard:  # the forward rotated a: rotate the gradient back
+            grad_x = hadamard_transform(grad_x)
+        return grad_x.reshape(ctx.a_shape), None, None, None, None, None, None
+
+
+def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
+               use_hadamard: bool = False, out_dtype: Optional[torch.dtype] = None, *,
+               fuse_gelu: bool = False) -> torch.Tensor:
+    """a [..., K] x b [N, K] -> [batch, M, N] through the fp8 GEMM; out_dtype must be 16-bit.
+
+    `fuse_gelu` (keyword only, default False = the reference's behaviour) applies tanh-GELU in the epilogue."""
+    if _needs_grad(a) and not fuse_gelu:
+        return FP8LinearFunc.apply(a, b, bias, scale_a, scale_b, out_dtype, use_hadamard)
+    return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu)[0]
+
+
+# ----------------------------------------------------------------------------- int8 base weight + 16-bit LoRA
+
+class Q8LinearLora(torch.autograd.Function):
+    """o = q8_mm(quant(H a), W') (+ bias) + (a lora_a^T) lora_b^T, optionally followed by tanh-GELU
+    (q8_kernels/functional/linear.py:56-133). a must be 16-bit here (the adapter branch reads it)."""
+
+    @staticmethod
+    def forward(ctx, a, b, bias, scale_a, scale_b, lora_a, lora_b, fuse_gelu, use_hadamard, out_dtype):
+        assert is_16bit(a) and scale_a is None, "Q8LinearFuncLora: a must be 16bit"
+        assert ((b.dtype == _FP8 or is_16bit(b)) and scale_b is None) or (b.dtype == torch.int8 and scale_b is not None), \
+            "Q8LinearFuncLora: b dtype missmatch"
+        assert a.shape[-1] == b.shape[-1], "Q8LinearFuncLora: mnk missmatch"
+        assert bias is None or bias.dtype == torch.float, "Q8LinearFuncLora: bias must be in fp32"
+        assert lora_a is not None and lora_b is not None, "Q8LinearFuncLora: lora_a and lora_b must be provided"
+        assert is_16bit(lora_a) and is_16bit(lora_b), "Q8LinearFuncLora: lora_a and lora_b must be in 16bit"
+        assert lora_a.shape[0] == lora_b.shape[-1], "Q8LinearFuncLora: lora_a and lora_b shape missmatch"
+        assert out_dtype is not None and is_16bit(out_dtype), "Q8LinearFuncLora: out_dtype must be float16 or bfloat16"
+        a_q, sa = _rotate_quant(a) if use_hadamard else quantize(a)
+        if b.dtype != torch.int8:
+            b, scale_b = _rotate_quant(b) if use_hadamard else quantize(b)
+        if bias is not None:
+            base = _C.q8_mm_bias(a_q, b, bias, sa, scale_b, False, out_dtype)
+        else:
+            base = _C.q8_mm(a_q, b, sa, scale_b, False, out_dtype)
+        lora_y = torch.nn.functional.linear(torch.nn.functional.linear(a, lora_a), lora_b)
+        o = base + lora_y.reshape(base.shape).to(out_dtype)
+        ctx.fuse_gelu, ctx.out_dtype, ctx.use_hadamard = fuse_gelu, out_dtype, use_hadamard
+        ctx.a_shape = a.shape
+        if fuse_gelu:
+            ctx.save_for_backward(o, a, b, scale_b, lora_a, lora_b)
+            return _C.gelu_forward(o, out_dtype)
+        ctx.save_for_backward(None, a, b, scale_b, lora_a, lora_b)
+        return o
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        o, a, b, scale_b, lora_a, lora_b = ctx.saved_tensors
+        out_dtype = ctx.out_dtype
+        if ctx.fuse_gelu:
+            grad_output = _C.gelu_backward(o, grad_output.to(out_dtype).contiguous(), out_dtype)
+        grad_output = grad_output.reshape(a.shape[:-1] + (grad_output.shape[-1],))
+        g_lb = grad_output @ lora_b  # [.., d] @ [d, r]
+        w = b.to(out_dtype) * scale_b[:, None].to(out_dtype)
+        grad_x = _grad_through_weight(grad_output, w, out_dtype).reshape(ctx.a_shape)
+        if ctx.use_hadamard:
+            grad_x = hadamard_transform(grad_x)
+        grad_x = grad_x + g_lb @ lora_a
+        a2 = a.reshape(-1, a.shape[-1])
+        g2 = grad_output.reshape(-1, grad_output.shape[-1])
+        glb2 = g_lb.reshape(-1, g_lb.shape[-1])
+        grad_lora_a = glb2.T @ a2                  # [r, h]
+        grad_lora_b = g2.T @ (a2 @ lora_a.T)       # [d, r]
+        return grad_x, None, None, None, None, grad_lora_a, grad_lora_b, None, None, None
+
+
+def q8_linear_lora(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                   scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
+                   lora_a: Optional[torch.Tensor] = None, lora_b: Optional[torch.Tensor] = None,
+                   fuse_gelu: bool = False, use_hadamard: bool = True,
+                   out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    return Q8LinearLora.apply(a, b, bias, scale_a, scale_b, lora_a, lora_b, fuse_gelu, use_hadamard, out_dtype)

@@ -357,3 +357,80 @@ def test_freqs_cis_against_loops():
                 assert abs(cos[0, t, col].item() - math.cos(a)) < 1e-5
                 assert cos[0, t, col] == cos[0, t, col + 1]
                 assert abs(sin[0, t, col].item() - math.sin(a)) < 1e-5
+
+
+# ------------------------------------------------------------------ fma, GELU, backward operators
+
+def test_fma_against_exact_rational_arithmetic():
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(31)
+    x = O.e4m3_c10(torch.randn(2, 3, 8, generator=g) * 3)
+    y = torch.randn(2, 1, 8, generator=g)
+    z = O.e4m3_c10(torch.randn(2, 3, 8, generator=g))
+    got = O.ref_fma(x, y, z, 1.0).view(torch.uint8)
+    table = O.e4m3_decode_table()
+    finite = [(float(table[c]), c) for c in range(256) if np.isfinite(table[c])]
+    for b in range(2):
+        for t in range(3):
+            for i in range(8):
+                ys = float((y[b, 0, i] + torch.tensor(1.0)).item())  # the fp32 sum y + scale_add
+                exact = Fraction(float(x[b, t, i])) * Fraction(ys) + Fraction(float(z[b, t, i]))
+                # nearest e4m3 value of the exact result (no tie and far from the fp32 rounding step in these data)
+                best = min(finite, key=lambda vc: abs(Fraction(vc[0]) - exact))
+                assert table[int(got[b, t, i])] == best[0], (b, t, i)
+
+
+def test_fma_broadcast_and_dtypes():
+    g = torch.Generator().manual_seed(32)
+    x = (torch.randn(2, 5, 16, generator=g)).to(torch.bfloat16)
+    y = torch.randn(2, 1, 16, generator=g).to(torch.bfloat16)
+    z = torch.randn(2, 5, 16, generator=g).to(torch.bfloat16)
+    want = (x.double() * (y.float() + 1.0).double() + z.double()).float().to(torch.bfloat16)
+    assert torch.equal(O.ref_fma(x, y, z, 1.0), want)
+
+
+def test_gelu_backward_is_the_derivative_of_gelu_forward():
+    g = torch.Generator().manual_seed(33)
+    x = (torch.randn(4, 64, generator=g) * 2).to(torch.bfloat16)
+    go = torch.randn(4, 64, generator=g).to(torch.bfloat16)
+    xd = x.double().requires_grad_(True)
+    torch.nn.functional.gelu(xd, approximate="tanh").backward(go.double())
+    got = O.ref_gelu_backward(x, go, torch.bfloat16)
+    assert torch.equal(got, xd.grad.float().to(torch.bfloat16))
+    fwd = O.ref_gelu_forward(x, torch.bfloat16)
+    assert torch.equal(fwd, torch.nn.functional.gelu(x.double(), approximate="tanh").float().to(torch.bfloat16))
+
+
+def test_rope_backward_is_the_adjoint_of_rope():
+    g = torch.Generator().manual_seed(34)
+    x = torch.randn(3, 32, generator=g)
+    go = torch.randn(3, 32, generator=g)
+    cos, sin = torch.randn(3, 32, generator=g), torch.randn(3, 32, generator=g)  # unequal within pairs on purpose
+    # <rope(x), g> == <x, rope_backward(g)> for every x, g
+    lhs = (O.ref_rope(x.to(torch.bfloat16), cos, sin, torch.float32).double() * go.to(torch.bfloat16).double()).sum()
+    rhs = (x.to(torch.bfloat16).double() * O.ref_rope_backward(go.to(torch.bfloat16), cos, sin, torch.float32).double()).sum()
+    assert abs(float(lhs - rhs)) < 1e-4 * max(1.0, abs(float(lhs)))
+    # and against float64 autograd of the forward formula
+    gb = go.to(torch.bfloat16)
+    xd = x.double().requires_grad_(True)
+    y0 = xd[:, 0::2] * cos[:, 0::2].double() - xd[:, 1::2] * sin[:, 0::2].double()
+    y1 = xd[:, 1::2] * cos[:, 1::2].double() + xd[:, 0::2] * sin[:, 1::2].double()
+    torch.stack((y0, y1), -1).reshape(3, 32).backward(gb.double())
+    got = O.ref_rope_backward(gb, cos, sin, torch.float32)
+    assert torch.allclose(got.double(), xd.grad, rtol=1e-6, atol=1e-6)
+
+
+def test_rms_norm_backward_against_autograd():
+    g = torch.Generator().manual_seed(35)
+    for with_w in (False, True):
+        x = torch.randn(5, 48, generator=g, dtype=torch.float64)
+        w = (1 + 0.2 * torch.randn(48, generator=g)).float() if with_w else None
+        go = torch.randn(5, 48, generator=g, dtype=torch.float64)
+        xd = x.clone().requires_grad_(True)
+        rstd = 1.0 / torch.sqrt((xd ** 2).mean(-1, keepdim=True))
+        y = xd * rstd * (w.double() if with_w else 1.0)
+        y.backward(go)
+        # feed the formula with exact (float64 -> fp32) forward outputs; fp32 operands are not a kernel type, so
+        # the oracle is called with out_type float32 on bf16-free data through its float path
+        got = O.ref_rms_norm_backward(y.detach().float(), rstd.detach().float().squeeze(-1), go.float(), w, torch.float32)
+        assert torch.allclose(got.double(), xd.grad, rtol=2e-5, atol=2e-6)
