@@ -5,8 +5,9 @@
 //   * K advances 128 bytes per stage. A stage is A 256 rows x 128 B + B 256 rows x 128 B = 64 KiB, two stages
 //     in LDS, filled by global_load_lds_dwordx4 with 8 lanes per row: every request to L2 is a full 128-byte
 //     line (measured 61 B/clk/CU against 28 B/clk/CU for 64-byte rows and 40 B/clk/CU through VGPRs).
-//   * One s_barrier per stage. The loads of stage k+1 are issued right after the barrier of stage k, into
-//     the buffer whose reads all waves have completed, and have a whole stage of MFMA time to land.
+//   * Two s_barriers per stage: one as soon as every wave holds the last fragments of stage k in registers
+//     (buffer k & 1 is free: the copies of stage k+2 start), one after the copies of stage k+1 have landed
+//     (before its first fragments are fetched). A copy has 1 to 1.5 stages of MFMA time to land.
 //   * Operand fragments are double-buffered in registers over the two 64-byte K halves of a stage: the
 //     ds_read_b128 of the next half are always issued before the MFMAs of the current half. LDS reads and
 //     the counters are inline assembly so that exactly the waits written below are executed.
@@ -24,7 +25,8 @@
 namespace q8 {
 
 constexpr int kPipeBM = 256, kPipeBN = 256, kPipeStages = 2, kPipeStageBytes = 65536;
-constexpr int kPipeLds = kPipeStages * kPipeStageBytes;
+constexpr int kPipeParamOffset = kPipeStages * kPipeStageBytes;  // sa[256], sb[256], bias[256] of the tile (fp32)
+constexpr int kPipeLds = kPipeParamOffset + 3 * 256 * 4;
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct PipeFrags {
@@ -172,6 +174,28 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][t][e] = 0;
 
+    // ---- per-row and per-column dequantization parameters of the tile: copied to LDS now (4 bytes per lane, rows
+    //      and columns past the edge clamped to the last valid one), read back in the epilogue. They are the oldest
+    //      outstanding copies, so every later vmcnt wait covers them.
+    float* const lds_par = reinterpret_cast<float*>(lds + kPipeParamOffset);
+    if constexpr (OUT != Q8_OUT_I32) {
+        const int j = (wave & 3) * 64 + lane;
+        if (wave < 4) {
+            const int m = (m0 + j < M) ? m0 + j : M - 1;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.sa + (size_t)za * M + m),
+                                             (__attribute__((address_space(3))) void*)(lds_par + (wave & 3) * 64), 4, 0, 0);
+        } else {
+            const int n = (n0 + j < N) ? n0 + j : N - 1;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.sb + (size_t)zb * N + n),
+                                             (__attribute__((address_space(3))) void*)(lds_par + 256 + (wave & 3) * 64), 4, 0, 0);
+        }
+        if (p.bias != nullptr && wave < 4) {
+            const int n = (n0 + j < N) ? n0 + j : N - 1;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.bias + n),
+                                             (__attribute__((address_space(3))) void*)(lds_par + 512 + (wave & 3) * 64), 4, 0, 0);
+        }
+    }
+
     // ---- prologue: stage 0 landed, stage 1 in flight, fragments of the first K half on their way
     PipeFrags f0, f1;
     issue_loads(0);
@@ -187,21 +211,45 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     read_half(f0, 0, 0);
 
     for (int k = 0; k < KT; ++k) {
-        // f0: first K half of stage k (reads in flight); loads of stage k+1 in flight
+        // f0: first K half of stage k (reads in flight); the copies of stage k+1 are in flight
         pipe_wait_frags(f0);
         read_half(f1, k, 1);
         pipe_pin(f0);
-        if constexpr (!(DBG & 4)) pipe_mfma<IN>(f0, acc, [](int) {});
-        __builtin_amdgcn_sched_barrier(0);  // all MFMAs of the first half are issued before the wave waits and syncs
-        // the second half of stage k is in registers and stage k+1 has landed: nobody reads buffer k & 1 any more
-        if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        pipe_wait_frags(f1);
-        if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
-        read_half(f0, k + 1, 0);
+        // First half. Once the second half of stage k is in registers everywhere (barrier 1, after the 4th MFMA
+        // tile), buffer k & 1 is free and the copies of stage k+2 start to trickle out, one per MFMA tile.
+        if constexpr (!(DBG & 4)) {
+            pipe_mfma<IN>(f0, acc, [&](int j) {
+                if (j == 3) {
+                    pipe_wait_frags(f1);
+                    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+                }
+                if (j >= 4) issue_load(k + 2, j - 4);
+            });
+        } else {
+            pipe_wait_frags(f1);
+            if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+            issue_loads(k + 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         pipe_pin(f1);
-        // the copies of stage k+2 (into the buffer just released) trickle out between the MFMAs of the second half
-        if constexpr (DBG & 4) issue_loads(k + 2);
-        else pipe_mfma<IN>(f1, acc, [&](int j) { issue_load(k + 2, j); });
+        // Second half. After the last copy of stage k+2 is out, everything older (stage k+1) must have landed
+        // (vmcnt counts in order); barrier 2 makes that true for every wave's copies, and the first half of
+        // stage k+1 is fetched under the remaining MFMA tiles. A copy has between 1 and 1.5 stages of MFMA
+        // time to land.
+        if constexpr (!(DBG & 4)) {
+            pipe_mfma<IN>(f1, acc, [&](int j) {
+                if (j < 4) issue_load(k + 2, 4 + j);
+                if (j == 4) {
+                    if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+                    read_half(f0, k + 1, 0);
+                }
+            });
+        } else {
+            if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+            read_half(f0, k + 1, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     // drain: the look-ahead loads and fragment reads past the last stage target LDS / registers that nobody uses
@@ -226,12 +274,22 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
             const int n = nw0 + 32 * t + 16 * wp + 8 * h;
             if (n >= N) continue;
             float sbv[8], bv[8];
-            load_col_params<OUT>(p, zb, n, sbv, bv);
+            if constexpr (OUT != Q8_OUT_I32) {
+                const int nl = n - n0;  // multiple of 8: two 16-byte LDS reads each
+                const v4f s0 = *reinterpret_cast<const v4f*>(lds_par + 256 + nl), s1 = *reinterpret_cast<const v4f*>(lds_par + 260 + nl);
+                v4f b0 = {0.f, 0.f, 0.f, 0.f}, b1 = b0;
+                if (p.bias != nullptr) {
+                    b0 = *reinterpret_cast<const v4f*>(lds_par + 512 + nl);
+                    b1 = *reinterpret_cast<const v4f*>(lds_par + 516 + nl);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { sbv[e] = s0[e]; sbv[4 + e] = s1[e]; bv[e] = b0[e]; bv[4 + e] = b1[e]; }
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = m0 + wave_m * 128 + 32 * i + r32;
                 if (m >= M) continue;
-                const float sam = (OUT == Q8_OUT_I32) ? 0.f : p.sa[(size_t)za * M + m];
+                const float sam = (OUT == Q8_OUT_I32) ? 0.f : lds_par[wave_m * 128 + 32 * i + r32];
                 using elem_t = typename std::conditional<IN == Q8_I8, int, float>::type;
                 elem_t a8[8];
 #pragma unroll

@@ -100,3 +100,16 @@ def test_functional_asserts_match_reference_contract():
         fp8_linear(a16, a16)  # out_dtype must be 16-bit
     with pytest.raises(AssertionError):
         fp8_linear(a16, a16, out_dtype=torch.float8_e4m3fn)
+
+
+def test_weight_converter_key_mapping():
+    from q8_kernels_amd.utils import converted_key
+    p = "transformer_blocks.3."
+    assert converted_key("proj_in.weight") == ("proj_in.weight", "keep")
+    assert converted_key(p + "scale_shift_table") == (p + "scale_shift_table", "keep")
+    assert converted_key(p + "attn1.to_out.0.weight") == (p + "attn1.to_out.weight", "quantize")
+    assert converted_key(p + "attn1.to_out.0.bias") == (p + "attn1.to_out.bias", "fp32")
+    assert converted_key(p + "attn2.q_norm.weight") == (p + "attn2.q_norm.weight", "fp32")
+    assert converted_key(p + "attn2.to_k.weight") == (p + "attn2.to_k.weight", "quantize")
+    assert converted_key(p + "ff.net.0.proj.weight") == (p + "ff.act.proj.weight", "quantize")
+    assert converted_key(p + "ff.net.2.bias") == (p + "ff.proj_down.bias", "fp32")

@@ -209,3 +209,34 @@ def test_ltx_transformer_block_matches_oracle(dev):
     assert got.shape == hidden.shape and got.dtype == BF16
     assert cosine(got.cpu(), want) > 0.999
     assert (got.cpu().double() - want.double()).abs().max() <= 0.06 * want.double().abs().max()
+
+
+# ------------------------------------------------------------------ weight conversion
+
+def test_convert_state_dict_loads_into_the_block(dev):
+    from q8_kernels_amd.blocks import LTXTransformerBlock
+    from q8_kernels_amd.utils import convert_state_dict
+    dim, heads, hd, kv_dim = 256, 4, 64, 192
+    g = torch.Generator().manual_seed(49)
+    rnd = lambda *s: (torch.randn(*s, generator=g) * 0.05).to(BF16)  # noqa: E731
+    p = "transformer_blocks.0."
+    orig = {"proj_in.weight": rnd(dim, 32), p + "scale_shift_table": torch.randn(6, dim, generator=g)}
+    for a, kd in (("attn1", dim), ("attn2", kv_dim)):
+        for name, i in (("to_q", dim), ("to_k", kd), ("to_v", kd), ("to_out.0", dim)):
+            orig[p + "%s.%s.weight" % (a, name)] = rnd(dim, i)
+            orig[p + "%s.%s.bias" % (a, name)] = rnd(dim)
+        orig[p + a + ".q_norm.weight"] = 1 + rnd(dim)
+        orig[p + a + ".k_norm.weight"] = 1 + rnd(dim)
+    orig[p + "ff.net.0.proj.weight"], orig[p + "ff.net.0.proj.bias"] = rnd(4 * dim, dim), rnd(4 * dim)
+    orig[p + "ff.net.2.weight"], orig[p + "ff.net.2.bias"] = rnd(dim, 4 * dim), rnd(dim)
+    new = convert_state_dict(orig, torch.device(dev))
+    assert new["proj_in.weight"] is orig["proj_in.weight"]
+    assert p + "attn1.to_out.weight" in new and p + "attn1.to_out.0.weight" not in new
+    wq, ws = O.ref_quant(O.ref_fht(orig[p + "ff.net.2.weight"]))
+    assert_bit_equal(new[p + "ff.proj_down.weight"], wq, "converted codes")
+    assert_bit_equal(new[p + "ff.proj_down.scales"], ws, "converted scales")
+    assert new[p + "attn2.k_norm.weight"].dtype == torch.float32 and new[p + "ff.act.proj.bias"].dtype == torch.float32
+    blk = LTXTransformerBlock(dim, heads, hd, kv_dim, bias=True, use_rope=True, norm_affine=False).to(dev)
+    missing, unexpected = blk.load_state_dict({k[len(p):]: v for k, v in new.items() if k.startswith(p)}, strict=True)
+    assert not missing and not unexpected
+    assert blk.ff.proj_down.weight.dtype == torch.int8 and blk.attn1.to_q.scales.dtype == torch.float32
