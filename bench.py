@@ -28,6 +28,16 @@ HBM_PEAK_GBS = 8000.0
 E4M3 = torch.float8_e4m3fn
 
 
+def _ramp_clocks(fn, seconds=0.4):
+    """Untimed: keep the device busy with `fn` until it has left its idle clock state (the engine clock of an idle
+    MI355X takes on the order of 100 ms of load to come up; short timings taken before that read about 25 % low)."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+
+
 def _time(fn, steps, warmup):
     """Mean seconds per call over exactly `steps` calls (HIP events on the current stream, which is the
     stream the library launches on)."""
@@ -147,8 +157,8 @@ def _extras(dev, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -174,6 +184,7 @@ def main():
         dst.copy_(src)  # reads 512 MiB, writes 512 MiB
         torch.cuda.synchronize()
         del src, dst
+    _ramp_clocks(step)
     sec, wall = _time(step, args.steps, args.warmup)
     flop = 2.0 * M * N * K
     tflops = flop / sec / 1e12

@@ -22,7 +22,7 @@
 //   * Workgroup ids are re-mapped so that each XCD (ids congruent mod 8 share an L2) owns a
 //     contiguous range of tiles, walked in groups of GROUP_M tile rows for L2 reuse of A and B.
 #include "gemm_common.h"
-#include "gemm_pipe.h"
+#include "gemm_persist.h"
 
 namespace q8 {
 
@@ -177,7 +177,8 @@ using CfgBig = GemmCfg<IN, 2, 4, 8, 4>;
 template <int IN>
 using CfgSmall = GemmCfg<IN, 2, 2, 4, 4>;
 
-static int g_force_cfg = 0;  // 0 = auto, 1 = pipelined 256x256, 2 = 128x128, 3 = plain 256x256 (see q8_gemm_set_config)
+static int g_force_cfg = 0;  // 0 = auto, 1 = pipelined 256x256 (one tile per workgroup), 2 = 128x128, 3 = plain 256x256,
+                             // 4 = persistent pipelined 256x256 where eligible (see q8_gemm_set_config)
 
 template <int IN, int OUT, bool GELU>
 static int launch_pipe(const GemmParams& p, hipStream_t stream) {
@@ -197,10 +198,42 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
     return launch_status("q8_gemm");
 }
 
+// One workgroup per CU walking over the tiles (gemm_persist.h); bf16 output, N % 8 == 0, K a multiple of 128 above 256.
+template <int IN, bool GELU>
+static int launch_persist(const GemmParams& p, hipStream_t stream) {
+    const int tiles_m = (p.M + kPipeBM - 1) / kPipeBM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
+    const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
+    const long total = (long)tiles_m * tiles_n * batch;
+    if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
+    auto kern = gemm_persist_kernel<IN, GELU>;
+    static thread_local bool attr_set = false;
+    static thread_local int cus = 0;
+    if (!attr_set) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPersistLds) !=
+                hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", kPersistLds);
+        }
+        cus = cus > 0 ? (cus / 8) * 8 : 256;  // a multiple of the 8 XCDs keeps every workgroup's tiles on one XCD
+        if (cus == 0) cus = 8;
+        attr_set = true;
+    }
+    const int grid = total < cus ? (int)total : cus;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), kPersistLds, stream, p, tiles_m, tiles_n, (int)total);
+    return launch_status("q8_gemm");
+}
+
 template <int IN, int OUT, bool GELU>
 static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
     const long big_tiles = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.batch_a > p.batch_b ? p.batch_a : p.batch_b);
-    const bool big = g_force_cfg == 1 || (g_force_cfg == 0 && big_tiles >= 192);
+    const bool big = g_force_cfg == 1 || g_force_cfg == 4 || (g_force_cfg == 0 && big_tiles >= 192);
+    if constexpr (OUT == Q8_BF16) {
+        if (big && g_force_cfg != 1 && (p.N % 8) == 0 && p.K > 256 && (p.K % 128) == 0 && (uint64_t)p.M * p.K < (1ull << 32) &&
+            (uint64_t)p.N * p.K < (1ull << 32))
+            return launch_persist<IN, GELU>(p, stream);
+    }
     if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
     if (g_force_cfg == 3) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);
     return launch_gemm<CfgSmall<IN>, OUT, GELU>(p, stream);
@@ -225,7 +258,7 @@ static int check_gemm(const char* who, const void* A, const void* B, const void*
 using namespace q8;
 
 extern "C" int q8_gemm_set_config(int cfg) {
-    if (cfg < 0 || cfg > 3) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 4) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
     g_force_cfg = cfg;
     return Q8_OK;
 }

@@ -1,0 +1,316 @@
+// Persistent form of the pipelined 256x256 GEMM tile (gemm_pipe.h): one workgroup per CU walks over several output
+// tiles and the HBM->LDS copy pipeline runs straight across the tile boundaries.
+//
+//   * Work item v (tile id + tiles * batch index) is handled by workgroup v % gridDim.x, which runs on XCD v % 8;
+//     the tile walk is the XCD-contiguous grouped walk of tile_of_block, so the L2 reuse is the same.
+//   * The compute side counts K stages globally (g); the copy side runs two stages ahead of it (gl = g + 2) with its
+//     own (item, k) position and source pointers. While the last two stages of a tile are multiplied, the first two
+//     stages of the next tile are already on their way, and they land while the epilogue of the finished tile runs.
+//   * The epilogue therefore may not touch the two stage buffers: every wave stages its results through 2 KiB of its
+//     own (16 rows x 128 B per round, two rounds per 32-row MFMA tile, chunks swizzled by (row >> 1) & 7) and writes
+//     8 complete 128-byte lines per store instruction. All LDS traffic of the epilogue is inline assembly with its own
+//     lgkmcnt waits; the stores are never waited for, they drain under the next tile's MFMAs.
+//   * sa / sb / bias of a tile are copied to LDS (double-buffered) when the copy side enters the tile.
+//   * Every wave issues the same number of copy instructions per stage (8, and 2 more in a stage where the copy
+//     side moves to the next tile; past the last tile the copies read a block of zeros), so the in-order vmcnt
+//     waits are exact.
+#pragma once
+#include "gemm_pipe.h"
+
+namespace q8 {
+
+constexpr int kPersistParOffset = kPipeStages * kPipeStageBytes;            // 2 x (sa[256], sb[256], bias[256])
+constexpr int kPersistStageOutOffset = kPersistParOffset + 2 * 3 * 256 * 4;   // 8 waves x 2 KiB
+constexpr int kPersistLds = kPersistStageOutOffset + 8 * 2048;
+
+__device__ __forceinline__ void lds_write_b128(unsigned addr, v4u v) {
+    asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ float lds_read_b32(unsigned addr) {
+    float r;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+
+// tile of work item `pid_in` out of `nb` = tiles_m * tiles_n (same walk as tile_of_block)
+__device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+    const int xcd = bid & 7, loc = bid >> 3, per = nb >> 3, rem = nb & 7;
+    const int pid = xcd * per + (xcd < rem ? xcd : rem) + loc;
+    const int group_size = kGroupM * tiles_n;
+    const int gid = pid / group_size, first_m = gid * kGroupM;
+    const int gsz = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+    tile_m = first_m + (pid % group_size) % gsz;
+    tile_n = (pid % group_size) / gsz;
+}
+
+// Requirements checked by the host: K % 128 == 0 and K > 256 (at least 3 whole stages per tile), N % 8 == 0,
+// M * K and N * K below 2^32 (32-bit source offsets), OUT == Q8_BF16.
+template <int IN, bool GELU>
+__global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    constexpr int BM = kPipeBM, BN = kPipeBN;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int wave_m = wave >> 2, wave_n = wave & 3;
+    const int M = p.M, N = p.N, K = p.K;
+    const int tiles = tiles_m * tiles_n;
+    const int KT = (K + 127) >> 7;
+    const int G = gridDim.x;
+    const int count = (total - (int)blockIdx.x + G - 1) / G;  // >= 1: the grid never exceeds `total`
+
+    struct Item { int m0, n0, z, za, zb; };
+    auto item_of = [&](int idx) {
+        const int v = blockIdx.x + idx * G;
+        const int z = v / tiles;
+        int tm, tn;
+        tile_of_id(v - z * tiles, tiles, tiles_m, tiles_n, tm, tn);
+        return Item{tm * BM, tn * BN, z, (p.batch_a == 1) ? 0 : z, (p.batch_b == 1) ? 0 : z};
+    };
+
+    // ---- copy side ------------------------------------------------------------------------------------------
+    // A stage is 64 row groups of 1 KiB (8 rows x 128 B): groups 0..31 hold A, 32..63 B. Wave w copies groups
+    // w, w+8, w+16, w+24 of each; lane (lane/8, lane%8) fills row 8 q + lane/8, physical chunk lane%8, from logical
+    // chunk (lane%8) ^ ((row >> 1) & 7).
+    // (the swizzle term is the same for the 8 row groups of a wave: their rows differ by multiples of 64).
+    // Sources are a uniform base per operand plus a 32-bit byte offset per lane and row group.
+    uint32_t off[8];
+    const uint8_t* baseA;
+    const uint8_t* baseB;
+    const uint32_t kchunk = 16 * ((lane & 7) ^ ((4 * wave + (lane >> 4)) & 7));
+    bool copy_live = true;  // the copy side still points at a real tile
+    auto set_src = [&](const Item& it) {
+        baseA = p.A + (size_t)it.za * M * K;
+        baseB = p.B + (size_t)it.zb * N * K;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int rho = 8 * (wave + 8 * (i & 3)) + (lane >> 3);
+            if (i < 4) {
+                int m = it.m0 + rho;
+                m = m < M ? m : M - 1;
+                off[i] = (uint32_t)m * (uint32_t)K + kchunk;
+            } else {
+                const int slab = rho >> 6, t = (rho >> 5) & 1, w = (rho >> 3) & 3, hh = (rho >> 2) & 1, r = rho & 3;
+                int n = it.n0 + 64 * slab + 32 * t + 16 * (w >> 1) + 8 * hh + 4 * (w & 1) + r;
+                n = n < N ? n : N - 1;
+                off[i] = (uint32_t)n * (uint32_t)K + kchunk;
+            }
+        }
+    };
+    auto set_src_zeros = [&]() {  // past the last tile: every lane reads the same 16 zero bytes
+        baseA = baseB = reinterpret_cast<const uint8_t*>(g_zero16);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) off[i] = 0;
+    };
+    // two 4-byte-per-lane copies per wave: waves 0-3 bring sa and bias, waves 4-7 sb (twice, to keep the count equal)
+    auto copy_params = [&](const Item& it, int buf, bool live) {
+        float* par = reinterpret_cast<float*>(lds + kPersistParOffset) + buf * 768;
+        const int j = (wave & 3) * 64 + lane;
+        const float* g0;
+        const float* g1;
+        float* d0;
+        float* d1;
+        if (wave < 4) {
+            const int m = (it.m0 + j < M) ? it.m0 + j : M - 1;
+            const int n = (it.n0 + j < N) ? it.n0 + j : N - 1;
+            g0 = p.sa + (size_t)it.za * M + m;
+            g1 = (p.bias != nullptr) ? p.bias + n : reinterpret_cast<const float*>(g_zero16);
+            d0 = par + (wave & 3) * 64;
+            d1 = par + 512 + (wave & 3) * 64;
+        } else {
+            const int n = (it.n0 + j < N) ? it.n0 + j : N - 1;
+            g0 = g1 = p.sb + (size_t)it.zb * N + n;
+            d0 = d1 = par + 256 + (wave & 3) * 64;
+        }
+        if (!live) g0 = g1 = reinterpret_cast<const float*>(g_zero16);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g0,
+                                         (__attribute__((address_space(3))) void*)d0, 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g1,
+                                         (__attribute__((address_space(3))) void*)d1, 4, 0, 0);
+    };
+    int l_item = 0, l_k = 0, gl = 0;  // copy side: item, stage inside the item, global stage count
+    auto issue_copy = [&](int i) {    // copy instruction i (0..7) of the copy side's current stage
+        uint8_t* base = lds + (gl & 1) * kPipeStageBytes;
+        const uint32_t k0 = copy_live ? (uint32_t)l_k << 7 : 0u;
+        const int q = (i < 4 ? 0 : 32) + wave + 8 * (i & 3);
+        const uint8_t* g = (i < 4 ? baseA : baseB) + k0 + off[i];
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                         (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
+    };
+    // after the 8th copy of a stage; returns true when the copy side moved to the next tile (2 more copies issued)
+    auto advance_copy = [&]() {
+        ++gl;
+        if (++l_k < KT) return false;
+        l_k = 0;
+        ++l_item;
+        copy_live = l_item < count;
+        const Item it = item_of(copy_live ? l_item : 0);
+        if (copy_live) set_src(it);
+        else set_src_zeros();
+        copy_params(it, l_item & 1, copy_live);
+        return true;
+    };
+
+    // ---- operand fetch addresses: [K half s][low / high chunk], byte offsets inside a stage
+    const unsigned lds0 = lds_addr(lds);
+    const unsigned a_row = lds0 + wave_m * 16384 + (lane & 31) * 128;
+    const unsigned b_row = lds0 + 32768 + wave_n * 8192 + (lane & 31) * 128;
+    unsigned pc[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        pc[s][0] = ((4 * s + 2 * (lane >> 5)) ^ (((lane & 31) >> 1) & 7)) * 16;
+        pc[s][1] = pc[s][0] ^ 16;
+    }
+    auto read_half = [&](PipeFrags& f, int stage, int s) {
+        const unsigned so = (stage & 1) * kPipeStageBytes;
+        pipe_read_frags(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+    };
+
+    using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
+    acc_t acc[4][2];
+
+    // ---- prologue: stage 0 landed, stage 1 in flight, fragments of the first K half on their way
+    Item cur = item_of(0);
+    set_src(cur);
+    copy_params(cur, 0, true);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) issue_copy(i);
+    advance_copy();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) issue_copy(i);
+    advance_copy();
+    PipeFrags f0, f1;
+    read_half(f0, 0, 0);
+
+    int g = 0;  // compute side: global stage count
+    for (int item = 0; item < count; ++item) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][t][e] = 0;
+
+        for (int k = 0; k < KT; ++k, ++g) {
+            const bool last = (k == KT - 1);
+            // f0: first K half of stage g (reads in flight); the copies of stage g+1 are in flight
+            pipe_wait_frags(f0);
+            read_half(f1, g, 1);
+            pipe_pin(f0);
+            // First half. Once the second half of stage g is in registers everywhere (barrier 1), buffer g & 1 is
+            // free and the copies of stage g+2 start to trickle out, one per MFMA tile.
+            pipe_mfma<IN>(f0, acc, [&](int j) {
+                if (j == 3) {
+                    pipe_wait_frags(f1);
+                    __builtin_amdgcn_s_barrier();
+                }
+                if (j >= 4) issue_copy(j - 4);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+            pipe_pin(f1);
+            // Second half. After the last copy of stage g+2 everything older (stage g+1, and the stores of the
+            // previous epilogue) must have completed; barrier 2 makes that true for every wave's copies, then the
+            // first half of stage g+1 is fetched under the remaining MFMA tiles (after the epilogue at a tile's end).
+            bool moved = false;
+            pipe_mfma<IN>(f1, acc, [&](int j) {
+                if (j < 4) issue_copy(4 + j);
+                if (j == 3) moved = advance_copy();
+                if (j == 4) {
+                    if (moved) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    // the fragment registers are free for the epilogue after the last stage of a tile
+                    if (!last) read_half(f0, g + 1, 0);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // ---- epilogue of tile `item`: lane (r32, h) holds for MFMA tile (i, t) and register octet wp the 8 columns
+        //      32 t + 16 wp + 8 h .. + 7 of the wave's 64-column slab, row 32 i + r32.
+        // (the lane id passes through an empty asm so that none of the address arithmetic below is hoisted out of
+        //  the tile loop, where it would take registers away from the main loop)
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
+        const int r32 = lane_e & 31, h = lane_e >> 5;
+        const unsigned stage_out = lds0 + kPersistStageOutOffset + wave * 2048;
+        const unsigned par = lds0 + kPersistParOffset + (item & 1) * 3072;
+        const size_t zc = (size_t)cur.z * M * N;
+        const int mw0 = cur.m0 + wave_m * 128, nw0 = cur.n0 + wave_n * 64;
+        v4i sbq[2][2][2], bq[2][2][2];  // [t][wp][low / high 4 columns]
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int wp = 0; wp < 2; ++wp) {
+                const unsigned o = (wave_n * 64 + 32 * t + 16 * wp + 8 * h) * 4;
+                sbq[t][wp][0] = lds_read_b128<1024>(par + o);
+                sbq[t][wp][1] = lds_read_b128<1024 + 16>(par + o);
+                bq[t][wp][0] = lds_read_b128<2048>(par + o);
+                bq[t][wp][1] = lds_read_b128<2048 + 16>(par + o);
+            }
+        float sam[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sam[i] = lds_read_b32(par + (wave_m * 128 + 32 * i + r32) * 4);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(sam[0]), "+v"(sam[1]), "+v"(sam[2]), "+v"(sam[3]), "+v"(sbq[0][0][0]), "+v"(sbq[0][0][1]),
+                       "+v"(sbq[0][1][0]), "+v"(sbq[0][1][1]), "+v"(sbq[1][0][0]), "+v"(sbq[1][0][1]), "+v"(sbq[1][1][0]),
+                       "+v"(sbq[1][1][1]), "+v"(bq[0][0][0]), "+v"(bq[0][0][1]), "+v"(bq[0][1][0]), "+v"(bq[0][1][1]),
+                       "+v"(bq[1][0][0]), "+v"(bq[1][0][1]), "+v"(bq[1][1][0]), "+v"(bq[1][1][1])
+                     :
+                     : "memory");
+        uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // the lane's 4 chunks of row 32 i + r32: chunk c = 4 t + 2 wp + h
+            v4u outc[2][2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int wp = 0; wp < 2; ++wp) {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float sbv = __int_as_float(sbq[t][wp][e >> 2][e & 3]);
+                        const float bv = __int_as_float(bq[t][wp][e >> 2][e & 3]);
+                        float x = fmaf((float)acc[i][t][8 * wp + e], sam[i] * sbv, bv);
+                        if constexpr (GELU) x = gelu_tanh_fast(x);
+                        v[e] = x;
+                    }
+                    outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
+                }
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                // rows 16 half .. 16 half + 15 of the MFMA tile: their lanes write, then all lanes store 16 full rows
+                if ((r32 >> 4) == half) {
+                    const int row = r32 & 15;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int wp = 0; wp < 2; ++wp)
+                            lds_write_b128(stage_out + row * 128 + (((4 * t + 2 * wp + h) ^ ((row >> 1) & 7)) * 16), outc[t][wp]);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                v4i w[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int row = 8 * j + (lane_e >> 3);
+                    w[j] = lds_read_b128<0>(stage_out + row * 128 + (((lane_e & 7) ^ ((row >> 1) & 7)) * 16));
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0]), "+v"(w[1]) : : "memory");
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int m = mw0 + 32 * i + 16 * half + 8 * j + (lane_e >> 3);
+                    const int n = nw0 + (lane_e & 7) * 8;
+                    if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * N + n) = w[j];
+                }
+            }
+        }
+        if (item + 1 < count) cur = item_of(item + 1);
+        read_half(f0, g, 0);  // first fragments of the next tile (its first two stages landed before barrier 2 above)
+    }
+    // drain: the look-ahead copies and fragment reads past the last stage target LDS / registers that nobody uses
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    pipe_wait_frags(f0);
+}
+
+}  // namespace q8

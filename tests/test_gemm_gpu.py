@@ -19,7 +19,7 @@ def _set_cfg(c):
     _lib.check(_lib.lib().q8_gemm_set_config(c))
 
 
-@pytest.fixture(params=[1, 2], ids=["tile256", "tile128"])
+@pytest.fixture(params=[1, 2, 4], ids=["tile256", "tile128", "persistent256"])
 def tile_cfg(request):
     _set_cfg(request.param)
     yield request.param
@@ -136,6 +136,33 @@ def test_mm_batch_broadcast(dev, tile_cfg):
         assert got.shape == want.shape
         diff = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
         assert diff.max() <= 1, "batch case a%s b%s" % (tuple(a.shape), tuple(b.shape))
+
+
+@pytest.mark.parametrize("case", [(1, 1, 4352, 4096, 384), (3, 1, 1100, 4600, 512), (1, 2, 2300, 2816, 640)])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu):
+    """More 256x256 tiles than CUs (272, 270 and 198+ with ragged edges and batch broadcast), so that workgroups of the
+    persistent kernel cross tile and batch boundaries; int8 operands make the accumulators exact, the epilogue
+    is fp32 on both sides: at most one bf16 ulp."""
+    ba, bb, m, n, k = case
+    g = torch.Generator().manual_seed(m + n)
+    a = _rand_i8(g, ba, m, k) if ba > 1 else _rand_i8(g, m, k)
+    b = _rand_i8(g, bb, n, k) if bb > 1 else _rand_i8(g, n, k)
+    sa = torch.rand(ba * m, generator=g) * 2e-3 + 1e-4
+    sb = torch.rand(bb * n, generator=g) * 2e-2 + 1e-3
+    bias = torch.randn(n, generator=g)
+    _set_cfg(4)
+    try:
+        got = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.to(dev), sb.to(dev), fuse_gelu, torch.bfloat16)
+    finally:
+        _set_cfg(0)
+    want = O.ref_q8_mm(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
+    assert got.shape == want.shape
+    diff = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    # far in GELU's negative tail the float64 formula 1 + tanh cancels to zero while the kernel keeps the tiny value
+    diff = torch.where((got.cpu().float() - want.float()).abs() <= 1e-7, torch.zeros_like(diff), diff)
+    assert int(diff.max()) <= 1, "max %d ulp at %s" % (int(diff.max()), (diff == diff.max()).nonzero()[0].tolist())
+    assert float((diff > 0).float().mean()) < (0.02 if fuse_gelu else 0.002)
 
 
 # ------------------------------------------------------------------ fp8 at the benchmark shapes

@@ -70,6 +70,10 @@ def test_hip_kernels_reproduce_fixture(dev):
     sa, sb, bias = (torch.from_numpy(G[n].copy()).to(dev) for n in ("gemm_sa", "gemm_sb", "gemm_bias"))
     out = _C.q8_mm_bias(a, b, bias, sa, sb, True, torch.bfloat16)[0].cpu()
     d = np.abs(out.view(torch.int16).numpy().astype(np.int32) - G["gemm_out_gelu_bf16"].astype(np.int32))
+    # far in GELU's negative tail the fixture's float64 formula 1 + tanh cancels to -0 while the kernel keeps the tiny
+    # value (about -1e-20): those elements are compared absolutely
+    want = torch.from_numpy(G["gemm_out_gelu_bf16"].astype(np.int16)).view(torch.bfloat16).float().numpy()
+    d[np.abs(out.float().numpy() - want) <= 1e-7] = 0
     assert d.max() <= 2
     out8 = _C.q8_mm_bias(a, b, bias, sa, sb, False, None)[0].cpu().view(torch.uint8).numpy()
     assert (out8 != G["gemm_out_e4m3"]).mean() < 0.02
