@@ -131,6 +131,13 @@ def _extras(dev, steps, warmup):
     sa, sb, bias = torch.rand(6144, generator=g).to(dev), torch.rand(2048, generator=g).to(dev), torch.randn(2048, generator=g).to(dev)
     t, _ = _time(lambda: _C.q8_mm_bias(a, b, bias, sa, sb, False, torch.bfloat16), steps, warmup)
     out["int8_gemm_6144x2048x2048"] = {"ms": t * 1e3, "tops": 2.0 * 6144 * 2048 * 2048 / t / 1e12}
+    # fp8 GEMMs of the block without GELU: projection (K = 2048) and FFN down projection (K = 8192), M = 12288 tokens
+    for name, (mm, nn, kk) in (("fp8_gemm_12288x2048x2048", (12288, 2048, 2048)), ("fp8_gemm_12288x2048x8192", (12288, 2048, 8192))):
+        _, _, gb, gxq, gsx, gwq, gsw = _gemm_inputs(dev, mm, nn, kk, seed=2)
+        gb = gb.to(dev)
+        t, _ = _time(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, False, torch.bfloat16), steps, warmup)
+        out[name] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12, "frac_of_fp8_peak": 2.0 * mm * nn * kk / t / 1e12 / FP8_PEAK_TFLOPS}
+        del gxq, gwq
     # row kernels on [12288, 2048] tokens
     x = torch.randn(12288, 2048, generator=g).to(torch.bfloat16).to(dev)
     n = x.numel()
@@ -139,6 +146,16 @@ def _extras(dev, steps, warmup):
     for name, fn, bpe in (("quant_fp8", lambda: _C.tokenwise_quant(x, E4M3), 3), ("quant_int8", lambda: _C.tokenwise_quant(x, None), 3),
                           ("fht_bf16", lambda: _C.fast_hadamard_transform(x, 2048 ** -0.5, None), 4),
                           ("rmsnorm_bf16", lambda: _C.rms_norm(x, w, None), 4), ("rope_bf16", lambda: _C.rope(x, cos, sin, None), 12)):
+        t, _ = _time(fn, steps, warmup)
+        out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    # fused row kernels: FHT + int8 quantizer, RMSNorm + e4m3 quantizer (2 B in, 1 B out per element), and the attention
+    # prologue RoPE + head split + FHT-64 + e4m3 cast (2 B in + 8 B of tables, 1 B out)
+    xs = x.view(2, 6144, 2048)
+    cs3, sn3 = cos.view(2, 6144, 2048), sin.view(2, 6144, 2048)
+    for name, fn, bpe in (("fht_quant_int8_fused", lambda: _C.fht_quant(x, 2048 ** -0.5, None), 3),
+                          ("rmsnorm_quant_fp8_fused", lambda: _C.rms_norm_quant(x, w, E4M3), 3),
+                          ("attn_prep_qk_rope_fht_fp8", lambda: _C.attn_prep_qk(xs, 32, cs3, sn3, True, 0.125), 11),
+                          ("attn_prep_v_fp8", lambda: _C.attn_prep_v(xs, 32), 3)):
         t, _ = _time(fn, steps, warmup)
         out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
     # the DiT block (config 5)
@@ -204,7 +221,7 @@ def main():
         "config": {"workload": "fp8 e4m3 GEMM + per-token/per-channel dequant + bias + tanh-GELU -> bf16, M=6144 N=8192 K=2048",
                    "inputs": "X~N(0,1), W~N(0,0.02), bias~N(0,0.02), per-row absmax e4m3 quantisation, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / FP8_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "gemm_pipe_kernel<e4m3, bf16, gelu>", "flop_per_launch": flop,
+                     "traffic": None, "kernel": "gemm_persist_kernel<e4m3, gelu>", "flop_per_launch": flop,
                      "avg_launch_us": sec * 1e6, "host_wall_us_per_step": wall * 1e6},
     }
     traffic_file = os.path.join(ROOT, "profiles", "gemm_fp8_traffic.json")

@@ -41,9 +41,11 @@ __global__ __launch_bounds__(kBlock) void fht_quant_kernel(const void* __restric
     for (int c = 0; c < CH; ++c) {
         const int e = (c * LANES + t) * 8;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            v[c][i] = round_mid<MID>(v[c][i] * fht_scale);
-            if (e < dim) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));  // outputs beyond dim are dropped
+        for (int i = 0; i < 8; ++i) v[c][i] *= fht_scale;
+        round_mid8<MID>(v[c]);
+        if (e < dim) {  // outputs beyond dim are dropped
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));
         }
     }
     row_reduce<LANES, true, 1>(amax, red);
@@ -101,11 +103,12 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
             float wv[8];
             load8<Q8_F32>(w, e, wv);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = round_mid<MID>((v[c][i] * rstd) * wv[i]);
+            for (int i = 0; i < 8; ++i) v[c][i] = (v[c][i] * rstd) * wv[i];
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = round_mid<MID>(v[c][i] * rstd);
+            for (int i = 0; i < 8; ++i) v[c][i] = v[c][i] * rstd;
         }
+        round_mid8<MID>(v[c]);
 #pragma unroll
         for (int i = 0; i < 8; ++i) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));
     }
@@ -143,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
     if (tok >= tokens) return;  // no barrier below; the lane exchanges stay inside a head, i.e. inside a token
     const int64_t b = tok / S, s = tok - b * S;
     const uint16_t* xr = x + tok * x_row_stride;
-    auto mid = [&](float f) { return mid_bf16 ? round_mid<Q8_BF16>(f) : f; };
+    auto mid8 = [&](float (&f)[8]) { if (mid_bf16) round_mid8<Q8_BF16>(f); };
 
     float v[CH][8];
 #pragma unroll
@@ -161,8 +164,9 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
                 o[i] = v[c][i] * cv[i] - v[c][i + 1] * sv[i];
                 o[i + 1] = v[c][i + 1] * cv[i + 1] + v[c][i] * sv[i + 1];
             }
+            mid8(o);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = mid(o[i]);
+            for (int i = 0; i < 8; ++i) v[c][i] = o[i];
         }
     }
 #pragma unroll
@@ -191,11 +195,9 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
         v2i w;
         if (scales != nullptr) {
             float amax = 0.f;
+            mid8(v[c]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                v[c][i] = mid(v[c][i]);
-                amax = fmaxf(amax, fabsf(v[c][i]));
-            }
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[c][i]));
             amax = group_max<LH>(amax);
             const float ratio = quant_ratio<Q8_E4M3>(amax);
             if ((t % LH) == 0) scales[orow] = quant_scale<Q8_E4M3>(amax, ratio, 0);

@@ -188,7 +188,7 @@ __device__ __forceinline__ void store8(void* p, int64_t e, const float (&v)[8]) 
     if constexpr (DT == Q8_BF16) {
         v4u w;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) w[i] = pack2_bf16(v[2 * i], v[2 * i + 1]);
         *reinterpret_cast<v4u*>(reinterpret_cast<uint16_t*>(p) + e) = w;
     } else {
         static_assert(DT == Q8_E4M3, "store8: unsupported element type");

@@ -236,6 +236,18 @@ __device__ __forceinline__ float round_mid(float x) {
     if constexpr (MID == Q8_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(x));
     else return x;
 }
+// the same for 8 values at once: four hardware pair conversions and their unpacking
+template <int MID>
+__device__ __forceinline__ void round_mid8(float (&v)[8]) {
+    if constexpr (MID == Q8_BF16) {
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            const uint32_t u = pack2_bf16(v[i], v[i + 1]);
+            v[i] = __uint_as_float(u << 16);
+            v[i + 1] = __uint_as_float(u & 0xffff0000u);
+        }
+    }
+}
 
 // reference order: r = QMAX / absmax, code = x * r, stored scale = 1 / r
 // (csrc/quantizer/tokenwise_quant_cuda.cu:135-147), in IEEE fp32; a row of zeros gets codes 0 and scale 0.
@@ -255,15 +267,30 @@ template <int OUT>
 __device__ __forceinline__ v2i quant_codes8(const float (&v)[8], float ratio, int flags) {
     v2i w;
     if constexpr (OUT == Q8_I8) {
-        uint32_t b[8];
+        // |q| <= 127 (1 + 2^-23). Round half away from zero = truncate(q + copysign(0.5 - 2^-25, q)) for every
+        // fp32 |q| < 2^22 (the sum rounds up to the next integer exactly for the ties and for nothing below them);
+        // round half even = v_rndne. Two saturating 32->16 packs and one byte permute gather the 4 codes of a word.
+        int qi[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float q = v[i] * ratio;
-            const float qr = (flags & Q8_QUANT_RNE) ? rintf(q) : roundf(q);
-            b[i] = (uint32_t)(int)qr & 0xffu;
+            if (flags & Q8_QUANT_RNE) {
+                qi[i] = (int)rintf(q);
+            } else {
+                const float half = __uint_as_float(0x3effffffu | (__float_as_uint(q) & 0x80000000u));
+                qi[i] = (int)(q + half);  // the conversion truncates
+            }
         }
-        w[0] = (int)(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24));
-        w[1] = (int)(b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            typedef short v2s __attribute__((ext_vector_type(2)));
+            const v2s p0 = __builtin_amdgcn_cvt_pk_i16(qi[4 * j], qi[4 * j + 1]);
+            const v2s p1 = __builtin_amdgcn_cvt_pk_i16(qi[4 * j + 2], qi[4 * j + 3]);
+            uint32_t u0, u1;
+            __builtin_memcpy(&u0, &p0, 4);
+            __builtin_memcpy(&u1, &p1, 4);
+            w[j] = (int)__builtin_amdgcn_perm(u1, u0, 0x06040200u);  // bytes 0 and 2 of u0, then of u1
+        }
     } else {
         // |x * r| <= 448 (1 + 2^-23): never reaches the NaN range of the c10 cast
         uint32_t p0 = cvt_pk_e4m3(v[0] * ratio, v[1] * ratio, 0u, false);
