@@ -36,19 +36,28 @@ struct PipeFrags {
 
 // a0/a1 (b0/b1): byte address of the lane's low/high 16-byte chunk in row (lane % 32) of the wave's first A (B)
 // tile; the following 32-row tiles are 4096 bytes apart.
+template <int SKIP = 0>  // tuning builds: 1 = leave the B fragments, 2 = leave the A fragments as they are
 __device__ __forceinline__ void pipe_read_frags(PipeFrags& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
-    f.b[0][0] = lds_read_b128<0>(b0);
-    f.b[0][1] = lds_read_b128<0>(b1);
-    f.a[0][0] = lds_read_b128<0>(a0);
-    f.a[0][1] = lds_read_b128<0>(a1);
-    f.b[1][0] = lds_read_b128<4096>(b0);
-    f.b[1][1] = lds_read_b128<4096>(b1);
-    f.a[1][0] = lds_read_b128<4096>(a0);
-    f.a[1][1] = lds_read_b128<4096>(a1);
-    f.a[2][0] = lds_read_b128<8192>(a0);
-    f.a[2][1] = lds_read_b128<8192>(a1);
-    f.a[3][0] = lds_read_b128<12288>(a0);
-    f.a[3][1] = lds_read_b128<12288>(a1);
+    if constexpr (SKIP != 1) {
+        f.b[0][0] = lds_read_b128<0>(b0);
+        f.b[0][1] = lds_read_b128<0>(b1);
+    }
+    if constexpr (SKIP != 2) {
+        f.a[0][0] = lds_read_b128<0>(a0);
+        f.a[0][1] = lds_read_b128<0>(a1);
+    }
+    if constexpr (SKIP != 1) {
+        f.b[1][0] = lds_read_b128<4096>(b0);
+        f.b[1][1] = lds_read_b128<4096>(b1);
+    }
+    if constexpr (SKIP != 2) {
+        f.a[1][0] = lds_read_b128<4096>(a0);
+        f.a[1][1] = lds_read_b128<4096>(a1);
+        f.a[2][0] = lds_read_b128<8192>(a0);
+        f.a[2][1] = lds_read_b128<8192>(a1);
+        f.a[3][0] = lds_read_b128<12288>(a0);
+        f.a[3][1] = lds_read_b128<12288>(a1);
+    }
 }
 
 // Wait until every LDS read issued so far has landed; the fragments pass through the statement so that no
@@ -93,7 +102,8 @@ __device__ __forceinline__ void pipe_mfma(const PipeFrags& f, ACC (&acc)[4][2], 
     }
 }
 
-// DBG (tuning builds only): bit 0 = no HBM->LDS loads, 1 = no LDS reads, 2 = no MFMA, 3 = no stores, 4 = no barrier
+// DBG (tuning builds only): bit 0 = no HBM->LDS loads, 1 = no LDS reads, 2 = no MFMA, 3 = no stores, 4 = no barrier,
+// 6 = no vmcnt wait, 7 = no B fragment reads, 8 = no A fragment reads in the loop
 template <int IN, int OUT, bool GELU, int DBG = 0>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -162,7 +172,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     auto read_half = [&](PipeFrags& f, int stage, int s) {
         if constexpr (DBG & 2) return;
         const unsigned so = (stage & 1) * kPipeStageBytes;
-        pipe_read_frags(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+        pipe_read_frags<(DBG & 128) ? 1 : ((DBG & 256) ? 2 : 0)>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0],
+                                                                   b_row + so + pc[s][1]);
     };
 
     using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
@@ -202,11 +213,17 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
     issue_loads(1);
-    if constexpr (DBG & 2) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { f0.a[i][0] = f0.a[i][1] = f1.a[i][0] = f1.a[i][1] = v4i{0x38383838, 0x38383838, 0x38383838, 0x38383838}; }
-#pragma unroll
-        for (int t = 0; t < 2; ++t) { f0.b[t][0] = f0.b[t][1] = f1.b[t][0] = f1.b[t][1] = v4i{0x38383838, 0x38383838, 0x38383838, 0x38383838}; }
+    if constexpr (DBG & 2) {  // fragments of stage 0 are read once and reused for every stage
+        pipe_read_frags(f0, a_row + pc[0][0], a_row + pc[0][1], b_row + pc[0][0], b_row + pc[0][1]);
+        pipe_read_frags(f1, a_row + pc[1][0], a_row + pc[1][1], b_row + pc[1][0], b_row + pc[1][1]);
+        pipe_wait_frags(f0);
+        pipe_wait_frags(f1);
+    }
+    if constexpr ((DBG & (128 | 256)) != 0) {  // the fragments that the loop leaves alone get real data once
+        pipe_read_frags(f0, a_row + pc[0][0], a_row + pc[0][1], b_row + pc[0][0], b_row + pc[0][1]);
+        pipe_read_frags(f1, a_row + pc[1][0], a_row + pc[1][1], b_row + pc[1][0], b_row + pc[1][1]);
+        pipe_wait_frags(f0);
+        pipe_wait_frags(f1);
     }
     read_half(f0, 0, 0);
 
