@@ -211,7 +211,8 @@ int q8_gemm(const void* A, const void* B, const float* bias, const float* sa, co
 /*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with
  * one tile per workgroup, 2 = 128x128 tiles, 3 = plain 256x256 tiles, 4 = persistent pipelined 256x256 tiles (bf16
- * output, N % 8 == 0, K % 128 == 0, K > 256; other calls fall back to 1). Process-wide; meant for tests and tuning, it has no counterpart in the reference
+ * output, N % 8 == 0, K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's
+ * tile to 192 / 256 rows / back to automatic. Process-wide; meant for tests and tuning, it has no counterpart in the reference
  * (whose tile is fixed at 128x128x64, csrc/gemm/fp8_matmul_bias.cu:426-429).
  */
 int q8_gemm_set_config(int cfg);

@@ -1,6 +1,8 @@
 // Persistent form of the pipelined 256x256 GEMM tile (gemm_pipe.h): one workgroup per CU walks over several output
 // tiles and the HBM->LDS copy pipeline runs straight across the tile boundaries.
 //
+//   * The tile is 256 x 256, or 192 x 256 (3 instead of 4 MFMA tiles per wave along M) when that spreads the work more
+//     evenly over the CUs.
 //   * Work item v (tile id + tiles * batch index) is handled by workgroup v % gridDim.x, which runs on XCD v % 8;
 //     the tile walk is the XCD-contiguous grouped walk of tile_of_block, so the L2 reuse is the same.
 //   * The compute side counts K stages globally (g); the copy side runs two stages ahead of it (gl = g + 2) with its
@@ -45,10 +47,14 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 
 // Requirements checked by the host: K % 128 == 0 and K > 256 (at least 3 whole stages per tile), N % 8 == 0,
 // M * K and N * K below 2^32 (32-bit source offsets), OUT == Q8_BF16.
-template <int IN, bool GELU>
+// MT = 32-row MFMA tiles per wave along M: the tile is 64 MT x 256, i.e. 256 x 256 (MT = 4) or 192 x 256 (MT = 3, for
+// problems whose 256-row tiles do not divide evenly over the CUs).
+template <int IN, bool GELU, int MT>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    constexpr int BM = kPipeBM, BN = kPipeBN;
+    constexpr int BM = 64 * MT, BN = kPipeBN;
+    constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
+    constexpr int NT = 2 * MT;     // MFMA tiles per K half
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wave_m = wave >> 2, wave_n = wave & 3;
     const int M = p.M, N = p.N, K = p.K;
@@ -67,12 +73,12 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
     };
 
     // ---- copy side ------------------------------------------------------------------------------------------
-    // A stage is 64 row groups of 1 KiB (8 rows x 128 B): groups 0..31 hold A, 32..63 B. Wave w copies groups
-    // w, w+8, w+16, w+24 of each; lane (lane/8, lane%8) fills row 8 q + lane/8, physical chunk lane%8, from logical
+    // A stage is 8 MT + 32 row groups of 1 KiB (8 rows x 128 B): the first 8 MT hold A, the others B. Wave w copies
+    // groups w, w+8, ... of each; lane (lane/8, lane%8) fills row 8 q + lane/8, physical chunk lane%8, from logical
     // chunk (lane%8) ^ ((row >> 1) & 7).
     // (the swizzle term is the same for the 8 row groups of a wave: their rows differ by multiples of 64).
     // Sources are a uniform base per operand plus a 32-bit byte offset per lane and row group.
-    uint32_t off[8];
+    uint32_t off[NCOPY];
     const uint8_t* baseA;
     const uint8_t* baseB;
     const uint32_t kchunk = 16 * ((lane & 7) ^ ((4 * wave + (lane >> 4)) & 7));
@@ -81,9 +87,9 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         baseA = p.A + (size_t)it.za * M * K;
         baseB = p.B + (size_t)it.zb * N * K;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int rho = 8 * (wave + 8 * (i & 3)) + (lane >> 3);
-            if (i < 4) {
+        for (int i = 0; i < NCOPY; ++i) {
+            const int rho = 8 * (wave + 8 * (i < MT ? i : i - MT)) + (lane >> 3);
+            if (i < MT) {
                 int m = it.m0 + rho;
                 m = m < M ? m : M - 1;
                 off[i] = (uint32_t)m * (uint32_t)K + kchunk;
@@ -98,7 +104,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
     auto set_src_zeros = [&]() {  // past the last tile: every lane reads the same 16 zero bytes
         baseA = baseB = reinterpret_cast<const uint8_t*>(g_zero16);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) off[i] = 0;
+        for (int i = 0; i < NCOPY; ++i) off[i] = 0;
     };
     // two 4-byte-per-lane copies per wave: waves 0-3 bring sa and bias, waves 4-7 sb (twice, to keep the count equal)
     auto copy_params = [&](const Item& it, int buf, bool live) {
@@ -109,7 +115,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         float* d0;
         float* d1;
         if (wave < 4) {
-            const int m = (it.m0 + j < M) ? it.m0 + j : M - 1;
+            const int m = (it.m0 + j < M) ? it.m0 + j : M - 1;  // (rows past the tile's BM are copied but never read)
             const int n = (it.n0 + j < N) ? it.n0 + j : N - 1;
             g0 = p.sa + (size_t)it.za * M + m;
             g1 = (p.bias != nullptr) ? p.bias + n : reinterpret_cast<const float*>(g_zero16);
@@ -127,11 +133,11 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                                          (__attribute__((address_space(3))) void*)d1, 4, 0, 0);
     };
     int l_item = 0, l_k = 0, gl = 0;  // copy side: item, stage inside the item, global stage count
-    auto issue_copy = [&](int i) {    // copy instruction i (0..7) of the copy side's current stage
+    auto issue_copy = [&](int i) {    // copy instruction i (0 .. NCOPY-1) of the copy side's current stage
         uint8_t* base = lds + (gl & 1) * kPipeStageBytes;
         const uint32_t k0 = copy_live ? (uint32_t)l_k << 7 : 0u;
-        const int q = (i < 4 ? 0 : 32) + wave + 8 * (i & 3);
-        const uint8_t* g = (i < 4 ? baseA : baseB) + k0 + off[i];
+        const int q = (i < MT ? 8 * i : 8 * MT + 8 * (i - MT)) + wave;
+        const uint8_t* g = (i < MT ? baseA : baseB) + k0 + off[i];
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
                                          (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
     };
@@ -151,41 +157,41 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
 
     // ---- operand fetch addresses: [K half s][low / high chunk], byte offsets inside a stage
     const unsigned lds0 = lds_addr(lds);
-    const unsigned a_row = lds0 + wave_m * 16384 + (lane & 31) * 128;
-    const unsigned b_row = lds0 + 32768 + wave_n * 8192 + (lane & 31) * 128;
+    const unsigned a_row = lds0 + wave_m * (MT * 4096) + (lane & 31) * 128;
+    const unsigned b_row = lds0 + BM * 128 + wave_n * 8192 + (lane & 31) * 128;
     unsigned pc[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
         pc[s][0] = ((4 * s + 2 * (lane >> 5)) ^ (((lane & 31) >> 1) & 7)) * 16;
         pc[s][1] = pc[s][0] ^ 16;
     }
-    auto read_half = [&](PipeFrags& f, int stage, int s) {
+    auto read_half = [&](PipeFragsT<MT>& f, int stage, int s) {
         const unsigned so = (stage & 1) * kPipeStageBytes;
-        pipe_read_frags(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+        pipe_read_frags<0, MT>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
     };
 
     using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
-    acc_t acc[4][2];
+    acc_t acc[MT][2];
 
     // ---- prologue: stage 0 landed, stage 1 in flight, fragments of the first K half on their way
     Item cur = item_of(0);
     set_src(cur);
     copy_params(cur, 0, true);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) issue_copy(i);
+    for (int i = 0; i < NCOPY; ++i) issue_copy(i);
     advance_copy();
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int i = 0; i < 8; ++i) issue_copy(i);
+    for (int i = 0; i < NCOPY; ++i) issue_copy(i);
     advance_copy();
-    PipeFrags f0, f1;
+    PipeFragsT<MT> f0, f1;
     read_half(f0, 0, 0);
 
     int g = 0;  // compute side: global stage count
     for (int item = 0; item < count; ++item) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -199,12 +205,12 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             pipe_pin(f0);
             // First half. Once the second half of stage g is in registers everywhere (barrier 1), buffer g & 1 is
             // free and the copies of stage g+2 start to trickle out, one per MFMA tile.
-            pipe_mfma<IN>(f0, acc, [&](int j) {
-                if (j == 3) {
+            pipe_mfma<IN, MT>(f0, acc, [&](int j) {
+                if (j == MT - 1) {
                     pipe_wait_frags(f1);
                     __builtin_amdgcn_s_barrier();
                 }
-                if (j >= 4) issue_copy(j - 4);
+                if (j >= MT) issue_copy(j - MT);
             });
             __builtin_amdgcn_sched_barrier(0);
             pipe_pin(f1);
@@ -212,12 +218,12 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             // previous epilogue) must have completed; barrier 2 makes that true for every wave's copies, then the
             // first half of stage g+1 is fetched under the remaining MFMA tiles (after the epilogue at a tile's end).
             bool moved = false;
-            pipe_mfma<IN>(f1, acc, [&](int j) {
-                if (j < 4) issue_copy(4 + j);
+            pipe_mfma<IN, MT>(f1, acc, [&](int j) {
+                if (j < 4) issue_copy(MT + j);
                 if (j == 3) moved = advance_copy();
                 if (j == 4) {
-                    if (moved) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-                    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                    if (moved) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NCOPY + 2) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NCOPY) : "memory");
                     __builtin_amdgcn_s_barrier();
                     // the fragment registers are free for the epilogue after the last stage of a tile
                     if (!last) read_half(f0, g + 1, 0);
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         const unsigned stage_out = lds0 + kPersistStageOutOffset + wave * 2048;
         const unsigned par = lds0 + kPersistParOffset + (item & 1) * 3072;
         const size_t zc = (size_t)cur.z * M * N;
-        const int mw0 = cur.m0 + wave_m * 128, nw0 = cur.n0 + wave_n * 64;
+        const int mw0 = cur.m0 + wave_m * (32 * MT), nw0 = cur.n0 + wave_n * 64;
         v4i sbq[2][2][2], bq[2][2][2];  // [t][wp][low / high 4 columns]
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -250,7 +256,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             }
         float sam[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sam[i] = lds_read_b32(par + (wave_m * 128 + 32 * i + r32) * 4);
+        for (int i = 0; i < 4; ++i) sam[i] = lds_read_b32(par + (wave_m * (32 * MT) + 32 * (i < MT ? i : 0) + r32) * 4);
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(sam[0]), "+v"(sam[1]), "+v"(sam[2]), "+v"(sam[3]), "+v"(sbq[0][0][0]), "+v"(sbq[0][0][1]),
                        "+v"(sbq[0][1][0]), "+v"(sbq[0][1][1]), "+v"(sbq[1][0][0]), "+v"(sbq[1][0][1]), "+v"(sbq[1][1][0]),
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                      : "memory");
         uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < MT; ++i) {
             // the lane's 4 chunks of row 32 i + r32: chunk c = 4 t + 2 wp + h
             v4u outc[2][2];
 #pragma unroll

@@ -29,15 +29,17 @@ constexpr int kPipeParamOffset = kPipeStages * kPipeStageBytes;  // sa[256], sb[
 constexpr int kPipeLds = kPipeParamOffset + 3 * 256 * 4;
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-struct PipeFrags {
-    v4i a[4][2];  // 4 m-tiles x (low, high) 16-byte halves of the lane's 32 K bytes
-    v4i b[2][2];  // 2 n-tiles
+template <int MT = 4>
+struct PipeFragsT {
+    v4i a[MT][2];  // MT m-tiles x (low, high) 16-byte halves of the lane's 32 K bytes
+    v4i b[2][2];   // 2 n-tiles
 };
+using PipeFrags = PipeFragsT<4>;
 
 // a0/a1 (b0/b1): byte address of the lane's low/high 16-byte chunk in row (lane % 32) of the wave's first A (B)
 // tile; the following 32-row tiles are 4096 bytes apart.
-template <int SKIP = 0>  // tuning builds: 1 = leave the B fragments, 2 = leave the A fragments as they are
-__device__ __forceinline__ void pipe_read_frags(PipeFrags& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
+template <int SKIP = 0, int MT = 4>  // SKIP (tuning builds): 1 = leave the B fragments, 2 = leave the A fragments as they are
+__device__ __forceinline__ void pipe_read_frags(PipeFragsT<MT>& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
     if constexpr (SKIP != 1) {
         f.b[0][0] = lds_read_b128<0>(b0);
         f.b[0][1] = lds_read_b128<0>(b1);
@@ -55,36 +57,55 @@ __device__ __forceinline__ void pipe_read_frags(PipeFrags& f, unsigned a0, unsig
         f.a[1][1] = lds_read_b128<4096>(a1);
         f.a[2][0] = lds_read_b128<8192>(a0);
         f.a[2][1] = lds_read_b128<8192>(a1);
-        f.a[3][0] = lds_read_b128<12288>(a0);
-        f.a[3][1] = lds_read_b128<12288>(a1);
+        if constexpr (MT == 4) {
+            f.a[3][0] = lds_read_b128<12288>(a0);
+            f.a[3][1] = lds_read_b128<12288>(a1);
+        }
     }
 }
 
 // Wait until every LDS read issued so far has landed; the fragments pass through the statement so that no
 // MFMA consuming them can be scheduled above it.
-__device__ __forceinline__ void pipe_wait_frags(PipeFrags& f) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
-                   "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1])
-                 :
-                 : "memory");
+template <int MT>
+__device__ __forceinline__ void pipe_wait_frags(PipeFragsT<MT>& f) {
+    static_assert(MT == 3 || MT == 4, "wave tiles of 96 or 128 rows");
+    if constexpr (MT == 4) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                       "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1])
+                     :
+                     : "memory");
+    } else {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                       "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1])
+                     :
+                     : "memory");
+    }
 }
 
 // Compiler-level fence for the fragments: statements that consume them stay below this point, i.e. below the
 // LDS reads issued before it.
-__device__ __forceinline__ void pipe_pin(PipeFrags& f) {
-    asm volatile(""
-                 : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
-                   "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1]));
+template <int MT>
+__device__ __forceinline__ void pipe_pin(PipeFragsT<MT>& f) {
+    if constexpr (MT == 4) {
+        asm volatile(""
+                     : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                       "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1]));
+    } else {
+        asm volatile(""
+                     : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                       "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1]));
+    }
 }
 
-// The 8 (fp8) / 16 (int8) MFMAs of one K half. `between(j)` runs after the j-th of the 8 tiles with scheduling
+// The 2 MT (fp8) / 4 MT (int8) MFMAs of one K half. `between(j)` runs after the j-th of the 2 MT tiles with scheduling
 // fences around it, so that whatever it issues (one HBM->LDS copy) stays between two MFMAs: a wave that issued
 // all copies of a stage back to back would sit in the full vector-memory queue instead of feeding the matrix pipe.
-template <int IN, typename ACC, typename F>
-__device__ __forceinline__ void pipe_mfma(const PipeFrags& f, ACC (&acc)[4][2], F between) {
+template <int IN, int MT, typename ACC, typename F>
+__device__ __forceinline__ void pipe_mfma(const PipeFragsT<MT>& f, ACC (&acc)[MT][2], F between) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MT; ++i) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             if constexpr (IN == Q8_I8) {
@@ -235,7 +256,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
         // First half. Once the second half of stage k is in registers everywhere (barrier 1, after the 4th MFMA
         // tile), buffer k & 1 is free and the copies of stage k+2 start to trickle out, one per MFMA tile.
         if constexpr (!(DBG & 4)) {
-            pipe_mfma<IN>(f0, acc, [&](int j) {
+            pipe_mfma<IN, 4>(f0, acc, [&](int j) {
                 if (j == 3) {
                     pipe_wait_frags(f1);
                     if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
@@ -254,7 +275,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
         // stage k+1 is fetched under the remaining MFMA tiles. A copy has between 1 and 1.5 stages of MFMA
         // time to land.
         if constexpr (!(DBG & 4)) {
-            pipe_mfma<IN>(f1, acc, [&](int j) {
+            pipe_mfma<IN, 4>(f1, acc, [&](int j) {
                 if (j < 4) issue_load(k + 2, 4 + j);
                 if (j == 4) {
                     if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");

@@ -140,7 +140,8 @@ def test_mm_batch_broadcast(dev, tile_cfg):
 
 @pytest.mark.parametrize("case", [(1, 1, 4352, 4096, 384), (3, 1, 1100, 4600, 512), (1, 2, 2300, 2816, 640)])
 @pytest.mark.parametrize("fuse_gelu", [False, True])
-def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu):
+@pytest.mark.parametrize("tile_rows", [43, 44], ids=["rows192", "rows256"])
+def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu, tile_rows):
     """More 256x256 tiles than CUs (272, 270 and 198+ with ragged edges and batch broadcast), so that workgroups of the
     persistent kernel cross tile and batch boundaries; int8 operands make the accumulators exact, the epilogue
     is fp32 on both sides: at most one bf16 ulp."""
@@ -152,9 +153,11 @@ def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu):
     sb = torch.rand(bb * n, generator=g) * 2e-2 + 1e-3
     bias = torch.randn(n, generator=g)
     _set_cfg(4)
+    _set_cfg(tile_rows)  # force the 192- or the 256-row tile of the persistent kernel
     try:
         got = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.to(dev), sb.to(dev), fuse_gelu, torch.bfloat16)
     finally:
+        _set_cfg(40)
         _set_cfg(0)
     want = O.ref_q8_mm(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
     assert got.shape == want.shape
