@@ -182,12 +182,17 @@ int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* code
  *   [D-point FHT * scale if apply_fht] -> e4m3 codes [B, H, S, D]. scales == NULL: direct c10 cast (the
  *   reference's cast); otherwise one absmax scale per (token, head) to scales [B, H, S].
  *   D in {64, 128}; H * D in {64, 128, 256} or a multiple of 512 up to 4096.
+ * q8_attn_prep_qk_pair: the same for Q and K of a self-attention in one pass (same S, same tables, read once).
  * q8_attn_prep_v: e4m3 codes [B, H, D, S_pad] (Q8_V_DS), columns S..S_pad-1 zero, S_pad % 16 == 0;
  *   scales as above. D == 64.
  */
 int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
                     float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
                     q8_stream_t stream);
+int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
+                         const float* cos_t, const float* sin_t, void* codes_q, float* scales_q, void* codes_k,
+                         float* scales_k, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                         q8_stream_t stream);
 int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
                    int S_pad, q8_stream_t stream);
 
@@ -207,6 +212,16 @@ int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scal
 int q8_gemm(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C,
             int batch_a, int batch_b, int M, int N, int K, int in_dtype, int out_dtype, int fuse_gelu,
             q8_stream_t stream);
+
+/*
+ * q8_gemm with bf16 output and a residual connection: C = bf16(bf16(epi(...)) + residual), residual bf16 [batch, M, N].
+ * Fuses the element-wise addition the reference's blocks run after a projection
+ * (q8_kernels/blocks/ltx_transformer_block.py:41-51) into the epilogue; the two roundings are those of the separate
+ * addition. Runs on the persistent kernel only: N % 8 == 0, K % 128 == 0, K > 256 (Q8_ERR_SHAPE otherwise).
+ */
+int q8_gemm_residual(const void* A, const void* B, const float* bias, const float* sa, const float* sb,
+                     const void* residual, void* C, int batch_a, int batch_b, int M, int N, int K, int in_dtype,
+                     int fuse_gelu, q8_stream_t stream);
 
 /*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with

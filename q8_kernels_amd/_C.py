@@ -165,8 +165,10 @@ def _check_input(t, name):
         raise RuntimeError("%s must be contiguous" % name)
 
 
-def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who):
-    """Shape rules of csrc/gemm/q8_gemm_api.cpp:45-91: a [.,M,K], b [.,N,K], result always [batch,M,N]."""
+def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who, residual=None):
+    """Shape rules of csrc/gemm/q8_gemm_api.cpp:45-91: a [.,M,K], b [.,N,K], result always [batch,M,N].
+    residual (bfloat16, batch*M*N elements, bfloat16 output only): out = bf16(bf16(result) + residual), in the GEMM's
+    epilogue where the kernel supports the shape, otherwise by a separate addition with the same two roundings."""
     _check_input(a, "a")
     _check_input(b, "b")
     if a.dtype != in_dtype or b.dtype != in_dtype:
@@ -193,31 +195,49 @@ def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who):
         if bias.dtype != torch.float32 or bias.numel() != n:
             raise RuntimeError("%s: bias must be float32 with %d elements" % (who, n))
     out = torch.empty((batch, m, n), dtype=out_type, device=a.device)
+    if residual is not None:
+        _require_gpu(residual, "residual")
+        if out_type != torch.bfloat16 or residual.dtype != torch.bfloat16 or residual.numel() != out.numel():
+            raise RuntimeError("%s: residual must be bfloat16 with the output's element count, output bfloat16" % who)
+        residual = residual.contiguous()
+        fusable = n % 8 == 0 and k % 128 == 0 and k > 256 and m * k < 2 ** 32 and n * k < 2 ** 32 and residual.data_ptr() % 16 == 0
+        if fusable:
+            with torch.cuda.device(a.device):
+                _lib.check(_lib.lib().q8_gemm_residual(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(),
+                                                       b_scales.data_ptr(), residual.data_ptr(), out.data_ptr(), bs_a, bs_b,
+                                                       m, n, k, _DT[in_dtype], 1 if fuse_gelu else 0, _stream(a)))
+            return out
     with torch.cuda.device(a.device):
         _lib.check(_lib.lib().q8_gemm(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
                                       out.data_ptr(), bs_a, bs_b, m, n, k, _DT[in_dtype], _DT[out_type],
                                       1 if fuse_gelu else 0, _stream(a)))
+    if residual is not None:
+        out += residual.view(out.shape)
     return out
 
 
-def q8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+def q8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
+          residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:40-97."""
-    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm")
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm", residual)
 
 
-def q8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+def q8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
+               residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:100-164."""
-    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm_bias")
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm_bias", residual)
 
 
-def fp8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+def fp8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
+           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:167-224."""
-    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm")
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm", residual)
 
 
-def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None) -> torch.Tensor:
+def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:227-291."""
-    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias")
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias", residual)
 
 
 def q8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
@@ -378,6 +398,33 @@ def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = 
                                               _ptr(scales), b, s, num_heads, d, int(apply_fht), float(scale),
                                               Q8_BF16 if round_intermediate else Q8_F32, _stream(x)))
     return (codes, scales) if per_token_scales else codes
+
+
+def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
+                      sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
+                      per_token_scales: bool = False, *, round_intermediate: bool = True):
+    """attn_prep_qk for the Q and K projections of a self-attention in one pass (the tables are read once).
+    Returns (q_out, k_out), each what attn_prep_qk returns."""
+    q, b, s, d = _token_major(q, num_heads, "attn_prep_qk_pair")
+    k, bk, sk, dk = _token_major(k, num_heads, "attn_prep_qk_pair")
+    if (bk, sk, dk) != (b, s, d):
+        raise RuntimeError("attn_prep_qk_pair: q and k must have the same shape")
+    if (cos is None) != (sin is None):
+        raise RuntimeError("attn_prep_qk_pair: cos and sin come together")
+    if cos is not None:
+        for t in (cos, sin):
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != q.numel():
+                raise RuntimeError("attn_prep_qk_pair: tables must be float32 CUDA tensors of q's shape")
+        cos, sin = cos.contiguous(), sin.contiguous()
+    mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=q.device)  # noqa: E731
+    mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=q.device) if per_token_scales else None  # noqa: E731
+    cq, ck, sq, sk_ = mk(), mk(), mks(), mks()
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().q8_attn_prep_qk_pair(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), _ptr(cos), _ptr(sin),
+                                                   cq.data_ptr(), _ptr(sq), ck.data_ptr(), _ptr(sk_), b, s, num_heads, d,
+                                                   int(apply_fht), float(scale),
+                                                   Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))
+    return ((cq, sq), (ck, sk_)) if per_token_scales else (cq, ck)
 
 
 def attn_prep_v(x: torch.Tensor, num_heads: int, per_token_scales: bool = False):

@@ -41,9 +41,10 @@ class Fp8DiTBlock(nn.Module):
                 m.bias.data = (torch.randn(m.bias.shape, generator=g) * std).to(torch.bfloat16).float().to(dev)
         return self
 
-    def _lin(self, layer, x, fuse_gelu=False):
+    def _lin(self, layer, x, fuse_gelu=False, residual=None):
+        """layer(x) (+ residual, added in the GEMM's epilogue)."""
         return Q8F.linear.fp8_linear(x, layer.weight.data, layer.bias.data, None, layer.scales, False, x.dtype,
-                                     fuse_gelu=fuse_gelu)
+                                     fuse_gelu=fuse_gelu, residual=residual)
 
     def _norm_lin(self, norm, layer, x, fuse_gelu=False):
         """layer(norm(x)) with the norm and the e4m3 quantizer of the layer's input in one kernel."""
@@ -58,13 +59,13 @@ class Fp8DiTBlock(nn.Module):
         qkv = self._norm_lin(self.norm1, self.to_qkv, hidden)
         a = Q8F.fused.flash_attn_token_major(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], h,
                                              apply_qk_hadamard=True, freqs_cis=freqs_cis, out_dtype=bf16)
-        hidden = hidden + self._lin(self.to_out, a)
+        hidden = self._lin(self.to_out, a, residual=hidden)
         # cross-attention to the text states
         q2 = self._norm_lin(self.norm2, self.to_q2, hidden)
         k2, v2 = self._lin(self.to_k2, text), self._lin(self.to_v2, text)
         a = Q8F.fused.flash_attn_token_major(q2, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
                                              out_dtype=bf16)
-        hidden = hidden + self._lin(self.to_out2, a)
+        hidden = self._lin(self.to_out2, a, residual=hidden)
         # feed-forward
         up = self._norm_lin(self.norm3, self.ff_up, hidden, fuse_gelu=True)
-        return hidden + self._lin(self.ff_down, up)
+        return self._lin(self.ff_down, up, residual=hidden)

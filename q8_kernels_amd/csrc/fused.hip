@@ -133,80 +133,95 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
 // so a head is one group of LH consecutive lanes of one chunk and the D-point Hadamard transform is the register
 // stages plus log2(LH) lane stages. Codes go to the head-major layout [B, H, S, D] the attention kernel reads.
 // The options are uniform branches: cs != NULL rotates, scales != NULL quantizes per (token, head).
-template <int LANES, int CH, int LH>
+// PAIR: a second tensor (K next to Q of a self-attention) goes through the same steps with the same tables, which are
+// then read once: they are 8 of the 11 bytes per element that one tensor moves.
+template <int LANES, int CH, int LH, bool PAIR>
 __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
+                                                              const uint16_t* __restrict__ x2, int64_t x2_row_stride,
                                                               const float* __restrict__ cs, const float* __restrict__ sn,
                                                               uint8_t* __restrict__ codes, float* __restrict__ scales,
+                                                              uint8_t* __restrict__ codes2, float* __restrict__ scales2,
                                                               int64_t tokens, int S, int apply_fht, float scale,
                                                               int mid_bf16) {
     static_assert(LH <= LANES, "a head may not span tokens");
-    constexpr int DIM = LANES * CH * 8, D = LH * 8, H = DIM / D;
+    constexpr int DIM = LANES * CH * 8, D = LH * 8, H = DIM / D, NT = PAIR ? 2 : 1;
     const int t = threadIdx.x % LANES;
     const int64_t tok = (int64_t)blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES;
     if (tok >= tokens) return;  // no barrier below; the lane exchanges stay inside a head, i.e. inside a token
     const int64_t b = tok / S, s = tok - b * S;
-    const uint16_t* xr = x + tok * x_row_stride;
     auto mid8 = [&](float (&f)[8]) { if (mid_bf16) round_mid8<Q8_BF16>(f); };
 
-    float v[CH][8];
+    float v[NT][CH][8];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) load8<Q8_BF16>(xr, (c * LANES + t) * 8, v[c]);
+    for (int c = 0; c < CH; ++c) {
+        load8<Q8_BF16>(x + tok * x_row_stride, (c * LANES + t) * 8, v[0][c]);
+        if constexpr (PAIR) load8<Q8_BF16>(x2 + tok * x2_row_stride, (c * LANES + t) * 8, v[NT - 1][c]);
+    }
     if (cs != nullptr) {
         // interleaved pairs with per-element tables (csrc/ops/rope_cuda.cu:99-103)
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int64_t e = tok * DIM + (c * LANES + t) * 8;
-            float cv[8], sv[8], o[8];
+            float cv[8], sv[8];
             load8<Q8_F32>(cs, e, cv);
             load8<Q8_F32>(sn, e, sv);
 #pragma unroll
-            for (int i = 0; i < 8; i += 2) {
-                o[i] = v[c][i] * cv[i] - v[c][i + 1] * sv[i];
-                o[i + 1] = v[c][i + 1] * cv[i + 1] + v[c][i] * sv[i + 1];
-            }
-            mid8(o);
+            for (int n = 0; n < NT; ++n) {
+                float o[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = o[i];
+                for (int i = 0; i < 8; i += 2) {
+                    o[i] = v[n][c][i] * cv[i] - v[n][c][i + 1] * sv[i];
+                    o[i + 1] = v[n][c][i + 1] * cv[i + 1] + v[n][c][i] * sv[i + 1];
+                }
+                mid8(o);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[n][c][i] = o[i];
+            }
         }
     }
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if (apply_fht) {
+    for (int n = 0; n < NT; ++n) {
+        uint8_t* const cout = n == 0 ? codes : codes2;
+        float* const sout = n == 0 ? scales : scales2;
 #pragma unroll
-            for (int st = 1; st < 8; st <<= 1) {
+        for (int c = 0; c < CH; ++c) {
+            if (apply_fht) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if ((i & st) == 0) {
-                        const float a0 = v[c][i], b0 = v[c][i + st];
-                        v[c][i] = a0 + b0;
-                        v[c][i + st] = a0 - b0;
+                for (int st = 1; st < 8; st <<= 1) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if ((i & st) == 0) {
+                            const float a0 = v[n][c][i], b0 = v[n][c][i + st];
+                            v[n][c][i] = a0 + b0;
+                            v[n][c][i + st] = a0 - b0;
+                        }
                     }
                 }
+                fht_lane_stage<1>(v[n][c], (unsigned)(t & 1) << 31);
+                fht_lane_stage<2>(v[n][c], (unsigned)(t & 2) << 30);
+                fht_lane_stage<4>(v[n][c], 0u);
+                if constexpr (LH > 8) fht_lane_stage<8>(v[n][c], 0u);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[n][c][i] *= scale;
             }
-            fht_lane_stage<1>(v[c], (unsigned)(t & 1) << 31);
-            fht_lane_stage<2>(v[c], (unsigned)(t & 2) << 30);
-            fht_lane_stage<4>(v[c], 0u);
-            if constexpr (LH > 8) fht_lane_stage<8>(v[c], 0u);
+            const int h = (c * LANES + t) / LH;
+            const int64_t orow = (b * H + h) * S + s;
+            v2i w;
+            if (sout != nullptr) {
+                float amax = 0.f;
+                mid8(v[n][c]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] *= scale;
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[n][c][i]));
+                amax = group_max<LH>(amax);
+                const float ratio = quant_ratio<Q8_E4M3>(amax);
+                if ((t % LH) == 0) sout[orow] = quant_scale<Q8_E4M3>(amax, ratio, 0);
+                w = quant_codes8<Q8_E4M3>(v[n][c], ratio, 0);
+            } else {
+                w[0] = (int)pack4_e4m3_c10(v[n][c][0], v[n][c][1], v[n][c][2], v[n][c][3]);
+                w[1] = (int)pack4_e4m3_c10(v[n][c][4], v[n][c][5], v[n][c][6], v[n][c][7]);
+            }
+            *reinterpret_cast<v2i*>(cout + orow * D + (t % LH) * 8) = w;
         }
-        const int h = (c * LANES + t) / LH;
-        const int64_t orow = (b * H + h) * S + s;
-        v2i w;
-        if (scales != nullptr) {
-            float amax = 0.f;
-            mid8(v[c]);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[c][i]));
-            amax = group_max<LH>(amax);
-            const float ratio = quant_ratio<Q8_E4M3>(amax);
-            if ((t % LH) == 0) scales[orow] = quant_scale<Q8_E4M3>(amax, ratio, 0);
-            w = quant_codes8<Q8_E4M3>(v[c], ratio, 0);
-        } else {
-            w[0] = (int)pack4_e4m3_c10(v[c][0], v[c][1], v[c][2], v[c][3]);
-            w[1] = (int)pack4_e4m3_c10(v[c][4], v[c][5], v[c][6], v[c][7]);
-        }
-        *reinterpret_cast<v2i*>(codes + orow * D + (t % LH) * 8) = w;
     }
 }
 
@@ -335,33 +350,40 @@ extern "C" int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w,
     return launch_status("q8_rmsnorm_quant_rows");
 }
 
-extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
-                               float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
-                               q8_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (B < 0 || S < 0 || H <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: B %d S %d H %d", B, S, H);
-    if (D != 64 && D != 128) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: head dim %d (want 64 or 128)", D);
+static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_stride, const void* x2, int64_t x2_row_stride,
+                             const float* cos_t, const float* sin_t, void* codes, float* scales, void* codes2,
+                             float* scales2, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                             hipStream_t stream) {
+    const bool pair = x2 != nullptr;
+    if (B < 0 || S < 0 || H <= 0) return fail(Q8_ERR_SHAPE, "%s: B %d S %d H %d", who, B, S, H);
+    if (D != 64 && D != 128) return fail(Q8_ERR_SHAPE, "%s: head dim %d (want 64 or 128)", who, D);
     const int64_t dim = (int64_t)H * D;
     const bool small = dim == 64 || dim == 128 || dim == 256;
     if (!small && (dim % 512 != 0 || dim > 4096))
-        return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: H * D = %lld must be 64, 128, 256 or a multiple of 512 up to 4096", (long long)dim);
+        return fail(Q8_ERR_SHAPE, "%s: H * D = %lld must be 64, 128, 256 or a multiple of 512 up to 4096", who, (long long)dim);
     if ((int64_t)B * S == 0) return Q8_OK;
-    if (!x || !codes) return fail(Q8_ERR_NULL, "q8_attn_prep_qk: null pointer");
-    if ((cos_t == nullptr) != (sin_t == nullptr)) return fail(Q8_ERR_NULL, "q8_attn_prep_qk: cos and sin come together");
-    if (x_row_stride < dim || x_row_stride % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: row stride %lld", (long long)x_row_stride);
-    if (!aligned16(x) || (cos_t && (!aligned16(cos_t) || !aligned16(sin_t))) || (reinterpret_cast<uintptr_t>(codes) % 8))
-        return fail(Q8_ERR_ALIGN, "q8_attn_prep_qk: x and tables must be 16-byte aligned, codes 8-byte aligned");
-    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32) return fail(Q8_ERR_DTYPE, "q8_attn_prep_qk: intermediate dtype %d", mid_dtype);
+    if (!x || !codes || (pair && !codes2)) return fail(Q8_ERR_NULL, "%s: null pointer", who);
+    if ((cos_t == nullptr) != (sin_t == nullptr)) return fail(Q8_ERR_NULL, "%s: cos and sin come together", who);
+    if (pair && ((scales == nullptr) != (scales2 == nullptr))) return fail(Q8_ERR_NULL, "%s: both scale outputs or none", who);
+    if (x_row_stride < dim || x_row_stride % 8 != 0 || (pair && (x2_row_stride < dim || x2_row_stride % 8 != 0)))
+        return fail(Q8_ERR_SHAPE, "%s: row stride %lld / %lld", who, (long long)x_row_stride, (long long)x2_row_stride);
+    if (!aligned16(x) || (pair && !aligned16(x2)) || (cos_t && (!aligned16(cos_t) || !aligned16(sin_t))) ||
+        (reinterpret_cast<uintptr_t>(codes) % 8) || (pair && (reinterpret_cast<uintptr_t>(codes2) % 8)))
+        return fail(Q8_ERR_ALIGN, "%s: x and tables must be 16-byte aligned, codes 8-byte aligned", who);
+    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32) return fail(Q8_ERR_DTYPE, "%s: intermediate dtype %d", who, mid_dtype);
     const int64_t tokens = (int64_t)B * S;
     const int lanes = small ? (int)(dim / 8) : 64;
     const int64_t grid = (tokens + (kBlock / lanes) - 1) / (kBlock / lanes);
-    if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_attn_prep_qk: too many tokens");
-#define PREP_LAUNCH(LANES, CH, LH)                                                                                  \
-    hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH>), dim3((unsigned)grid), dim3(kBlock), 0, stream,         \
-                       static_cast<const uint16_t*>(x), x_row_stride, cos_t, sin_t, static_cast<uint8_t*>(codes), \
-                       scales, tokens, S, apply_fht, scale, mid_dtype == Q8_BF16 ? 1 : 0)
+    if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "%s: too many tokens", who);
+#define PREP_ARGS                                                                                                        \
+    static_cast<const uint16_t*>(x), x_row_stride, static_cast<const uint16_t*>(x2), x2_row_stride, cos_t, sin_t,        \
+        static_cast<uint8_t*>(codes), scales, static_cast<uint8_t*>(codes2), scales2, tokens, S, apply_fht, scale,       \
+        mid_dtype == Q8_BF16 ? 1 : 0
+#define PREP_LAUNCH(LANES, CH, LH)                                                                                       \
+    if (pair) hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH, true>), dim3((unsigned)grid), dim3(kBlock), 0, stream, PREP_ARGS); \
+    else hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH, false>), dim3((unsigned)grid), dim3(kBlock), 0, stream, PREP_ARGS)
 #define PREP_D(LANES, CH) \
-    if (D == 64) PREP_LAUNCH(LANES, CH, 8); else PREP_LAUNCH(LANES, CH, 16)
+    if (D == 64) { PREP_LAUNCH(LANES, CH, 8); } else { PREP_LAUNCH(LANES, CH, 16); }
     switch (dim) {
         case 64: PREP_LAUNCH(8, 1, 8); break;
         case 128: PREP_D(16, 1); break;
@@ -377,7 +399,24 @@ extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float*
     }
 #undef PREP_D
 #undef PREP_LAUNCH
-    return launch_status("q8_attn_prep_qk");
+#undef PREP_ARGS
+    return launch_status(who);
+}
+
+extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
+                               float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                               q8_stream_t stream_) {
+    return attn_prep_qk_impl("q8_attn_prep_qk", x, x_row_stride, nullptr, 0, cos_t, sin_t, codes, scales, nullptr, nullptr, B, S,
+                             H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
+}
+
+extern "C" int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
+                                    const float* cos_t, const float* sin_t, void* codes_q, float* scales_q, void* codes_k,
+                                    float* scales_k, int B, int S, int H, int D, int apply_fht, float scale,
+                                    int mid_dtype, q8_stream_t stream_) {
+    if (!xk) return fail(Q8_ERR_NULL, "q8_attn_prep_qk_pair: null pointer");
+    return attn_prep_qk_impl("q8_attn_prep_qk_pair", xq, xq_row_stride, xk, xk_row_stride, cos_t, sin_t, codes_q, scales_q,
+                             codes_k, scales_k, B, S, H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,

@@ -215,14 +215,14 @@ static int persist_cus() {
     return cus;
 }
 
-template <int IN, bool GELU, int MT>
+template <int IN, bool GELU, int MT, bool RES>
 static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     constexpr int BM = 64 * MT;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     const long total = (long)tiles_m * tiles_n * batch;
     if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
-    auto kern = gemm_persist_kernel<IN, GELU, MT>;
+    auto kern = gemm_persist_kernel<IN, GELU, MT, RES>;
     static thread_local bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPersistLds) !=
@@ -249,7 +249,14 @@ static int launch_persist(const GemmParams& p, hipStream_t stream) {
         return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? 1.0 : 1.2);
     };
     const bool small = g_persist_mt == 3 || (g_persist_mt == 0 && cost(192) < cost(256));
-    return small ? launch_persist_mt<IN, GELU, 3>(p, stream) : launch_persist_mt<IN, GELU, 4>(p, stream);
+    if (p.residual != nullptr)
+        return small ? launch_persist_mt<IN, GELU, 3, true>(p, stream) : launch_persist_mt<IN, GELU, 4, true>(p, stream);
+    return small ? launch_persist_mt<IN, GELU, 3, false>(p, stream) : launch_persist_mt<IN, GELU, 4, false>(p, stream);
+}
+
+// shapes the persistent kernel takes (its output is bf16)
+static bool persist_eligible(const GemmParams& p) {
+    return (p.N % 8) == 0 && p.K > 256 && (p.K % 128) == 0 && (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32);
 }
 
 template <int IN, int OUT, bool GELU>
@@ -257,9 +264,7 @@ static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
     const long big_tiles = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.batch_a > p.batch_b ? p.batch_a : p.batch_b);
     const bool big = g_force_cfg == 1 || g_force_cfg == 4 || (g_force_cfg == 0 && big_tiles >= 192);
     if constexpr (OUT == Q8_BF16) {
-        if (big && g_force_cfg != 1 && (p.N % 8) == 0 && p.K > 256 && (p.K % 128) == 0 && (uint64_t)p.M * p.K < (1ull << 32) &&
-            (uint64_t)p.N * p.K < (1ull << 32))
-            return launch_persist<IN, GELU>(p, stream);
+        if (big && g_force_cfg != 1 && persist_eligible(p)) return launch_persist<IN, GELU>(p, stream);
     }
     if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
     if (g_force_cfg == 3) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);
@@ -310,6 +315,23 @@ extern "C" int q8_gemm(const void* A, const void* B, const float* bias, const fl
         if (out_dtype == Q8_BF16) { Q8_GEMM_CASE(Q8_E4M3, Q8_BF16); } else { Q8_GEMM_CASE(Q8_E4M3, Q8_E4M3); }
     }
 #undef Q8_GEMM_CASE
+}
+
+extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias, const float* sa, const float* sb,
+                                const void* residual, void* C, int batch_a, int batch_b, int M, int N, int K, int in_dtype,
+                                int fuse_gelu, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int st = check_gemm("q8_gemm_residual", A, B, C, batch_a, batch_b, M, N, K)) return st;
+    if (!sa || !sb || !residual) return fail(Q8_ERR_NULL, "q8_gemm_residual: scales and residual are required");
+    if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_gemm_residual: input dtype %d", in_dtype);
+    if ((reinterpret_cast<uintptr_t>(C) % 16) || (reinterpret_cast<uintptr_t>(residual) % 16))
+        return fail(Q8_ERR_ALIGN, "q8_gemm_residual: C and residual must be 16-byte aligned");
+    GemmParams p{static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), bias, sa, sb, C, batch_a, batch_b, M, N, K};
+    p.residual = residual;
+    if (!persist_eligible(p))
+        return fail(Q8_ERR_SHAPE, "q8_gemm_residual: needs N %% 8 == 0 and K a multiple of 128 above 256 (N %d K %d)", N, K);
+    if (in_dtype == Q8_I8) return fuse_gelu ? launch_persist<Q8_I8, true>(p, stream) : launch_persist<Q8_I8, false>(p, stream);
+    return fuse_gelu ? launch_persist<Q8_E4M3, true>(p, stream) : launch_persist<Q8_E4M3, false>(p, stream);
 }
 
 extern "C" int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int K, q8_stream_t stream_) {

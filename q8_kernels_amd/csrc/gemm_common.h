@@ -14,6 +14,7 @@ struct GemmParams {
     void* C;
     int batch_a, batch_b;
     int M, N, K;
+    const void* residual = nullptr;  // bf16 [batch, M, N] added to the rounded bf16 result (persistent kernel only)
 };
 
 __device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0};

@@ -49,12 +49,13 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 // M * K and N * K below 2^32 (32-bit source offsets), OUT == Q8_BF16.
 // MT = 32-row MFMA tiles per wave along M: the tile is 64 MT x 256, i.e. 256 x 256 (MT = 4) or 192 x 256 (MT = 3, for
 // problems whose 256-row tiles do not divide evenly over the CUs).
-template <int IN, bool GELU, int MT>
+// RES: C = bf16(bf16(result) + residual), the residual connection around a projection (two roundings, as the separate
+// element-wise addition of the two bf16 tensors gives).
+template <int IN, bool GELU, int MT, bool RES>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     constexpr int BM = 64 * MT, BN = kPipeBN;
     constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
-    constexpr int NT = 2 * MT;     // MFMA tiles per K half
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wave_m = wave >> 2, wave_n = wave & 3;
     const int M = p.M, N = p.N, K = p.K;
@@ -265,8 +266,22 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                      :
                      : "memory");
         uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
+        const uint16_t* const rbase = reinterpret_cast<const uint16_t*>(p.residual) + zc;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
+            // the residual rows this lane will store in the four rounds of this MFMA tile: fetched now, used after the
+            // arithmetic below
+            v4u res[2][2];
+            if constexpr (RES) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int m = mw0 + 32 * i + 16 * half + 8 * j + (lane_e >> 3);
+                        const int n = nw0 + (lane_e & 7) * 8;
+                        res[half][j] = (m < M && n < N) ? *reinterpret_cast<const v4u*>(rbase + (size_t)m * N + n) : v4u{0u, 0u, 0u, 0u};
+                    }
+            }
             // the lane's 4 chunks of row 32 i + r32: chunk c = 4 t + 2 wp + h
             v4u outc[2][2];
 #pragma unroll
@@ -303,6 +318,16 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     w[j] = lds_read_b128<0>(stage_out + row * 128 + (((lane_e & 7) ^ ((row >> 1) & 7)) * 16));
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0]), "+v"(w[1]) : : "memory");
+                if constexpr (RES) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e];
+                            w[j][e] = (int)pack2_bf16(__uint_as_float(a << 16) + __uint_as_float(r << 16),
+                                                      __uint_as_float(a & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
+                        }
+                }
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int m = mw0 + 32 * i + 16 * half + 8 * j + (lane_e >> 3);

@@ -55,8 +55,11 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
-    qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
-    kc = _C.attn_prep_qk(k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+    if q.shape == k.shape:  # self-attention: one pass over both, the tables are read once
+        qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+    else:
+        qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+        kc = _C.attn_prep_qk(k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
     vc = _C.attn_prep_v(v, num_heads, per_token_scales)
     if per_token_scales:
         (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc

@@ -92,7 +92,7 @@ def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = N
 
 # ----------------------------------------------------------------------------- fp8
 
-def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu):
+def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual=None):
     assert (is_16bit(a) and scale_a is None) or (a.dtype == _FP8 and scale_a is not None), \
         "FP8LinearFunc: a dtype missmatch"
     assert (is_16bit(b) and scale_b is None) or (b.dtype == _FP8 and scale_b is not None), \
@@ -109,9 +109,9 @@ def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gel
     if is_16bit(b):
         b, scale_b = quant(b)
     if bias is not None:
-        out = _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
     else:
-        out = _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
     return out, b, scale_b
 
 
@@ -138,13 +138,14 @@ class FP8LinearFunc(torch.autograd.Function):
 def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
                scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
                use_hadamard: bool = False, out_dtype: Optional[torch.dtype] = None, *,
-               fuse_gelu: bool = False) -> torch.Tensor:
+               fuse_gelu: bool = False, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [..., K] x b [N, K] -> [batch, M, N] through the fp8 GEMM; out_dtype must be 16-bit.
 
-    `fuse_gelu` (keyword only, default False = the reference's behaviour) applies tanh-GELU in the epilogue."""
-    if _needs_grad(a) and not fuse_gelu:
+    Keyword-only extensions (defaults = the reference's behaviour): `fuse_gelu` applies tanh-GELU in the epilogue;
+    `residual` (bfloat16, the output's shape) returns `residual + linear(a)` with the addition done in the epilogue."""
+    if _needs_grad(a) and not fuse_gelu and residual is None:
         return FP8LinearFunc.apply(a, b, bias, scale_a, scale_b, out_dtype, use_hadamard)
-    return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu)[0]
+    return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual)[0]
 
 
 # ----------------------------------------------------------------------------- int8 base weight + 16-bit LoRA

@@ -131,6 +131,29 @@ def test_attn_prep_qk(dev, shape, rope, fht, scaled):
         assert_bit_equal(got, want, "codes")
 
 
+@pytest.mark.parametrize("shape", [(2, 70, 8, 64), (1, 33, 32, 64), (2, 7, 2, 128)])
+@pytest.mark.parametrize("rope", [False, True])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_qk_pair_equals_two_single_calls(dev, shape, rope, scaled):
+    b, s, h, d = shape
+    g = torch.Generator().manual_seed(s * 7 + h)
+    qkv = (torch.randn(b, s, 3 * h * d, generator=g) * 1.5).to(BF16).to(dev)
+    q, k = qkv[..., :h * d], qkv[..., h * d:2 * h * d]
+    cos = sin = None
+    if rope:
+        ang = torch.rand(b, s, h * d // 2, generator=g) * 6.28
+        cos, sin = torch.cos(ang).repeat_interleave(2, -1).to(dev), torch.sin(ang).repeat_interleave(2, -1).to(dev)
+    pq, pk = _C().attn_prep_qk_pair(q, k, h, cos, sin, True, 0.125, scaled)
+    sq, sk = _C().attn_prep_qk(q, h, cos, sin, True, 0.125, scaled), _C().attn_prep_qk(k, h, cos, sin, True, 0.125, scaled)
+    if scaled:
+        for got, want in ((pq, sq), (pk, sk)):
+            assert_bit_equal(got[0], want[0], "codes")
+            assert_bit_equal(got[1], want[1], "scales")
+    else:
+        assert_bit_equal(pq, sq, "q codes")
+        assert_bit_equal(pk, sk, "k codes")
+
+
 def test_attn_prep_qk_strided_slice_of_fused_projection(dev):
     g = torch.Generator().manual_seed(77)
     qkv = torch.randn(2, 50, 3 * 2048, generator=g).to(BF16)

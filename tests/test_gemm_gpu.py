@@ -168,6 +168,28 @@ def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu, tile_r
     assert float((diff > 0).float().mean()) < (0.02 if fuse_gelu else 0.002)
 
 
+@pytest.mark.parametrize("case", [(1, 1, 2300, 2816, 640), (2, 1, 1100, 4608, 384), (1, 1, 200, 264, 208)])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu):
+    """out = residual + linear(a): the fused epilogue (first two cases, persistent kernel) and the fallback (last case,
+    K not a multiple of 128) both give the bits of the bf16 GEMM followed by a bf16 addition."""
+    ba, bb, m, n, k = case
+    g = torch.Generator().manual_seed(m + n + 1)
+    a = (_rand_i8(g, ba, m, k) if ba > 1 else _rand_i8(g, m, k)).to(dev)
+    b = _rand_i8(g, n, k).to(dev)
+    sa = (torch.rand(ba * m, generator=g) * 2e-3 + 1e-4).to(dev)
+    sb = (torch.rand(n, generator=g) * 2e-2 + 1e-3).to(dev)
+    bias = torch.randn(n, generator=g).to(dev)
+    res = torch.randn(ba, m, n, generator=g).to(torch.bfloat16).to(dev)
+    _set_cfg(4)
+    try:
+        plain = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
+        fused = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16, residual=res)
+    finally:
+        _set_cfg(0)
+    assert_bit_equal(fused, plain + res, "residual epilogue")
+
+
 # ------------------------------------------------------------------ fp8 at the benchmark shapes
 
 @pytest.mark.parametrize("m", [2048, 6144])

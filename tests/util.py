@@ -35,5 +35,5 @@ def bf16_ulp(x: torch.Tensor) -> torch.Tensor:
 
 
 def cosine(a: torch.Tensor, b: torch.Tensor) -> float:
-    a, b = a.double().flatten(), b.double().flatten()
+    a, b = a.detach().double().flatten(), b.detach().double().flatten()
     return float((a @ b) / (a.norm() * b.norm()).clamp_min(1e-300))
