@@ -168,6 +168,23 @@ def _extras(dev, steps, warmup):
     with torch.no_grad():
         t, _ = _time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
     out["dit_block"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12, "shape": "tokens [2,6144,2048], text [2,128,2048]"}
+    del blk
+    # the reference's own block: AdaLN-modulated LTXTransformerBlock on int8 (Hadamard-rotated) Q8Linear layers
+    from q8_kernels_amd.blocks import LTXTransformerBlock
+    from q8_kernels_amd.modules import Q8Linear
+    ltx = LTXTransformerBlock(2048, 32, 64, 2048, bias=True, use_rope=True, norm_affine=False).to(dev)
+    for m in ltx.modules():
+        if isinstance(m, Q8Linear):
+            wq = (torch.randn(m.weight.shape, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+            m.weight.data, m.scales.data = _C.fht_quant(wq, wq.shape[-1] ** -0.5, None)
+            m.bias.data = (torch.randn(m.bias.shape, generator=g) * 0.02).to(dev)
+            del wq
+    timestep = (torch.randn(2, 1, 6 * 2048, generator=g) * 0.3).to(dev)
+    with torch.no_grad():
+        t, _ = _time(lambda: ltx(hidden, (cosf, sinf), None, text, lens, timestep, attn_type="q8_kernels"),
+                     max(3, steps // 4), max(1, warmup // 2))
+    out["ltx_transformer_block_int8"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12,
+                                         "shape": "tokens [2,6144,2048], text [2,128,2048], int8 linears, fp8 attention"}
     return out
 
 

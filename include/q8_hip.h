@@ -158,7 +158,8 @@ int q8_rmsnorm_backward(const void* y, int y_dtype, const float* rstd, const voi
 /*
  * Fused row kernels: launch sequences of the reference with the 16-bit tensor between two kernels kept in
  * registers. Each intermediate value is rounded to `mid_dtype` exactly where the unfused sequence stores it
- * (mid_dtype = Q8_BF16 gives the same bits as the separate calls; Q8_F32 skips that rounding).
+ * (mid_dtype = Q8_BF16 gives the same bits as the separate calls; Q8_F32 skips that rounding; Q8_E4M3, for an
+ * E4M3 input, is the e4m3 intermediate that hadamard_transform's default output type produces).
  *
  * q8_fht_quant_rows: codes, scales = quant(FHT(x) * fht_scale). The prologue of the int8 linear layer,
  *   hadamard_transform followed by quantize (q8_kernels/functional/linear.py:30-31), = q8_fht then q8_quant_rows.
@@ -178,7 +179,9 @@ int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* code
  * Replaces the torch glue of flash_attn_func (q8_kernels/functional/flash_attention.py:38-55: transpose, pad,
  * cast, hadamard_transform) and the RoPE in front of it (q8_kernels/modules/attention.py:84-87).
  *
- * q8_attn_prep_qk: per token and head: [RoPE with tables cos, sin fp32 [B*S, H*D], both NULL = none] ->
+ * q8_attn_prep_qk: per token: [RMSNorm over the H*D row with fp32 weights norm_w [H*D], no epsilon (the qk-norm of
+ *   q8_kernels/modules/attention.py:67-77), NULL = none] -> per head: [RoPE with tables cos, sin fp32 [B*S, H*D],
+ *   both NULL = none] ->
  *   [D-point FHT * scale if apply_fht] -> e4m3 codes [B, H, S, D]. scales == NULL: direct c10 cast (the
  *   reference's cast); otherwise one absmax scale per (token, head) to scales [B, H, S].
  *   D in {64, 128}; H * D in {64, 128, 256} or a multiple of 512 up to 4096.
@@ -186,13 +189,13 @@ int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* code
  * q8_attn_prep_v: e4m3 codes [B, H, D, S_pad] (Q8_V_DS), columns S..S_pad-1 zero, S_pad % 16 == 0;
  *   scales as above. D == 64.
  */
-int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
-                    float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* norm_w, const float* cos_t, const float* sin_t,
+                    void* codes, float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
                     q8_stream_t stream);
 int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
-                         const float* cos_t, const float* sin_t, void* codes_q, float* scales_q, void* codes_k,
-                         float* scales_k, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
-                         q8_stream_t stream);
+                         const float* norm_wq, const float* norm_wk, const float* cos_t, const float* sin_t,
+                         void* codes_q, float* scales_q, void* codes_k, float* scales_k, int B, int S, int H, int D,
+                         int apply_fht, float scale, int mid_dtype, q8_stream_t stream);
 int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
                    int S_pad, q8_stream_t stream);
 

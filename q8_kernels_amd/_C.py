@@ -322,9 +322,10 @@ def _quant_out(x2, out_type, who):
 
 
 def fht_quant(x: torch.Tensor, scale: float, out_type: Optional[torch.dtype] = None, *,
-              round_intermediate: bool = True) -> List[torch.Tensor]:
-    """tokenwise_quant(fast_hadamard_transform(x, scale, bfloat16), out_type) in one pass over x.
-    x bfloat16 or e4m3 with last dim a multiple of 8. Returns [codes(x.shape), scales(x.shape[:-1])]."""
+              round_intermediate: bool = True, mid_type: Optional[torch.dtype] = None) -> List[torch.Tensor]:
+    """tokenwise_quant(fast_hadamard_transform(x, scale, mid_type), out_type) in one pass over x.
+    x bfloat16 or e4m3 with last dim a multiple of 8; mid_type None -> bfloat16 (float8_e4m3fn is allowed for an
+    e4m3 x: what hadamard_transform returns for it by default). Returns [codes(x.shape), scales(x.shape[:-1])]."""
     _require_gpu(x, "x")
     if x.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
         raise RuntimeError("fht_quant: input must be bfloat16 or float8_e4m3fn")
@@ -335,7 +336,8 @@ def fht_quant(x: torch.Tensor, scale: float, out_type: Optional[torch.dtype] = N
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().q8_fht_quant_rows(x2.data_ptr(), _DT[x2.dtype], out.data_ptr(), _DT[out_type],
                                                 scales.data_ptr(), rows, dim, float(scale),
-                                                Q8_BF16 if round_intermediate else Q8_F32, 0, _stream(x)))
+                                                (_DT[mid_type] if mid_type is not None else Q8_BF16) if round_intermediate
+                                                else Q8_F32, 0, _stream(x)))
     return [out.reshape(shape), scales.reshape(shape[:-1])]
 
 
@@ -376,11 +378,20 @@ def _token_major(x, num_heads, who):
     return x, b, s, dim // num_heads
 
 
+def _norm_w(w, x):
+    if w is None:
+        return None
+    if w.dtype != torch.float32 or not w.is_cuda or w.numel() != x.shape[-1]:
+        raise RuntimeError("attn_prep_qk: norm weights must be float32 CUDA tensors with H*D elements")
+    return w.contiguous()
+
+
 def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
                  sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
-                 per_token_scales: bool = False, *, round_intermediate: bool = True):
+                 per_token_scales: bool = False, *, round_intermediate: bool = True,
+                 norm_weight: Optional[torch.Tensor] = None):
     """x [B, S, H*D] bfloat16 (a strided slice of a fused projection is fine) -> e4m3 [B, H, S, D]:
-    optional RoPE (tables fp32 [B, S, H*D]), head split, optional D-point Hadamard transform times `scale`,
+    optional RMSNorm over the H*D row (norm_weight fp32 [H*D], no epsilon), optional RoPE (tables fp32 [B, S, H*D]), head split, optional D-point Hadamard transform times `scale`,
     then the direct e4m3 cast, or per-(token, head) absmax quantization when per_token_scales
     (returns (codes, scales [B, H, S]) in that case)."""
     x, b, s, d = _token_major(x, num_heads, "attn_prep_qk")
@@ -394,7 +405,8 @@ def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = 
     codes = torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty((b, num_heads, s), dtype=torch.float32, device=x.device) if per_token_scales else None
     with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().q8_attn_prep_qk(x.data_ptr(), x.stride(1), _ptr(cos), _ptr(sin), codes.data_ptr(),
+        _lib.check(_lib.lib().q8_attn_prep_qk(x.data_ptr(), x.stride(1), _ptr(_norm_w(norm_weight, x)), _ptr(cos), _ptr(sin),
+                                              codes.data_ptr(),
                                               _ptr(scales), b, s, num_heads, d, int(apply_fht), float(scale),
                                               Q8_BF16 if round_intermediate else Q8_F32, _stream(x)))
     return (codes, scales) if per_token_scales else codes
@@ -402,7 +414,8 @@ def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = 
 
 def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
                       sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
-                      per_token_scales: bool = False, *, round_intermediate: bool = True):
+                      per_token_scales: bool = False, *, round_intermediate: bool = True,
+                      q_norm_weight: Optional[torch.Tensor] = None, k_norm_weight: Optional[torch.Tensor] = None):
     """attn_prep_qk for the Q and K projections of a self-attention in one pass (the tables are read once).
     Returns (q_out, k_out), each what attn_prep_qk returns."""
     q, b, s, d = _token_major(q, num_heads, "attn_prep_qk_pair")
@@ -420,7 +433,9 @@ def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Opt
     mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=q.device) if per_token_scales else None  # noqa: E731
     cq, ck, sq, sk_ = mk(), mk(), mks(), mks()
     with torch.cuda.device(q.device):
-        _lib.check(_lib.lib().q8_attn_prep_qk_pair(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), _ptr(cos), _ptr(sin),
+        _lib.check(_lib.lib().q8_attn_prep_qk_pair(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1),
+                                                   _ptr(_norm_w(q_norm_weight, q)), _ptr(_norm_w(k_norm_weight, k)),
+                                                   _ptr(cos), _ptr(sin),
                                                    cq.data_ptr(), _ptr(sq), ck.data_ptr(), _ptr(sk_), b, s, num_heads, d,
                                                    int(apply_fht), float(scale),
                                                    Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))

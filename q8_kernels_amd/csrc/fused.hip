@@ -1,7 +1,8 @@
 // Row kernels that fuse what the reference runs as separate launches with a 16-bit tensor in HBM between them:
 //   FHT -> token-wise quantizer            (the Q8Linear prologue, q8_kernels/functional/linear.py:30-31)
 //   RMSNorm -> token-wise quantizer        (norm followed by an 8-bit linear, q8_kernels/modules/attention.py:67-77)
-//   RoPE -> head split -> FHT -> e4m3      (the Q / K side of q8_kernels/functional/flash_attention.py:47-55)
+//   qk-RMSNorm -> RoPE -> head split -> FHT -> e4m3   (q8_kernels/modules/attention.py:67-87 and the Q / K side of
+//                                             q8_kernels/functional/flash_attention.py:47-55)
 //   head split -> e4m3 -> transpose        (the V side, flash_attention.py:38-45)
 // Every intermediate value is rounded to the dtype the unfused sequence would have stored (template MID), so the
 // results are the same bits as the separate kernels give.
@@ -138,6 +139,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
 template <int LANES, int CH, int LH, bool PAIR>
 __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
                                                               const uint16_t* __restrict__ x2, int64_t x2_row_stride,
+                                                              const float* __restrict__ nw, const float* __restrict__ nw2,
                                                               const float* __restrict__ cs, const float* __restrict__ sn,
                                                               uint8_t* __restrict__ codes, float* __restrict__ scales,
                                                               uint8_t* __restrict__ codes2, float* __restrict__ scales2,
@@ -156,6 +158,28 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
     for (int c = 0; c < CH; ++c) {
         load8<Q8_BF16>(x + tok * x_row_stride, (c * LANES + t) * 8, v[0][c]);
         if constexpr (PAIR) load8<Q8_BF16>(x2 + tok * x2_row_stride, (c * LANES + t) * 8, v[NT - 1][c]);
+    }
+    // qk-RMSNorm over the whole row (all heads) with fp32 weights, no epsilon: the sum runs in the order of
+    // rmsnorm_kernel (chunks, registers, lanes), so the result is the same bits (csrc/ops/rms_norm_cuda.cu:127-156)
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        const float* w = n == 0 ? nw : nw2;
+        if (w == nullptr) continue;
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += v[n][c][i] * v[n][c][i];
+        ss = group_sum<LANES>(ss);
+        const float rstd = 1.0f / sqrtf(ss * (1.0f / (float)DIM));
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float wv[8];
+            load8<Q8_F32>(w, (c * LANES + t) * 8, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[n][c][i] = (v[n][c][i] * rstd) * wv[i];
+            mid8(v[n][c]);
+        }
     }
     if (cs != nullptr) {
         // interleaved pairs with per-element tables (csrc/ops/rope_cuda.cu:99-103)
@@ -296,8 +320,8 @@ static int check_quant_args(const char* who, const void* x, int x_dtype, const v
     if (code_dtype != Q8_I8 && code_dtype != Q8_E4M3)
         return fail(Q8_ERR_DTYPE, "%s: code dtype %d (want I8 or E4M3)", who, code_dtype);
     if (x_dtype != Q8_BF16 && x_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "%s: input dtype %d (want BF16 or E4M3)", who, x_dtype);
-    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32)
-        return fail(Q8_ERR_DTYPE, "%s: intermediate dtype %d (want BF16 or F32)", who, mid_dtype);
+    if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32 && !(mid_dtype == Q8_E4M3 && x_dtype == Q8_E4M3))
+        return fail(Q8_ERR_DTYPE, "%s: intermediate dtype %d (want BF16 or F32, or E4M3 for an E4M3 input)", who, mid_dtype);
     if ((reinterpret_cast<uintptr_t>(x) % (x_dtype == Q8_BF16 ? 16 : 8)) || (reinterpret_cast<uintptr_t>(codes) % 8) ||
         (reinterpret_cast<uintptr_t>(scales) % 4))
         return fail(Q8_ERR_ALIGN, "%s: x must be 16-byte (bf16) or 8-byte (e4m3) aligned, codes 8-byte aligned", who);
@@ -309,6 +333,8 @@ static int check_quant_args(const char* who, const void* x, int x_dtype, const v
     else if (XD == Q8_BF16 && CD == Q8_E4M3 && MD == Q8_BF16) { constexpr int IN = Q8_BF16, OUT = Q8_E4M3, MID = Q8_BF16; __VA_ARGS__; } \
     else if (XD == Q8_BF16 && CD == Q8_I8) { constexpr int IN = Q8_BF16, OUT = Q8_I8, MID = Q8_F32; __VA_ARGS__; } \
     else if (XD == Q8_BF16) { constexpr int IN = Q8_BF16, OUT = Q8_E4M3, MID = Q8_F32; __VA_ARGS__; } \
+    else if (CD == Q8_I8 && MD == Q8_E4M3) { constexpr int IN = Q8_E4M3, OUT = Q8_I8, MID = Q8_E4M3; __VA_ARGS__; } \
+    else if (CD == Q8_E4M3 && MD == Q8_E4M3) { constexpr int IN = Q8_E4M3, OUT = Q8_E4M3, MID = Q8_E4M3; __VA_ARGS__; } \
     else if (CD == Q8_I8 && MD == Q8_BF16) { constexpr int IN = Q8_E4M3, OUT = Q8_I8, MID = Q8_BF16; __VA_ARGS__; } \
     else if (CD == Q8_E4M3 && MD == Q8_BF16) { constexpr int IN = Q8_E4M3, OUT = Q8_E4M3, MID = Q8_BF16; __VA_ARGS__; } \
     else if (CD == Q8_I8) { constexpr int IN = Q8_E4M3, OUT = Q8_I8, MID = Q8_F32; __VA_ARGS__; } \
@@ -351,7 +377,7 @@ extern "C" int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w,
 }
 
 static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_stride, const void* x2, int64_t x2_row_stride,
-                             const float* cos_t, const float* sin_t, void* codes, float* scales, void* codes2,
+                             const float* norm_w, const float* norm_w2, const float* cos_t, const float* sin_t, void* codes, float* scales, void* codes2,
                              float* scales2, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
                              hipStream_t stream) {
     const bool pair = x2 != nullptr;
@@ -367,6 +393,8 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
     if (pair && ((scales == nullptr) != (scales2 == nullptr))) return fail(Q8_ERR_NULL, "%s: both scale outputs or none", who);
     if (x_row_stride < dim || x_row_stride % 8 != 0 || (pair && (x2_row_stride < dim || x2_row_stride % 8 != 0)))
         return fail(Q8_ERR_SHAPE, "%s: row stride %lld / %lld", who, (long long)x_row_stride, (long long)x2_row_stride);
+    if ((norm_w && !aligned16(norm_w)) || (norm_w2 && !aligned16(norm_w2)))
+        return fail(Q8_ERR_ALIGN, "%s: norm weights must be 16-byte aligned", who);
     if (!aligned16(x) || (pair && !aligned16(x2)) || (cos_t && (!aligned16(cos_t) || !aligned16(sin_t))) ||
         (reinterpret_cast<uintptr_t>(codes) % 8) || (pair && (reinterpret_cast<uintptr_t>(codes2) % 8)))
         return fail(Q8_ERR_ALIGN, "%s: x and tables must be 16-byte aligned, codes 8-byte aligned", who);
@@ -376,7 +404,8 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
     const int64_t grid = (tokens + (kBlock / lanes) - 1) / (kBlock / lanes);
     if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "%s: too many tokens", who);
 #define PREP_ARGS                                                                                                        \
-    static_cast<const uint16_t*>(x), x_row_stride, static_cast<const uint16_t*>(x2), x2_row_stride, cos_t, sin_t,        \
+    static_cast<const uint16_t*>(x), x_row_stride, static_cast<const uint16_t*>(x2), x2_row_stride, norm_w, norm_w2,     \
+        cos_t, sin_t,                                                                                                    \
         static_cast<uint8_t*>(codes), scales, static_cast<uint8_t*>(codes2), scales2, tokens, S, apply_fht, scale,       \
         mid_dtype == Q8_BF16 ? 1 : 0
 #define PREP_LAUNCH(LANES, CH, LH)                                                                                       \
@@ -403,19 +432,19 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
     return launch_status(who);
 }
 
-extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* cos_t, const float* sin_t, void* codes,
-                               float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
-                               q8_stream_t stream_) {
-    return attn_prep_qk_impl("q8_attn_prep_qk", x, x_row_stride, nullptr, 0, cos_t, sin_t, codes, scales, nullptr, nullptr, B, S,
-                             H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
+extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* norm_w, const float* cos_t,
+                               const float* sin_t, void* codes, float* scales, int B, int S, int H, int D, int apply_fht,
+                               float scale, int mid_dtype, q8_stream_t stream_) {
+    return attn_prep_qk_impl("q8_attn_prep_qk", x, x_row_stride, nullptr, 0, norm_w, nullptr, cos_t, sin_t, codes, scales, nullptr,
+                             nullptr, B, S, H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
-                                    const float* cos_t, const float* sin_t, void* codes_q, float* scales_q, void* codes_k,
-                                    float* scales_k, int B, int S, int H, int D, int apply_fht, float scale,
-                                    int mid_dtype, q8_stream_t stream_) {
+                                    const float* norm_wq, const float* norm_wk, const float* cos_t, const float* sin_t,
+                                    void* codes_q, float* scales_q, void* codes_k, float* scales_k, int B, int S, int H,
+                                    int D, int apply_fht, float scale, int mid_dtype, q8_stream_t stream_) {
     if (!xk) return fail(Q8_ERR_NULL, "q8_attn_prep_qk_pair: null pointer");
-    return attn_prep_qk_impl("q8_attn_prep_qk_pair", xq, xq_row_stride, xk, xk_row_stride, cos_t, sin_t, codes_q, scales_q,
+    return attn_prep_qk_impl("q8_attn_prep_qk_pair", xq, xq_row_stride, xk, xk_row_stride, norm_wq, norm_wk, cos_t, sin_t, codes_q, scales_q,
                              codes_k, scales_k, B, S, H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
 }
 

@@ -236,10 +236,15 @@ __device__ __forceinline__ float round_mid(float x) {
     if constexpr (MID == Q8_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(x));
     else return x;
 }
-// the same for 8 values at once: four hardware pair conversions and their unpacking
+// the same for 8 values at once: four hardware pair conversions and their unpacking (bf16), or the c10 e4m3 cast
+// and its decoding
 template <int MID>
 __device__ __forceinline__ void round_mid8(float (&v)[8]) {
-    if constexpr (MID == Q8_BF16) {
+    if constexpr (MID == Q8_E4M3) {
+        const int w0 = (int)pack4_e4m3_c10(v[0], v[1], v[2], v[3]), w1 = (int)pack4_e4m3_c10(v[4], v[5], v[6], v[7]);
+        v[0] = e4m3_to_f32<0>(w0); v[1] = e4m3_to_f32<1>(w0); v[2] = e4m3_to_f32<2>(w0); v[3] = e4m3_to_f32<3>(w0);
+        v[4] = e4m3_to_f32<0>(w1); v[5] = e4m3_to_f32<1>(w1); v[6] = e4m3_to_f32<2>(w1); v[7] = e4m3_to_f32<3>(w1);
+    } else if constexpr (MID == Q8_BF16) {
 #pragma unroll
         for (int i = 0; i < 8; i += 2) {
             const uint32_t u = pack2_bf16(v[i], v[i + 1]);

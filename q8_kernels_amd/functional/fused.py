@@ -18,16 +18,17 @@ _FP8 = torch.float8_e4m3fn
 
 def hadamard_quantize(x: torch.Tensor, out_type: Optional[torch.dtype] = None,
                       scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """bfloat16 x (..., dim) -> (codes, scales) of the Hadamard-rotated rows; out_type None -> int8."""
+    """bfloat16 or e4m3 x (..., dim) -> (codes, scales) of the Hadamard-rotated rows; out_type None -> int8. The
+    transform's intermediate result is rounded to x's dtype, as hadamard_transform(x) stores it."""
     if scale is None:
         scale = 1.0 / math.sqrt(x.shape[-1])
-    codes, scales = _C.fht_quant(x, scale, out_type)
+    codes, scales = _C.fht_quant(x, scale, out_type, mid_type=x.dtype)
     return codes, scales
 
 
 def can_fuse_hadamard_quantize(x: torch.Tensor) -> bool:
-    """The fused kernel reproduces the two-kernel sequence for bfloat16 inputs whose rows need no padding."""
-    return x.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 and x.shape[-1] <= 32768
+    """The fused kernel reproduces the two-kernel sequence for bfloat16 / e4m3 inputs whose rows need no padding."""
+    return x.dtype in (torch.bfloat16, _FP8) and x.shape[-1] % 8 == 0 and x.shape[-1] <= 32768
 
 
 def rms_norm_quantize(x: torch.Tensor, weights: Optional[torch.Tensor] = None,
@@ -40,11 +41,13 @@ def rms_norm_quantize(x: torch.Tensor, weights: Optional[torch.Tensor] = None,
 def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int,
                            softmax_scale: Optional[float] = None, batch_mask: Optional[torch.Tensor] = None,
                            apply_qk_hadamard: bool = False, freqs_cis=None, out_dtype: Optional[torch.dtype] = None,
-                           per_token_scales: bool = False) -> torch.Tensor:
+                           per_token_scales: bool = False, q_norm_weight: Optional[torch.Tensor] = None,
+                           k_norm_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [B, M, H*64], k, v [B, N, H*64] bfloat16 projections (strided slices of a fused projection are read in
     place) -> attention output [B, M, H*64].
 
-    freqs_cis = (cos, sin) fp32 tables of q's shape rotates q and k first (k must then have q's shape).
+    q_norm_weight / k_norm_weight (fp32 [H*64]) apply the qk-RMSNorm (over all heads of a token, no epsilon) first;
+    freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape).
     Without per_token_scales the operands are cast to e4m3 exactly as flash_attn_func does; with it each
     (token, head) row of q, k and v gets its own absmax scale."""
     d = q.shape[-1] // num_heads
@@ -56,10 +59,13 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
     if q.shape == k.shape:  # self-attention: one pass over both, the tables are read once
-        qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+        qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                                      q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
     else:
-        qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
-        kc = _C.attn_prep_qk(k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales)
+        qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                             norm_weight=q_norm_weight)
+        kc = _C.attn_prep_qk(k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                             norm_weight=k_norm_weight)
     vc = _C.attn_prep_v(v, num_heads, per_token_scales)
     if per_token_scales:
         (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc

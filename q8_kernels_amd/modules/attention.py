@@ -39,6 +39,11 @@ class Attention(nn.Module):
         self.to_v = Q8Linear(kv_dim, self.inner_dim, bias=bias)
         self.to_out = Q8Linear(self.inner_dim, out_dim, out_bias)
 
+    def _norm_weight(self, norm):
+        if norm.weight is not None:
+            return norm.weight
+        return torch.ones(self.inner_dim, dtype=torch.float32, device=self.to_q.weight.device)
+
     def _split_heads(self, t, batch):
         return t.view(batch, -1, self.num_heads, self.head_dim).transpose(1, 2)
 
@@ -49,22 +54,36 @@ class Attention(nn.Module):
             attention_mask = attention_mask.argmin(-1).squeeze().int()
 
         kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
-        query = self.to_q(hidden_states, out_dtype=mm_out_dtype)
-        key = self.to_k(kv_src, out_dtype=mm_out_dtype)
-        value = self.to_v(kv_src, out_dtype=mm_out_dtype)
+
+        def project(layers, x):
+            """[layer(x) for layer in layers]; x is rotated and int8-quantized once for all of them (every Q8Linear
+            would do exactly that to the same x on its own)."""
+            if self.fuse_prologue and len(layers) > 1 and x.is_cuda and Q8F.fused.can_fuse_hadamard_quantize(x):
+                xq, xs = Q8F.fused.hadamard_quantize(x)
+                return [layer(xq, xs, out_dtype=mm_out_dtype) for layer in layers]
+            return [layer(x, out_dtype=mm_out_dtype) for layer in layers]
+
+        if encoder_hidden_states is None:
+            query, key, value = project([self.to_q, self.to_k, self.to_v], hidden_states)
+        else:
+            (query,), (key, value) = project([self.to_q], hidden_states), project([self.to_k, self.to_v], kv_src)
+        rope = encoder_hidden_states is None and self.use_rope
+        batch = query.shape[0]
+        if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64
+                and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
+                and non_mm_precision == torch.bfloat16 and query.dim() == 3
+                and all(t.dtype == torch.bfloat16 for t in (query, key, value))):
+            # qk-RMSNorm, RoPE, head split, Hadamard and the e4m3 cast in one prologue kernel, head-merged attention
+            # output: the same bits as the sequence below
+            hidden_states = Q8F.fused.flash_attn_token_major(
+                query, key, value, self.num_heads, batch_mask=attention_mask, apply_qk_hadamard=apply_qk_hadamard,
+                freqs_cis=freqs_cis if rope else None,
+                q_norm_weight=self._norm_weight(self.q_norm) if self.qk_rms_norm else None,
+                k_norm_weight=self._norm_weight(self.k_norm) if self.qk_rms_norm else None)
+            return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
         if self.qk_rms_norm:
             query = self.q_norm(query, non_mm_precision)
             key = self.k_norm(key, non_mm_precision)
-        rope = encoder_hidden_states is None and self.use_rope
-        batch = query.shape[0]
-        if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64 and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
-                and non_mm_precision == torch.bfloat16 and query.dim() == 3
-                and all(t.dtype == torch.bfloat16 for t in (query, key, value))):
-            # one prologue kernel per operand and head-merged output: the same bits as the sequence below
-            hidden_states = Q8F.fused.flash_attn_token_major(
-                query, key, value, self.num_heads, batch_mask=attention_mask, apply_qk_hadamard=apply_qk_hadamard,
-                freqs_cis=freqs_cis if rope else None)
-            return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
         if rope:
             query = Q8F.rope.apply_rope(query, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)
             key = Q8F.rope.apply_rope(key, freqs_cis[0], freqs_cis[1], out_type=non_mm_precision)

@@ -66,6 +66,42 @@ def test_strerror_and_argument_validation_without_gpu():
         _lib.check(-3)
 
 
+def test_argument_validation_of_the_fused_and_elementwise_entry_points():
+    from q8_kernels_amd import _lib
+    L = _lib.lib()
+    B16, E4, I8, F32 = _lib.Q8_BF16, _lib.Q8_E4M3, _lib.Q8_I8, _lib.Q8_F32
+    # rows == 0 is a no-op before anything else is looked at
+    assert L.q8_fma(None, E4, None, F32, None, F32, None, E4, 0, 64, 1, 1, 0.0, None) == 0
+    assert L.q8_fht_quant_rows(None, B16, None, I8, None, 0, 64, 1.0, B16, 0, None) == 0
+    assert L.q8_attn_prep_qk(None, 512, None, None, None, None, None, 0, 5, 8, 64, 1, 1.0, B16, None) == 0
+    assert L.q8_fma(None, E4, 16, F32, 16, F32, 16, E4, 4, 64, 1, 1, 0.0, None) == -1
+    assert L.q8_fma(16, E4, 16, F32, 16, F32, 16, E4, 4, 60, 1, 1, 0.0, None) == -3
+    assert L.q8_fma(16, E4, 16, F32, 16, F32, 16, E4, 4, 64, 0, 1, 0.0, None) == -3
+    assert L.q8_fma(16, F32, 16, F32, 16, F32, 16, E4, 4, 64, 1, 1, 0.0, None) == -2
+    assert L.q8_fma(16, B16, 8, B16, 16, F32, 16, E4, 4, 64, 1, 1, 0.0, None) == -4
+    assert L.q8_gelu(16, B16, 16, B16, 12, None) == -3
+    assert L.q8_gelu_backward(16, B16, None, B16, 16, B16, 64, None) == -1
+    assert L.q8_rope_backward(16, B16, None, 16, 16, B16, 4, 64, None) == -1
+    assert L.q8_rmsnorm_backward(16, B16, None, 16, B16, None, 16, B16, 4, 64, None) == -1
+    assert L.q8_rmsnorm_backward(16, B16, 16, 16, F32, None, 16, B16, 4, 64, None) == -2
+    assert L.q8_fht_quant_rows(16, B16, 16, B16, 16, 4, 64, 1.0, B16, 0, None) == -2
+    assert L.q8_fht_quant_rows(16, B16, 16, I8, 16, 4, 64, 1.0, E4, 0, None) == -2   # e4m3 intermediate needs an e4m3 input
+    assert L.q8_rmsnorm_quant_rows(16, B16, 8, 16, I8, 16, None, 4, 64, 0.0, B16, 0, None) == -4
+    assert L.q8_attn_prep_qk(16, 512, None, None, None, 16, None, 1, 5, 8, 32, 1, 1.0, B16, None) == -3
+    assert b"head dim" in L.q8_last_error()
+    assert L.q8_attn_prep_qk(16, 512, None, None, None, 16, None, 1, 5, 12, 64, 1, 1.0, B16, None) == -3   # H * D = 768
+    assert L.q8_attn_prep_qk(16, 500, None, None, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -3    # stride < H * D
+    assert L.q8_attn_prep_qk(16, 512, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1      # cos without sin
+    assert L.q8_attn_prep_qk_pair(16, 512, None, 512, None, None, None, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
+    assert L.q8_attn_prep_qk_pair(16, 512, 16, 512, None, None, None, None, 16, 16, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
+    assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 64, 5, None) == -3                          # S_pad % 16
+    assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 128, 16, None) == -3
+    assert L.q8_gemm_residual(16, 16, None, 16, 16, None, 16, 1, 1, 8, 8, 384, I8, 0, None) == -1
+    assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 8, 256, I8, 0, None) == -3     # K must exceed 256
+    assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 12, 384, I8, 0, None) == -3    # N % 8
+    assert L.q8_gemm_set_config(7) == -6
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     import torch
     from q8_kernels_amd import _C

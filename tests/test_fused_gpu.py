@@ -57,6 +57,43 @@ def _accepts_f32():
         return False
 
 
+def test_fht_quant_e4m3_intermediate(dev):
+    """e4m3 in, e4m3 intermediate (what the int8 linear does to an fp8 activation): quantize(hadamard_transform(x))."""
+    g = torch.Generator().manual_seed(8)
+    x = O.e4m3_c10(torch.randn(37, 2048, generator=g) * 3)
+    for out_type in (None, E4M3):
+        codes, scales = _C().fht_quant(x.to(dev), 2048 ** -0.5, out_type, mid_type=E4M3)
+        wc, ws = O.ref_quant(O.ref_fht(x, 2048 ** -0.5, E4M3), out_type)
+        assert_bit_equal(codes, wc, "codes")
+        assert_bit_equal(scales, ws, "scales")
+
+
+@pytest.mark.parametrize("shape", [(2, 70, 8, 64), (1, 33, 32, 64), (2, 9, 24, 64), (2, 37, 4, 64)])
+@pytest.mark.parametrize("pair", [False, True])
+def test_attn_prep_qk_with_qk_rmsnorm(dev, shape, pair):
+    """RMSNorm over the whole token row, then RoPE, head split, FHT and the cast: equal to the separate kernels."""
+    b, s, h, d = shape
+    dim = h * d
+    g = torch.Generator().manual_seed(dim + s)
+    q, k = ((torch.randn(b, s, dim, generator=g) * 1.5).to(BF16).to(dev) for _ in range(2))
+    wq, wk = ((1 + 0.1 * torch.randn(dim, generator=g)).to(dev) for _ in range(2))
+    ang = torch.rand(b, s, dim // 2, generator=g) * 6.28
+    cos, sin = torch.cos(ang).repeat_interleave(2, -1).to(dev), torch.sin(ang).repeat_interleave(2, -1).to(dev)
+    wantq = _C().attn_prep_qk(_C().rms_norm(q, wq, BF16)[0], h, cos, sin, True, 0.125)
+    wantk = _C().attn_prep_qk(_C().rms_norm(k, wk, BF16)[0], h, cos, sin, True, 0.125)
+    if pair:
+        gotq, gotk = _C().attn_prep_qk_pair(q, k, h, cos, sin, True, 0.125, q_norm_weight=wq, k_norm_weight=wk)
+    else:
+        gotq = _C().attn_prep_qk(q, h, cos, sin, True, 0.125, norm_weight=wq)
+        gotk = _C().attn_prep_qk(k, h, cos, sin, True, 0.125, norm_weight=wk)
+    assert_bit_equal(gotq, wantq, "q")
+    assert_bit_equal(gotk, wantk, "k")
+    # and against the oracle's composition (the row sum of squares is accumulated in another order there)
+    yo = O.ref_rope(O.ref_rms_norm(q.cpu(), wq.cpu(), BF16)[0], cos.cpu(), sin.cpu(), BF16)
+    want = O.ref_fht(_heads(yo, h), 0.125, E4M3)
+    assert float((gotq.cpu().view(torch.uint8) != want.view(torch.uint8)).float().mean()) < 0.01
+
+
 def test_fht_quant_equals_separate_kernels_full_size(dev):
     g = torch.Generator().manual_seed(6)
     x = torch.randn(12288, 2048, generator=g).to(BF16).to(dev)
