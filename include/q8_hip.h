@@ -172,6 +172,18 @@ int q8_fht_quant_rows(const void* x, int x_dtype, void* codes, int code_dtype, f
 int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w, void* codes, int code_dtype, float* scales,
                           float* rstd, int64_t rows, int dim, float eps, int mid_dtype, int flags,
                           q8_stream_t stream);
+/*
+ * The whole prologue of a projection behind an AdaLN-modulated norm, bf16 x [rows, dim] -> codes, scales:
+ *   [apply_norm: rmsnorm(x) * norm_w (norm_w NULL = 1), no epsilon] -> [x * (mod_scale + scale_add) + mod_shift, one
+ *   fused multiply-add as q8_fma; mod_scale / mod_shift [rows / rows_per_mod, dim] in mod_dtype (BF16 or F32), both
+ *   NULL = none] -> [apply_fht: FHT * fht_scale] -> quantizer. Every step rounds to bfloat16 where the separate calls
+ *   (q8_rmsnorm, q8_fma, q8_fht, q8_quant_rows: q8_kernels/blocks/ltx_transformer_block.py:38-40,
+ *   q8_kernels/functional/linear.py:30-31) store a bfloat16 tensor, so the codes and scales are the same bits.
+ */
+int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, int apply_norm, const void* mod_scale,
+                               const void* mod_shift, int mod_dtype, int64_t rows_per_mod, float scale_add,
+                               int apply_fht, float fht_scale, void* codes, int code_dtype, float* scales,
+                               int64_t rows, int dim, int flags, q8_stream_t stream);
 
 /*
  * Attention prologues: from token-major 16-bit projections [B, S, H*D] (row stride in elements, so a slice of a

@@ -365,6 +365,43 @@ def rms_norm_quant(x: torch.Tensor, weights: Optional[torch.Tensor] = None, out_
     return [out.reshape(shape), scales.reshape(shape[:-1]), rstd.reshape(shape[:-1])]
 
 
+def norm_mod_fht_quant(x: torch.Tensor, norm: bool = True, norm_weight: Optional[torch.Tensor] = None,
+                       mod_scale: Optional[torch.Tensor] = None, mod_shift: Optional[torch.Tensor] = None,
+                       scale_add: float = 0.0, fht_scale: Optional[float] = None,
+                       out_type: Optional[torch.dtype] = None) -> List[torch.Tensor]:
+    """bfloat16 x [B, T, dim] -> [codes, scales] of quant(FHT(fma(rms_norm(x, norm_weight), mod_scale + scale_add,
+    mod_shift)) * fht_scale) in one pass; every step is optional (norm False, mod_scale / mod_shift None, fht_scale
+    None) and rounds to bfloat16 like the separate operators. mod_scale / mod_shift: [B, 1 or T, dim], bfloat16 or
+    float32. out_type None -> int8."""
+    _require_gpu(x, "x")
+    if x.dtype != torch.bfloat16 or x.dim() != 3:
+        raise RuntimeError("norm_mod_fht_quant: x must be a bfloat16 tensor [B, T, dim]")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).contiguous()
+    out_type, out, scales = _quant_out(x2, out_type, "norm_mod_fht_quant")
+    rows, dim = x2.shape
+    if norm_weight is not None and (norm_weight.dtype != torch.float32 or not norm_weight.is_cuda or norm_weight.numel() != dim):
+        raise RuntimeError("norm_mod_fht_quant: norm weights must be a float32 CUDA tensor with dim elements")
+    if (mod_scale is None) != (mod_shift is None):
+        raise RuntimeError("norm_mod_fht_quant: mod_scale and mod_shift come together")
+    rows_per_mod, mod_dt = 1, Q8_BF16
+    if mod_scale is not None:
+        for t in (mod_scale, mod_shift):
+            _require_gpu(t, "modulation")
+            if (t.dtype != mod_scale.dtype or t.dtype not in (torch.bfloat16, torch.float32) or t.dim() != 3 or t.shape[0] != shape[0]
+                    or t.shape[-1] != dim or t.shape[1] != mod_scale.shape[1] or t.shape[1] not in (1, shape[1])):
+                raise RuntimeError("norm_mod_fht_quant: mod_scale / mod_shift must be [B, 1 or T, dim], both bfloat16 or float32")
+        mod_scale, mod_shift = mod_scale.contiguous(), mod_shift.contiguous()
+        rows_per_mod, mod_dt = shape[1] // mod_scale.shape[1], _DT[mod_scale.dtype]
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().q8_norm_mod_fht_quant_rows(
+            x2.data_ptr(), _ptr(None if norm_weight is None else norm_weight.contiguous()), int(norm), _ptr(mod_scale),
+            _ptr(mod_shift), mod_dt, rows_per_mod, float(scale_add), int(fht_scale is not None),
+            float(fht_scale if fht_scale is not None else 1.0), out.data_ptr(), _DT[out_type], scales.data_ptr(), rows, dim,
+            0, _stream(x)))
+    return [out.reshape(shape), scales.reshape(shape[:-1])]
+
+
 def _token_major(x, num_heads, who):
     """x [B, S, H*D] bfloat16 with unit last stride and one row stride over (B, S)."""
     _require_gpu(x, "x")

@@ -34,6 +34,7 @@ SIGNATURES = {
     "q8_rmsnorm_backward": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i, _vp]),
     "q8_fht_quant_rows": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _f, _i, _i, _vp]),
     "q8_rmsnorm_quant_rows": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i64, _i, _f, _i, _i, _vp]),
+    "q8_norm_mod_fht_quant_rows": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i64, _f, _i, _f, _vp, _i, _vp, _i64, _i, _i, _vp]),
     "q8_attn_prep_qk": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "q8_attn_prep_qk_pair": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "q8_attn_prep_v": (_i, [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

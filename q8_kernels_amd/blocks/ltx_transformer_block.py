@@ -15,6 +15,10 @@ from ..modules.rms_norm import RMSNorm
 
 
 class LTXTransformerBlock(nn.Module):
+    # True (default): norm, modulation, Hadamard rotation and int8 quantization in front of attn1 and of the
+    # feed-forward run as one kernel; False: operator by operator. Both give the same bits.
+    fuse_prologue = True
+
     def __init__(self, dim, num_heads, head_dim, kv_dim, bias=True, use_rope=True, norm_affine=False):
         super().__init__()
         self.norm1 = RMSNorm(dim, norm_affine)
@@ -40,7 +44,16 @@ class LTXTransformerBlock(nn.Module):
             hidden_states.shape[0], timestep.shape[1], num_ada_params, -1)
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada_values.unbind(dim=2)
 
-        norm_hidden_states = self._fma(self.norm1(hidden_states, non_mm_precision), scale_msa, shift_msa, 1.0)
+        fuse = (self.fuse_prologue and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16
+                and non_mm_precision == torch.bfloat16 and hidden_states.dim() == 3 and hidden_states.shape[-1] % 8 == 0
+                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or timestep.requires_grad)))
+        bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
+
+        if fuse:  # (int8 codes, row scales) of the rotated, modulated norm: what attn1's projections would compute
+            norm_hidden_states = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm1.weight, bf(scale_msa),
+                                                                  bf(shift_msa), 1.0)
+        else:
+            norm_hidden_states = self._fma(self.norm1(hidden_states, non_mm_precision), scale_msa, shift_msa, 1.0)
         attn_output = self.attn1(norm_hidden_states, freqs_cis, None, attention_mask, non_mm_precision, mm_out_dtype,
                                  attn_type=attn_type)
         hidden_states = self._fma(attn_output, gate_msa, hidden_states, 0.0)
@@ -50,7 +63,12 @@ class LTXTransformerBlock(nn.Module):
                                  mm_out_dtype=mm_out_dtype, attn_type=attn_type)
         hidden_states = attn_output + hidden_states
 
-        norm_hidden_states = self._fma(self.norm2(hidden_states, non_mm_precision), scale_mlp, shift_mlp, 1.0)
-        ff_output = self.ff(norm_hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
+        if fuse:
+            codes, row_scales = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm2.weight, bf(scale_mlp),
+                                                                 bf(shift_mlp), 1.0)
+            ff_output = self.ff(codes, out_dtype=mm_out_dtype, x_scales=row_scales).to(non_mm_precision)
+        else:
+            norm_hidden_states = self._fma(self.norm2(hidden_states, non_mm_precision), scale_mlp, shift_mlp, 1.0)
+            ff_output = self.ff(norm_hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
         hidden_states = self._fma(ff_output, gate_mlp, hidden_states, 0.0)
         return hidden_states

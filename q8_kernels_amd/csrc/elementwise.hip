@@ -6,17 +6,6 @@
 
 namespace q8 {
 
-__device__ __forceinline__ void load8_any(const void* p, int dt, int64_t e, float (&v)[8]) {
-    switch (dt) {
-        case Q8_BF16: load8<Q8_BF16>(p, e, v); break;
-        case Q8_F32: load8<Q8_F32>(p, e, v); break;
-        default: load8<Q8_E4M3>(p, e, v); break;
-    }
-}
-__device__ __forceinline__ void store8_any(void* p, int dt, int64_t e, const float (&v)[8]) {
-    if (dt == Q8_BF16) store8<Q8_BF16>(p, e, v); else store8<Q8_E4M3>(p, e, v);
-}
-
 // s = 0.5 (1 + tanh(t)) = 1 / (1 + exp(-2 t)) and 1 - s, both without cancellation in either tail:
 // with u = exp(-2 |t|) <= 1, (s, 1 - s) = (1, u) / (1 + u) for t >= 0 and (u, 1) / (1 + u) for t < 0.
 __device__ __forceinline__ void half_one_plus_tanh(float t, float& s, float& one_minus_s) {

@@ -128,6 +128,106 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
     }
 }
 
+// ---- RMSNorm -> AdaLN modulation -> FHT -> quantizer ---------------------------------------------------------
+//
+// The prologue of an int8 projection behind a modulated norm (q8_kernels/blocks/ltx_transformer_block.py:38-40 followed
+// by q8_kernels/functional/linear.py:30-31): y1 = bf16(rmsnorm(x) w), y2 = bf16(y1 (mod_scale + scale_add) + mod_shift)
+// (one fused multiply-add, as q8_fma), y3 = bf16(FHT(y2) fht_scale), codes = quant(y3). Each step is optional
+// (w, mod_scale / mod_shift NULL, apply_fht 0) and rounds where the separate kernels store a bfloat16 tensor.
+template <int LANES, int CH, int OUT>
+__global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* __restrict__ x, const float* __restrict__ w,
+                                                                    int apply_norm, const void* __restrict__ ms,
+                                                                    const void* __restrict__ mt, int mod_dtype,
+                                                                    int64_t rows_per_mod, float scale_add, int apply_fht,
+                                                                    float fht_scale, void* __restrict__ codes,
+                                                                    float* __restrict__ scales, int64_t rows, int dim,
+                                                                    int flags) {
+    constexpr int RPB = kBlock / LANES;
+    __shared__ float red[4];
+    const int t = threadIdx.x % LANES;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
+    const bool row_ok = row < rows;
+    const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * 2;
+
+    float v[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (row_ok && e < dim) {
+            load8<Q8_BF16>(xr, e, v[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+        }
+    }
+    if (apply_norm) {
+        float ss[1] = {0.f};
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss[0] += v[c][i] * v[c][i];
+        row_reduce<LANES, false, 1>(ss, red);
+        const float rstd = 1.0f / sqrtf(ss[0] * (1.0f / (float)dim));
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (e >= dim) continue;
+            if (w != nullptr) {
+                float wv[8];
+                load8<Q8_F32>(w, e, wv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[c][i] = (v[c][i] * rstd) * wv[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[c][i] = v[c][i] * rstd;
+            }
+            round_mid8<Q8_BF16>(v[c]);
+        }
+    }
+    if (ms != nullptr) {
+        const int64_t mrow = row_ok ? row / rows_per_mod : 0;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (e >= dim) continue;
+            float sv[8], tv[8];
+            load8_any(ms, mod_dtype, mrow * dim + e, sv);
+            load8_any(mt, mod_dtype, mrow * dim + e, tv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = __builtin_fmaf(v[c][i], sv[i] + scale_add, tv[i]);
+            round_mid8<Q8_BF16>(v[c]);
+        }
+    }
+    if (apply_fht) {
+        fht_row<LANES, CH>(v, t);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] *= fht_scale;
+            round_mid8<Q8_BF16>(v[c]);
+        }
+    }
+    float amax[1] = {0.f};
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (e < dim) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax[0] = fmaxf(amax[0], fabsf(v[c][i]));
+        }
+    }
+    row_reduce<LANES, true, 1>(amax, red);
+    if (!row_ok) return;
+    const float ratio = quant_ratio<OUT>(amax[0]);
+    if (t == 0) scales[row] = quant_scale<OUT>(amax[0], ratio, flags);
+    uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
+    }
+}
+
 // ---- attention prologue for Q and K ---------------------------------------------------------------------
 //
 // LANES threads per token: the row of H * D = 8 * LANES * CH elements (H heads of D = 8 * LH) uses the row mapping,
@@ -374,6 +474,36 @@ extern "C" int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w,
         })
     })
     return launch_status("q8_rmsnorm_quant_rows");
+}
+
+extern "C" int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, int apply_norm, const void* mod_scale,
+                                          const void* mod_shift, int mod_dtype, int64_t rows_per_mod, float scale_add,
+                                          int apply_fht, float fht_scale, void* codes, int code_dtype, float* scales,
+                                          int64_t rows, int dim, int flags, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "q8_norm_mod_fht_quant_rows";
+    if (int st = check_rows(who, rows, dim)) return st;
+    if (rows == 0) return Q8_OK;
+    if (int st = check_quant_args(who, x, Q8_BF16, codes, code_dtype, scales, Q8_BF16, flags)) return st;
+    if (norm_w && !aligned16(norm_w)) return fail(Q8_ERR_ALIGN, "%s: weights must be 16-byte aligned", who);
+    if ((mod_scale == nullptr) != (mod_shift == nullptr)) return fail(Q8_ERR_NULL, "%s: scale and shift come together", who);
+    if (mod_scale) {
+        if (mod_dtype != Q8_BF16 && mod_dtype != Q8_F32) return fail(Q8_ERR_DTYPE, "%s: modulation dtype %d (want BF16 or F32)", who, mod_dtype);
+        if (rows_per_mod <= 0) return fail(Q8_ERR_SHAPE, "%s: rows_per_mod must be positive", who);
+        if (!aligned16(mod_scale) || !aligned16(mod_shift)) return fail(Q8_ERR_ALIGN, "%s: modulation rows must be 16-byte aligned", who);
+    }
+    const int N = pow2_ceil(dim);
+    const int64_t rpm = mod_scale ? rows_per_mod : 1;
+#define NMQ_LAUNCH(OUT)                                                                                                  \
+    Q8_ROW_SHAPE_SWITCH(N, {                                                                                             \
+        const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);                                           \
+        hipLaunchKernelGGL((norm_mod_fht_quant_kernel<LANES, CH, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, \
+                           norm_w, apply_norm, mod_scale, mod_shift, mod_dtype, rpm, scale_add, apply_fht, fht_scale,    \
+                           codes, scales, rows, dim, flags);                                                             \
+    })
+    if (code_dtype == Q8_I8) { NMQ_LAUNCH(Q8_I8) } else { NMQ_LAUNCH(Q8_E4M3) }
+#undef NMQ_LAUNCH
+    return launch_status(who);
 }
 
 static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_stride, const void* x2, int64_t x2_row_stride,

@@ -228,6 +228,19 @@ __device__ __forceinline__ void fht_row(float (&v)[CH][8], int t) {
     }
 }
 
+// ---- 8-element chunks with a run-time element type (uniform switch) ------------------------------------
+
+__device__ __forceinline__ void load8_any(const void* p, int dt, int64_t e, float (&v)[8]) {
+    switch (dt) {
+        case Q8_BF16: load8<Q8_BF16>(p, e, v); break;
+        case Q8_F32: load8<Q8_F32>(p, e, v); break;
+        default: load8<Q8_E4M3>(p, e, v); break;
+    }
+}
+__device__ __forceinline__ void store8_any(void* p, int dt, int64_t e, const float (&v)[8]) {
+    if (dt == Q8_BF16) store8<Q8_BF16>(p, e, v); else store8<Q8_E4M3>(p, e, v);
+}
+
 // ---- quantizer arithmetic -------------------------------------------------------------------------
 
 // value an intermediate tensor of dtype MID would hold (round trip through its storage format)

@@ -3,6 +3,8 @@ same bits as the sequence it names; none has a counterpart of its own in the ref
 
     hadamard_quantize      = quantize(hadamard_transform(x))              (q8_kernels/functional/linear.py:30-31)
     rms_norm_quantize      = quantize(rms_norm_8bit(x, w)[0])             (q8_kernels/modules/attention.py:67-77)
+    norm_modulate_quantize = quantize(hadamard_transform(multiply_add(rms_norm_8bit(x, w), scale, shift, 1)))
+                                                                          (q8_kernels/blocks/ltx_transformer_block.py:38-40)
     flash_attn_token_major = apply_rope -> split heads -> flash_attn_func -> merge heads
                                                                           (q8_kernels/modules/attention.py:84-105)
 """
@@ -35,6 +37,18 @@ def rms_norm_quantize(x: torch.Tensor, weights: Optional[torch.Tensor] = None,
                       out_type: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """bfloat16 x -> (codes, scales) of rms_norm(x) * weights; out_type None -> int8."""
     codes, scales, _ = _C.rms_norm_quant(x, weights, out_type)
+    return codes, scales
+
+
+def norm_modulate_quantize(x: torch.Tensor, norm_weight: Optional[torch.Tensor], mod_scale: torch.Tensor,
+                           mod_shift: torch.Tensor, scale_add: float = 1.0,
+                           out_type: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """quantize(hadamard_transform(multiply_add(rms_norm_8bit(x, norm_weight), mod_scale, mod_shift, scale_add))) in one
+    kernel: the input of an int8 projection behind an AdaLN-modulated norm
+    (q8_kernels/blocks/ltx_transformer_block.py:38-40 + q8_kernels/functional/linear.py:30-31), same bits.
+    x [B, T, dim] bfloat16; mod_scale / mod_shift [B, 1 or T, dim] bfloat16."""
+    codes, scales = _C.norm_mod_fht_quant(x, True, norm_weight, mod_scale, mod_shift, scale_add,
+                                          1.0 / math.sqrt(x.shape[-1]), out_type)
     return codes, scales
 
 

@@ -10,5 +10,6 @@ class GELU(nn.Module):
         super().__init__()
         self.proj = Q8Linear(dim_in, dim_out, bias=bias)
 
-    def forward(self, hidden_states, out_dtype=None):
-        return self.proj(hidden_states, fuse_gelu=True, out_dtype=out_dtype)
+    def forward(self, hidden_states, out_dtype=None, x_scales=None):
+        """x_scales: row scales of an already rotated and int8-quantized hidden_states (passed on to Q8Linear)."""
+        return self.proj(hidden_states, x_scales, fuse_gelu=True, out_dtype=out_dtype)

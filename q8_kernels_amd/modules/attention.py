@@ -49,6 +49,8 @@ class Attention(nn.Module):
 
     def forward(self, hidden_states, freqs_cis=None, encoder_hidden_states=None, attention_mask=None,
                 non_mm_precision=torch.bfloat16, mm_out_dtype=None, apply_qk_hadamard=True, attn_type="torch"):
+        """hidden_states: the activations, or (for self-attention) a tuple (int8 codes, row scales) of their
+        Hadamard-rotated quantization, which is what the q / k / v projections consume."""
         if attention_mask is not None and attention_mask.ndim > 1 and attn_type == "q8_kernels":
             # [B, Skv] 0/1 mask -> valid lengths, the reference's rule (first zero; an all-ones row gives 0)
             attention_mask = attention_mask.argmin(-1).squeeze().int()
@@ -58,6 +60,8 @@ class Attention(nn.Module):
         def project(layers, x):
             """[layer(x) for layer in layers]; x is rotated and int8-quantized once for all of them (every Q8Linear
             would do exactly that to the same x on its own)."""
+            if isinstance(x, tuple):  # already (int8 codes, row scales)
+                return [layer(x[0], x[1], out_dtype=mm_out_dtype) for layer in layers]
             if self.fuse_prologue and len(layers) > 1 and x.is_cuda and Q8F.fused.can_fuse_hadamard_quantize(x):
                 xq, xs = Q8F.fused.hadamard_quantize(x)
                 return [layer(xq, xs, out_dtype=mm_out_dtype) for layer in layers]

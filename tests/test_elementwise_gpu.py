@@ -209,6 +209,59 @@ def test_ltx_transformer_block_matches_oracle(dev):
     assert got.shape == hidden.shape and got.dtype == BF16
     assert cosine(got.cpu(), want) > 0.999
     assert (got.cpu().double() - want.double()).abs().max() <= 0.06 * want.double().abs().max()
+    # operator by operator (no fused prologues anywhere): the same bits. The fused kernel is counted, so that
+    # the comparison cannot pass by both runs taking the same path.
+    from q8_kernels_amd.modules import Attention
+    impl, calls = _C().norm_mod_fht_quant, []
+    def counted(*a, **k):
+        calls.append(1)
+        return impl(*a, **k)
+    run = lambda: blk(hidden.to(dev), (cos.to(dev), sin.to(dev)), None, text.to(dev), lens.to(dev),  # noqa: E731
+                      timestep.to(dev), attn_type="q8_kernels")
+    try:
+        _C().norm_mod_fht_quant = counted
+        with torch.no_grad():
+            again = run()
+        assert len(calls) == 2, f"fused prologue ran {len(calls)} times, expected 2 (attn1 and feed-forward)"
+        LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = False
+        with torch.no_grad():
+            seq = run()
+        assert len(calls) == 2, "the operator-by-operator path called the fused prologue"
+    finally:
+        _C().norm_mod_fht_quant = impl
+        LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = True
+    assert_bit_equal(got, again, "fused block, second run")
+    assert_bit_equal(got, seq, "fused block vs operator sequence")
+
+
+@pytest.mark.parametrize("dim", [256, 1000, 2048, 8192])
+@pytest.mark.parametrize("out_type", [torch.int8, E4M3])
+def test_norm_mod_fht_quant_equals_the_operator_sequence(dev, dim, out_type):
+    g = torch.Generator().manual_seed(dim + 3)
+    b, t = 2, 19
+    x = (torch.randn(b, t, dim, generator=g) * 1.3).to(BF16)
+    w = 1 + 0.1 * torch.randn(dim, generator=g)
+    for tm, mod_type in ((1, BF16), (t, BF16), (1, torch.float32)):
+        sc = (torch.randn(b, tm, dim, generator=g) * 0.2).to(mod_type)
+        sh = (torch.randn(b, tm, dim, generator=g) * 0.2).to(mod_type)
+        codes, scales = _C().norm_mod_fht_quant(x.to(dev), True, w.to(dev), sc.to(dev), sh.to(dev), 1.0, dim ** -0.5, out_type)
+        y = O.ref_fma(O.ref_rms_norm(x, w, BF16)[0], sc, sh, 1.0)
+        # the separate HIP kernels (same summation order): bit for bit
+        yd = _C().fma_8bit(_C().rms_norm(x.to(dev), w.to(dev), BF16)[0], sc.to(dev), sh.to(dev), 1.0)
+        wc, ws = _C().tokenwise_quant(_C().fast_hadamard_transform(yd, dim ** -0.5, None), out_type)
+        assert_bit_equal(codes, wc, "codes vs separate kernels")
+        assert_bit_equal(scales, ws, "scales vs separate kernels")
+        # the oracle (float64 sum of squares): codes may move where a value sits on a rounding boundary
+        oc, _ = O.ref_quant(O.ref_fht(y, dim ** -0.5, BF16), out_type)
+        assert float((codes.cpu().view(torch.uint8) != oc.view(torch.uint8)).float().mean()) < 0.02
+    # steps switched off: plain FHT + quantizer, and plain quantizer
+    codes, scales = _C().norm_mod_fht_quant(x.to(dev), False, None, None, None, 0.0, dim ** -0.5, out_type)
+    wc, ws = O.ref_quant(O.ref_fht(x, dim ** -0.5, BF16), out_type)
+    assert_bit_equal(codes, wc, "fht + quant")
+    assert_bit_equal(scales, ws, "fht + quant scales")
+    codes, scales = _C().norm_mod_fht_quant(x.to(dev), False, None, None, None, 0.0, None, out_type)
+    wc, ws = O.ref_quant(x, out_type)
+    assert_bit_equal(codes, wc, "quant only")
 
 
 # ------------------------------------------------------------------ weight conversion
