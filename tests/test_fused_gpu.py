@@ -252,10 +252,23 @@ def test_attention_module_fused_path_equals_operator_sequence(dev):
     ang = torch.rand(2, 77, 256, device=dev) * 6.28
     freqs = (torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1))
     kw = dict(freqs_cis=freqs, mm_out_dtype=BF16, attn_type="q8_kernels")
-    fused = attn(x, **kw)
+    # both gated sites are counted, so that the comparison cannot pass by both runs taking the same path
+    import q8_kernels_amd.functional.fused as FU
+    saved, calls = (FU.hadamard_quantize, FU.flash_attn_token_major), {"rotate": 0, "prologue": 0}
+    def rotate(*a, **k):
+        calls["rotate"] += 1
+        return saved[0](*a, **k)
+    def prologue(*a, **k):
+        calls["prologue"] += 1
+        return saved[1](*a, **k)
     try:
+        FU.hadamard_quantize, FU.flash_attn_token_major = rotate, prologue
+        fused = attn(x, **kw)
+        assert calls == {"rotate": 1, "prologue": 1}, f"fused path not taken: {calls}"
         Attention.fuse_prologue = False
         seq = attn(x, **kw)
+        assert calls == {"rotate": 1, "prologue": 1}, f"operator path used a fused kernel: {calls}"
     finally:
+        FU.hadamard_quantize, FU.flash_attn_token_major = saved
         Attention.fuse_prologue = True
     assert_bit_equal(fused, seq, "attention module output")
