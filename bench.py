@@ -38,9 +38,13 @@ def _ramp_clocks(fn, seconds=0.4):
         torch.cuda.synchronize()
 
 
-def _time(fn, steps, warmup):
+def _time(fn, steps, warmup, ramp=0.15):
     """Mean seconds per call over exactly `steps` calls (HIP events on the current stream, which is the
-    stream the library launches on)."""
+    stream the library launches on). `ramp` seconds of untimed calls come first: every workload here is set up
+    on the host while the device idles, and `warmup` calls of a 20-100 us kernel are far shorter than the time
+    the engine clock needs to come back up."""
+    if ramp > 0:
+        _ramp_clocks(fn, ramp)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
