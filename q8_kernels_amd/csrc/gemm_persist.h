@@ -56,7 +56,11 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     constexpr int BM = 64 * MT, BN = kPipeBN;
     constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // The wave index is read back as a scalar: everything derived from it then lives in scalar registers. With it in
+    // a vector register the 256-row variants spill tile-change and epilogue state, and every reload of a spilled value
+    // costs a wait for ALL outstanding copies (scratch loads share the in-order counter of the copy pipeline).
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave >> 2, wave_n = wave & 3;
     const int M = p.M, N = p.N, K = p.K;
     const int tiles = tiles_m * tiles_n;
