@@ -53,7 +53,8 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
     __shared__ __attribute__((aligned(256))) float lds_sc[SCALED ? kStages * 128 : 4];  // per stage: sk[64], sv[64]
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what is derived from it stays off the VALU
     const int ql = lane & 31, h = lane >> 5;
     const int bh = blockIdx.y, b = bh / p.H;
     const int M = p.M, N = p.N;
