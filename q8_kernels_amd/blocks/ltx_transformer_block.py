@@ -58,10 +58,10 @@ class LTXTransformerBlock(nn.Module):
                                  attn_type=attn_type)
         hidden_states = self._fma(attn_output, gate_msa, hidden_states, 0.0)
 
-        attn_output = self.attn2(hidden_states, freqs_cis=freqs_cis, encoder_hidden_states=encoder_hidden_states,
-                                 attention_mask=encoder_attention_mask, non_mm_precision=non_mm_precision,
-                                 mm_out_dtype=mm_out_dtype, attn_type=attn_type)
-        hidden_states = attn_output + hidden_states
+        # the residual around the cross-attention is added in the epilogue of its output projection where that applies
+        hidden_states = self.attn2(hidden_states, freqs_cis=freqs_cis, encoder_hidden_states=encoder_hidden_states,
+                                   attention_mask=encoder_attention_mask, non_mm_precision=non_mm_precision,
+                                   mm_out_dtype=mm_out_dtype, attn_type=attn_type, residual=hidden_states)
 
         if fuse:
             codes, row_scales = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm2.weight, bf(scale_mlp),

@@ -35,7 +35,7 @@ def _needs_grad(t) -> bool:
 
 # ----------------------------------------------------------------------------- int8
 
-def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype):
+def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=None):
     a_needs_q = a.dtype == _FP8 or is_16bit(a)
     b_needs_q = b.dtype == _FP8 or is_16bit(b)
     assert (a_needs_q and scale_a is None) or (a.dtype == torch.int8 and scale_a is not None), \
@@ -49,9 +49,9 @@ def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype):
     if b_needs_q:
         b, scale_b = _rotate_quant(b)
     if bias is not None:
-        out = _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
     else:
-        out = _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype)
+        out = _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
     return out, b, scale_b
 
 
@@ -83,11 +83,15 @@ class Q8LinearFunc(torch.autograd.Function):
 
 def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
               scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
-              fuse_gelu: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """a [..., K] x b [N, K] -> [batch, M, N] through the int8 GEMM; out_dtype None -> e4m3 (as the reference)."""
+              fuse_gelu: bool = False, out_dtype: Optional[torch.dtype] = None,
+              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [..., K] x b [N, K] -> [batch, M, N] through the int8 GEMM; out_dtype None -> e4m3 (as the reference).
+    `residual` (bfloat16, the output's shape, out_dtype bfloat16) returns `residual + linear(a)` with the addition done
+    in the GEMM's epilogue: the bits of the separate bfloat16 addition."""
     if _needs_grad(a):
-        return Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
-    return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)[0]
+        out = Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+        return out if residual is None else out + residual.reshape(out.shape)
+    return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual)[0]
 
 
 # ----------------------------------------------------------------------------- fp8

@@ -213,22 +213,29 @@ def test_ltx_transformer_block_matches_oracle(dev):
     # the comparison cannot pass by both runs taking the same path.
     from q8_kernels_amd.modules import Attention
     impl, calls = _C().norm_mod_fht_quant, []
+    mm_impl, with_residual = _C().q8_mm_bias, []
     def counted(*a, **k):
         calls.append(1)
         return impl(*a, **k)
+    def counted_mm(*a, **k):
+        if k.get("residual") is not None:
+            with_residual.append(1)
+        return mm_impl(*a, **k)
     run = lambda: blk(hidden.to(dev), (cos.to(dev), sin.to(dev)), None, text.to(dev), lens.to(dev),  # noqa: E731
                       timestep.to(dev), attn_type="q8_kernels")
     try:
-        _C().norm_mod_fht_quant = counted
+        _C().norm_mod_fht_quant, _C().q8_mm_bias = counted, counted_mm
         with torch.no_grad():
             again = run()
         assert len(calls) == 2, f"fused prologue ran {len(calls)} times, expected 2 (attn1 and feed-forward)"
+        assert len(with_residual) == 1, f"{len(with_residual)} GEMMs carried a residual, expected 1 (attn2's output projection)"
         LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = False
         with torch.no_grad():
             seq = run()
         assert len(calls) == 2, "the operator-by-operator path called the fused prologue"
+        assert len(with_residual) == 1, "the operator-by-operator path added a residual inside a GEMM"
     finally:
-        _C().norm_mod_fht_quant = impl
+        _C().norm_mod_fht_quant, _C().q8_mm_bias = impl, mm_impl
         LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = True
     assert_bit_equal(got, again, "fused block, second run")
     assert_bit_equal(got, seq, "fused block vs operator sequence")
