@@ -9,7 +9,7 @@ The reference ships no tests or golden vectors, so each function is pinned in te
 independent closed forms (scipy Hadamard matrix, brute-force e4m3 rounding tables, exact integer matmul,
 float64 softmax, complex-number rotation ...).
 
-Pinning status (also listed in DESIGN.md):
+Pinning status:
   pinned by closed forms ....... e4m3 casts, ref_fht, ref_quant, ref_gemm_i32, ref_gemm_fp8_acc,
                                  ref_epilogue, ref_rms_norm, ref_rope, ref_attention, ref_freqs_cis,
                                  ref_fma (exact rational arithmetic), ref_gelu_backward, ref_rms_norm_backward,
