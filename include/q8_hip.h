@@ -248,6 +248,22 @@ int q8_gemm_residual(const void* A, const void* B, const float* bias, const floa
 int q8_gemm_set_config(int cfg);
 
 /*
+ * Which kernel the most recent q8_gemm / q8_gemm_residual / q8_gemm_i32 call of the calling thread launched
+ * (0 before the first call): one of the Q8_GEMM_KERNEL_* values, Q8_GEMM_KERNEL_RESIDUAL or-ed in when the residual
+ * was added in the epilogue. For tests, so that a test of a pinned kernel can tell that the call did not fall back
+ * to another one; no counterpart in the reference.
+ */
+enum {
+    Q8_GEMM_KERNEL_PIPE256 = 1,    /* pipelined 256x256 tiles, one tile per workgroup */
+    Q8_GEMM_KERNEL_TILE128 = 2,    /* 128x128 tiles                                    */
+    Q8_GEMM_KERNEL_PLAIN256 = 3,   /* plain 256x256 tiles                              */
+    Q8_GEMM_KERNEL_PERSIST256 = 4, /* persistent, 256-row tiles                        */
+    Q8_GEMM_KERNEL_PERSIST192 = 5, /* persistent, 192-row tiles                        */
+    Q8_GEMM_KERNEL_RESIDUAL = 16
+};
+int q8_gemm_last_kernel(void);
+
+/*
  * Raw int32 accumulators of the int8 GEMM, C[m,n] = sum_k A[m,k]*B[n,k], for bit-exact checks.
  * Same mainloop as q8_gemm with in_dtype = Q8_I8 (csrc/gemm/q8_matmul.cu:109-, accumulators
  * before the float conversion at q8_matmul_bias.cu:315-320).

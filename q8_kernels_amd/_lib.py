@@ -43,6 +43,7 @@ SIGNATURES = {
     "q8_gemm_i32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "q8_gemm_set_config": (_i, [_i]),
     "q8_attn_set_config": (_i, [_i]),
+    "q8_gemm_last_kernel": (_i, []),
     "q8_attn_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i64, _f, _i, _i, _vp]),
 }
 

@@ -152,8 +152,12 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
     }
 }
 
+// which kernel the last q8_gemm* call of this thread launched (q8_gemm_last_kernel)
+static thread_local int g_last_kernel = 0;
+
 template <class C, int OUT, bool GELU>
 static int launch_gemm(const GemmParams& p, hipStream_t stream) {
+    g_last_kernel = (C::BM == 256) ? Q8_GEMM_KERNEL_PLAIN256 : Q8_GEMM_KERNEL_TILE128;
     const int tiles_m = (p.M + C::BM - 1) / C::BM, tiles_n = (p.N + C::BN - 1) / C::BN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     auto kern = gemm_kernel<C, OUT, GELU>;
@@ -185,6 +189,7 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
     const int tiles_m = (p.M + kPipeBM - 1) / kPipeBM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     auto kern = gemm_pipe_kernel<IN, OUT, GELU>;
+    g_last_kernel = Q8_GEMM_KERNEL_PIPE256;
     static thread_local bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPipeLds) !=
@@ -223,6 +228,7 @@ static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     const long total = (long)tiles_m * tiles_n * batch;
     if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
     auto kern = gemm_persist_kernel<IN, GELU, MT, RES>;
+    g_last_kernel = (MT == 4 ? Q8_GEMM_KERNEL_PERSIST256 : Q8_GEMM_KERNEL_PERSIST192) | (RES ? Q8_GEMM_KERNEL_RESIDUAL : 0);
     static thread_local bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPersistLds) !=
@@ -288,6 +294,8 @@ static int check_gemm(const char* who, const void* A, const void* B, const void*
 }  // namespace q8
 
 using namespace q8;
+
+extern "C" int q8_gemm_last_kernel(void) { return g_last_kernel; }
 
 extern "C" int q8_gemm_set_config(int cfg) {
     if (cfg == 43 || cfg == 44 || cfg == 40) { g_persist_mt = cfg - 40; return Q8_OK; }  // tuning: persistent tile height

@@ -56,8 +56,17 @@ def _check(got, q, k, v, scale, lens=None, sc=(None, None, None), what="", p_sca
         assert cosine(g, exact) >= 0.999, "%s: cosine %g" % (what, cosine(g, exact))
 
 
+@pytest.fixture(params=[0, 1, 2], ids=["8waves_x32q", "4waves_x64q", "4waves_x32q"])
+def attn_cfg(request):
+    """every workgroup shape q8_attn_set_config offers (the library's default is the first)"""
+    from q8_kernels_amd import _lib
+    _lib.check(_lib.lib().q8_attn_set_config(request.param))
+    yield request.param
+    _lib.check(_lib.lib().q8_attn_set_config(0))
+
+
 @pytest.mark.parametrize("m,n", [(256, 64), (64, 128), (1, 1), (33, 17), (255, 100), (257, 200), (300, 640), (512, 1000)])
-def test_attention_shapes(dev, m, n):
+def test_attention_shapes(dev, attn_cfg, m, n):
     q, k, v = _inputs(m * 1000 + n, 2, 3, m, n)
     got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16)
     assert got.shape == (2, 3, m, 64) and got.dtype == torch.bfloat16
@@ -75,7 +84,7 @@ def test_attention_fp8_output_default(dev):
 
 
 @pytest.mark.parametrize("lens", [[128, 16], [1, 64], [65, 127], [0, 100], [63, 200]])
-def test_attention_kv_length_mask(dev, lens):
+def test_attention_kv_length_mask(dev, attn_cfg, lens):
     n = 128
     q, k, v = _inputs(sum(lens), 2, 4, 200, n)
     kv_len = torch.tensor(lens, dtype=torch.int32)
@@ -113,7 +122,7 @@ def test_attention_reference_probability_range(dev):
     assert (dflt.cpu().double() - exact).abs().mean() < (ref_mode.cpu().double() - exact).abs().mean()
 
 
-def test_attention_per_token_scales(dev):
+def test_attention_per_token_scales(dev, attn_cfg):
     g = torch.Generator().manual_seed(9)
     b, h, m, n = 2, 2, 150, 333
     qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)

@@ -19,6 +19,27 @@ def _set_cfg(c):
     _lib.check(_lib.lib().q8_gemm_set_config(c))
 
 
+K_PIPE256, K_TILE128, K_PLAIN256, K_PERSIST256, K_PERSIST192, K_RESIDUAL = 1, 2, 3, 4, 5, 16  # q8_gemm_last_kernel
+
+
+def _last_kernel():
+    from q8_kernels_amd import _lib
+    return _lib.lib().q8_gemm_last_kernel()
+
+
+def _kernels_for(cfg, n, k, bf16_out=True):
+    """The kernels a call may launch under q8_gemm_set_config(cfg): the pins 1 and 2 always hold; 4 means the
+    persistent kernel for the shapes it takes (bf16 output, N % 8 == 0, K a multiple of 128 above 256) and the
+    per-tile pipelined kernel otherwise. Asserted after the calls below so that a test of a pinned kernel cannot
+    pass on a silent fall-back to another one."""
+    if cfg == 1:
+        return {K_PIPE256}
+    if cfg == 2:
+        return {K_TILE128}
+    eligible = bf16_out and n % 8 == 0 and k > 256 and k % 128 == 0
+    return {K_PERSIST256, K_PERSIST192} if eligible else {K_PIPE256}
+
+
 @pytest.fixture(params=[1, 2, 4], ids=["tile256", "tile128", "persistent256"])
 def tile_cfg(request):
     _set_cfg(request.param)
@@ -48,6 +69,7 @@ def test_int8_accumulators_bit_exact(dev, tile_cfg, mnk):
     g = torch.Generator().manual_seed(m * 7 + n * 3 + k)
     a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
     got = _C().q8_mm_i32(a.to(dev), b.to(dev))
+    assert _last_kernel() in _kernels_for(tile_cfg, n, k, bf16_out=False)
     assert_bit_equal(got, O.ref_gemm_i32(a, b), "int32 acc %s" % (mnk,))
 
 
@@ -98,6 +120,7 @@ def test_mm_epilogue_vs_oracle(dev, tile_cfg, in_dtype, fuse_gelu, with_bias):
     args = (a.to(dev), b.to(dev)) + ((bias.to(dev),) if with_bias else ()) + (sa.to(dev), sb.to(dev), fuse_gelu)
     fn = mmb if with_bias else mm
     got = fn(*args, torch.bfloat16)
+    assert _last_kernel() in _kernels_for(tile_cfg, n, k), "kernel %d under config %d" % (_last_kernel(), tile_cfg)
     assert got.shape == (1, m, n)
     acc = O.ref_gemm_i32(a, b).double() if in_dtype == "i8" else O.ref_gemm_fp8_acc(a, b)
     v = acc * (sa[:, None] * sb[None, :]).double() + (bias.double() if with_bias else 0)
@@ -132,6 +155,7 @@ def test_mm_batch_broadcast(dev, tile_cfg):
     cases = [(a3, b3[0], sa3, sb3[0]), (a3[0], b3, sa3[0], sb3), (a3, b3, sa3, sb3), (a3[1], b3[2], sa3[1], sb3[2])]
     for a, b, sa, sb in cases:
         got = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.contiguous().to(dev), sb.contiguous().to(dev), False, torch.bfloat16)
+        assert _last_kernel() in _kernels_for(tile_cfg, n, k)
         want = O.ref_q8_mm(a, b, bias, sa, sb, False, torch.bfloat16)
         assert got.shape == want.shape
         diff = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
@@ -156,6 +180,7 @@ def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu, tile_r
     _set_cfg(tile_rows)  # force the 192- or the 256-row tile of the persistent kernel
     try:
         got = _C().q8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.to(dev), sb.to(dev), fuse_gelu, torch.bfloat16)
+        assert _last_kernel() == (K_PERSIST192 if tile_rows == 43 else K_PERSIST256)
     finally:
         _set_cfg(40)
         _set_cfg(0)
@@ -184,7 +209,12 @@ def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu):
     _set_cfg(4)
     try:
         plain = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
+        assert _last_kernel() in _kernels_for(4, n, k)
         fused = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16, residual=res)
+        if k % 128 == 0:  # added in the persistent kernel's epilogue
+            assert _last_kernel() in {K_PERSIST256 | K_RESIDUAL, K_PERSIST192 | K_RESIDUAL}
+        else:             # the GEMM without residual, then a separate addition
+            assert _last_kernel() == K_PIPE256
     finally:
         _set_cfg(0)
     assert_bit_equal(fused, plain + res, "residual epilogue")
