@@ -149,3 +149,13 @@ def test_weight_converter_key_mapping():
     assert converted_key(p + "attn2.to_k.weight") == (p + "attn2.to_k.weight", "quantize")
     assert converted_key(p + "ff.net.0.proj.weight") == (p + "ff.act.proj.weight", "quantize")
     assert converted_key(p + "ff.net.2.bias") == (p + "ff.proj_down.bias", "fp32")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 exits with a message that says why (nothing here spans GPUs)."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and "--gpus 2" in r.stderr
+    assert r.stdout.strip() == ""

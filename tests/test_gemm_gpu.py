@@ -165,6 +165,32 @@ def test_mm_batch_broadcast(dev, tile_cfg):
 @pytest.mark.parametrize("case", [(1, 1, 4352, 4096, 384), (3, 1, 1100, 4600, 512), (1, 2, 2300, 2816, 640)])
 @pytest.mark.parametrize("fuse_gelu", [False, True])
 @pytest.mark.parametrize("tile_rows", [43, 44], ids=["rows192", "rows256"])
+def test_persistent_kernel_many_tiles_fp8(dev, case, fuse_gelu, tile_rows):
+    """The same walk over many tiles, ragged edges and batches with e4m3 operands (fp32 accumulation in MFMA order
+    against the oracle's float64: the tolerance of the other fp8 checks)."""
+    ba, bb, m, n, k = case
+    g = torch.Generator().manual_seed(m + n + 5)
+    a = O.e4m3_c10(torch.randn(*((ba, m, k) if ba > 1 else (m, k)), generator=g) * 50)
+    b = O.e4m3_c10(torch.randn(*((bb, n, k) if bb > 1 else (n, k)), generator=g) * 50)
+    sa = torch.rand(ba * m, generator=g) * 1e-2 + 1e-4
+    sb = torch.rand(bb * n, generator=g) * 1e-2 + 1e-4
+    bias = torch.randn(n, generator=g)
+    _set_cfg(4)
+    _set_cfg(tile_rows)
+    try:
+        got = _C().fp8_mm_bias(a.to(dev), b.to(dev), bias.to(dev), sa.to(dev), sb.to(dev), fuse_gelu, torch.bfloat16)
+        assert _last_kernel() == (K_PERSIST192 if tile_rows == 43 else K_PERSIST256)
+    finally:
+        _set_cfg(40)
+        _set_cfg(0)
+    want = O.ref_fp8_mm(a, b, bias, sa, sb, fuse_gelu, torch.float64)
+    assert got.shape == want.shape
+    _check_float_out(got, want, "fp8 persistent %s" % (case,))
+
+
+@pytest.mark.parametrize("case", [(1, 1, 4352, 4096, 384), (3, 1, 1100, 4600, 512), (1, 2, 2300, 2816, 640)])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+@pytest.mark.parametrize("tile_rows", [43, 44], ids=["rows192", "rows256"])
 def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu, tile_rows):
     """More 256x256 tiles than CUs (272, 270 and 198+ with ragged edges and batch broadcast), so that workgroups of the
     persistent kernel cross tile and batch boundaries; int8 operands make the accumulators exact, the epilogue
@@ -195,7 +221,8 @@ def test_persistent_kernel_many_tiles_per_workgroup(dev, case, fuse_gelu, tile_r
 
 @pytest.mark.parametrize("case", [(1, 1, 2300, 2816, 640), (2, 1, 1100, 4608, 384), (1, 1, 200, 264, 208)])
 @pytest.mark.parametrize("fuse_gelu", [False, True])
-def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu):
+@pytest.mark.parametrize("tile_rows", [40, 43, 44], ids=["rows_auto", "rows192", "rows256"])
+def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu, tile_rows):
     """out = residual + linear(a): the fused epilogue (first two cases, persistent kernel) and the fallback (last case,
     K not a multiple of 128) both give the bits of the bf16 GEMM followed by a bf16 addition."""
     ba, bb, m, n, k = case
@@ -207,15 +234,18 @@ def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu):
     bias = torch.randn(n, generator=g).to(dev)
     res = torch.randn(ba, m, n, generator=g).to(torch.bfloat16).to(dev)
     _set_cfg(4)
+    _set_cfg(tile_rows)
     try:
         plain = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
         assert _last_kernel() in _kernels_for(4, n, k)
         fused = _C().q8_mm_bias(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16, residual=res)
         if k % 128 == 0:  # added in the persistent kernel's epilogue
-            assert _last_kernel() in {K_PERSIST256 | K_RESIDUAL, K_PERSIST192 | K_RESIDUAL}
+            want_kernels = {40: {K_PERSIST256, K_PERSIST192}, 43: {K_PERSIST192}, 44: {K_PERSIST256}}[tile_rows]
+            assert _last_kernel() in {kk | K_RESIDUAL for kk in want_kernels}
         else:             # the GEMM without residual, then a separate addition
             assert _last_kernel() == K_PIPE256
     finally:
+        _set_cfg(40)
         _set_cfg(0)
     assert_bit_equal(fused, plain + res, "residual epilogue")
 
