@@ -14,6 +14,9 @@ Q8_I8, Q8_E4M3, Q8_BF16, Q8_F16, Q8_F32 = 0, 1, 2, 3, 4
 Q8_QUANT_RNE, Q8_QUANT_SCALE_DIV = 1, 2
 Q8_V_DS, Q8_V_SD = 0, 1
 Q8_ATTN_SUM_ROUNDED_P, Q8_ATTN_P_UNIT_RANGE, Q8_ATTN_O_TOKEN_MAJOR = 1, 2, 4
+# values of q8_gemm_last_kernel (tests)
+Q8_GEMM_KERNEL_PIPE256, Q8_GEMM_KERNEL_TILE128, Q8_GEMM_KERNEL_PLAIN256 = 1, 2, 3
+Q8_GEMM_KERNEL_PERSIST256, Q8_GEMM_KERNEL_PERSIST192, Q8_GEMM_KERNEL_RESIDUAL = 4, 5, 16
 
 _c = ctypes
 _vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float

@@ -33,7 +33,9 @@ def test_header_enums_match_python_constants():
     from q8_kernels_amd import _lib
     text = open(HEADER).read()
     for name in ("Q8_I8", "Q8_E4M3", "Q8_BF16", "Q8_F16", "Q8_F32", "Q8_QUANT_RNE", "Q8_QUANT_SCALE_DIV",
-                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR"):
+                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR",
+                 "Q8_GEMM_KERNEL_PIPE256", "Q8_GEMM_KERNEL_TILE128", "Q8_GEMM_KERNEL_PLAIN256", "Q8_GEMM_KERNEL_PERSIST256",
+                 "Q8_GEMM_KERNEL_PERSIST192", "Q8_GEMM_KERNEL_RESIDUAL"):
         m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
         assert m, name
         assert int(m.group(1)) == getattr(_lib, name), name
@@ -149,6 +151,34 @@ def test_weight_converter_key_mapping():
     assert converted_key(p + "attn2.to_k.weight") == (p + "attn2.to_k.weight", "quantize")
     assert converted_key(p + "ff.net.0.proj.weight") == (p + "ff.act.proj.weight", "quantize")
     assert converted_key(p + "ff.net.2.bias") == (p + "ff.proj_down.bias", "fp32")
+
+
+def test_missing_library_is_an_error_not_a_fallback():
+    """A fresh interpreter with the library path pointed at nothing: the loader (and with it every call that reaches
+    it) raises the build hint, and no operator hands back a result for CPU tensors instead. What a machine without a
+    GPU cannot show - an operator on a device tensor reaching the loader - is test_api_gpu.py's version of this."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, torch\n"
+        "sys.path.insert(0, %r)\n"
+        "from q8_kernels_amd import _lib\n"
+        "_lib.LIB_PATH = '/nonexistent/libq8_hip.so'\n"
+        "from q8_kernels_amd import _C\n"
+        "x = torch.zeros(4, 64, dtype=torch.bfloat16)\n"
+        "for name, fn in (('loader', _lib.lib), ('device_info', _lib.device_info), ('quant_cpu', lambda: _C.tokenwise_quant(x, None))):\n"
+        "    try:\n"
+        "        fn()\n"
+        "    except RuntimeError as e:\n"
+        "        print(name, '|', e)\n"
+        "    else:\n"
+        "        print(name, '| RETURNED')\n" % ROOT)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = dict(line.split(" | ", 1) for line in r.stdout.strip().splitlines())
+    assert "no fallback" in got["loader"] and "/nonexistent/libq8_hip.so" in got["loader"]
+    assert "no fallback" in got["device_info"]
+    assert "CUDA" in got["quant_cpu"] and "RETURNED" not in got["quant_cpu"]
 
 
 def test_bench_refuses_more_than_one_gpu():

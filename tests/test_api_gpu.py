@@ -144,3 +144,34 @@ def test_dit_block_matches_oracle_block(dev):
     # end to end in bf16 with requantisation between ops: small differences get re-rounded along the way
     assert cosine(got.cpu(), want) > 0.9995
     assert (got.cpu().double() - want.double()).abs().max() <= 0.05 * want.double().abs().max()
+
+
+def test_operator_on_a_device_tensor_raises_when_the_library_is_missing(dev):
+    """A fresh interpreter whose library path points at nothing: an operator given a device tensor reaches the
+    loader and raises its build hint; there is no other path that could compute the result."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, torch\n"
+        "sys.path.insert(0, %r)\n"
+        "from q8_kernels_amd import _lib\n"
+        "_lib.LIB_PATH = '/nonexistent/libq8_hip.so'\n"
+        "from q8_kernels_amd import _C\n"
+        "import q8_kernels_amd.functional as F\n"
+        "x = torch.zeros(4, 64, dtype=torch.bfloat16, device='cuda')\n"
+        "for name, fn in (('quant', lambda: _C.tokenwise_quant(x, None)), ('fht', lambda: _C.fast_hadamard_transform(x, 1.0, None)),\n"
+        "                 ('linear', lambda: F.linear.q8_linear(x, x, out_dtype=torch.bfloat16))):\n"
+        "    try:\n"
+        "        fn()\n"
+        "    except RuntimeError as e:\n"
+        "        print(name, '|', e)\n"
+        "    else:\n"
+        "        print(name, '| RETURNED')\n" % root)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = dict(line.split(" | ", 1) for line in r.stdout.strip().splitlines())
+    assert set(got) == {"quant", "fht", "linear"}
+    for name, msg in got.items():
+        assert "no fallback" in msg and "libq8_hip.so not found" in msg, (name, msg)

@@ -19,7 +19,9 @@ def _set_cfg(c):
     _lib.check(_lib.lib().q8_gemm_set_config(c))
 
 
-K_PIPE256, K_TILE128, K_PLAIN256, K_PERSIST256, K_PERSIST192, K_RESIDUAL = 1, 2, 3, 4, 5, 16  # q8_gemm_last_kernel
+from q8_kernels_amd._lib import (Q8_GEMM_KERNEL_PERSIST192 as K_PERSIST192, Q8_GEMM_KERNEL_PERSIST256 as K_PERSIST256,  # noqa: E402
+                                 Q8_GEMM_KERNEL_PIPE256 as K_PIPE256, Q8_GEMM_KERNEL_RESIDUAL as K_RESIDUAL,
+                                 Q8_GEMM_KERNEL_TILE128 as K_TILE128)
 
 
 def _last_kernel():
