@@ -175,3 +175,40 @@ def test_operator_on_a_device_tensor_raises_when_the_library_is_missing(dev):
     assert set(got) == {"quant", "fht", "linear"}
     for name, msg in got.items():
         assert "no fallback" in msg and "libq8_hip.so not found" in msg, (name, msg)
+
+
+def test_operators_run_on_the_current_stream(dev):
+    """The input of each operator is produced on a side stream behind tens of milliseconds of other work, and the
+    operator is called on that stream without any synchronisation in between. Launched anywhere else (torch's side
+    streams do not wait for the default stream, nor it for them) it would read the input before it is written."""
+    from q8_kernels_amd import _C
+    g = torch.Generator().manual_seed(11)
+    src = torch.randn(512, 2048, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(1024, 2048, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    q = torch.randn(1, 4, 256, 64, generator=g).to(torch.bfloat16).to(dev)
+    wq, ws = _C.tokenwise_quant(w, torch.int8)
+    want_codes, want_scales = _C.tokenwise_quant(src, torch.int8)
+    want_mm = _C.q8_mm(want_codes, wq, want_scales, ws, False, torch.bfloat16)
+    q8 = _C.fast_hadamard_transform(q, 0.125, E4M3)
+    v8 = q8.transpose(2, 3).contiguous()
+    want_attn = _C.flash_attention(q8, q8, v8, 1.0, None, out_dtype=torch.bfloat16)
+    busy = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+    x = torch.zeros_like(src)
+    qx = torch.zeros_like(q8.view(torch.uint8))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    assert side.cuda_stream != torch.cuda.default_stream().cuda_stream
+    with torch.cuda.stream(side):
+        for _ in range(25):
+            busy @ busy                       # roughly a millisecond each
+        x.copy_(src)
+        qx.copy_(q8.view(torch.uint8))
+        codes, scales = _C.tokenwise_quant(x, torch.int8)
+        mm = _C.q8_mm(codes, wq, scales, ws, False, torch.bfloat16)
+        qs = qx.view(E4M3)
+        attn = _C.flash_attention(qs, qs, qs.transpose(2, 3).contiguous(), 1.0, None, out_dtype=torch.bfloat16)
+    side.synchronize()
+    assert_bit_equal(codes, want_codes, "quantizer on a side stream")
+    assert_bit_equal(scales, want_scales, "quantizer scales on a side stream")
+    assert_bit_equal(mm, want_mm, "GEMM on a side stream")
+    assert_bit_equal(attn, want_attn, "attention on a side stream")
