@@ -212,3 +212,65 @@ def test_operators_run_on_the_current_stream(dev):
     assert_bit_equal(scales, want_scales, "quantizer scales on a side stream")
     assert_bit_equal(mm, want_mm, "GEMM on a side stream")
     assert_bit_equal(attn, want_attn, "attention on a side stream")
+
+
+def _replays_match_eager(step, inputs, make_inputs):
+    """Captures step() into a HIP graph once and replays it with new contents in the (static) input tensors; between
+    the replays the same step runs eagerly on separate tensors, with synchronisations, and every replay has to give
+    the eager bits. The C entry points allocate nothing, wait for nothing and clear no memory, so a captured block is
+    a pure sequence of kernel launches."""
+    with torch.no_grad():
+        for _ in range(3):
+            step(*inputs)                      # first calls outside the capture (per-kernel LDS attribute set-up)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = step(*inputs)
+        for rep in range(4):
+            fresh = make_inputs(100 + rep)
+            for dst, src in zip(inputs, fresh):
+                dst.copy_(src)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.clone()
+            want = step(*fresh)
+            torch.cuda.synchronize()
+            assert_bit_equal(got, want, "graph replay %d" % rep)
+
+
+def test_dit_block_replays_from_a_graph(dev):
+    from q8_kernels_amd.blocks import Fp8DiTBlock
+    b, s, t, d = 2, 512, 64, 2048
+    blk = Fp8DiTBlock(device=dev).init_random()
+    grid = torch.stack(torch.meshgrid(torch.arange(8), torch.arange(8), torch.arange(8), indexing="ij")).reshape(3, -1).float() / 8
+    cos, sin = (x.to(dev) for x in O.ref_freqs_cis(grid[None].repeat(b, 1, 1), d))
+    lens = torch.tensor([t, 33], dtype=torch.int32, device=dev)
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(b, s, d, generator=g).to(torch.bfloat16).to(dev), torch.randn(b, t, d, generator=g).to(torch.bfloat16).to(dev))
+
+    _replays_match_eager(lambda h, x: blk(h, x, (cos, sin), lens), make(1), make)
+
+
+def test_ltx_block_replays_from_a_graph(dev):
+    import torch.nn as nn
+    from q8_kernels_amd.blocks import LTXTransformerBlock
+    from q8_kernels_amd.modules import Q8Linear
+    torch.manual_seed(5)
+    dim, heads, hd, kv_dim, s_tok, s_txt = 512, 8, 64, 256, 384, 32
+    blk = LTXTransformerBlock(dim, heads, hd, kv_dim, bias=True, use_rope=True, norm_affine=False).to(dev)
+    for m in blk.modules():
+        if isinstance(m, Q8Linear):
+            q = Q8Linear.from_linear(nn.Linear(m.in_features, m.out_features).to(dev).to(torch.bfloat16))
+            m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    grid = torch.stack(torch.meshgrid(torch.arange(8), torch.arange(8), torch.arange(6), indexing="ij")).reshape(3, -1)
+    cos, sin = (x.to(dev) for x in O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim))
+    lens = torch.tensor([32, 9], dtype=torch.int32, device=dev)
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(2, s_tok, dim, generator=g).to(torch.bfloat16).to(dev), torch.randn(2, s_txt, kv_dim, generator=g).to(torch.bfloat16).to(dev),
+                (torch.randn(2, 1, 6 * dim, generator=g) * 0.3).to(dev))
+
+    _replays_match_eager(lambda h, x, ts: blk(h, (cos, sin), None, x, lens, ts, attn_type="q8_kernels"), make(1), make)
