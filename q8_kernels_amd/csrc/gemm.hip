@@ -155,21 +155,31 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
 // which kernel the last q8_gemm* call of this thread launched (q8_gemm_last_kernel)
 static thread_local int g_last_kernel = 0;
 
+// A kernel's dynamic LDS limit is a per-device attribute: it is set once per (thread, kernel, device). `done_dev` is
+// the caller's thread-local record of the device it was last set on.
+static int reserve_lds(const void* kern, int bytes, int& done_dev) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(Q8_ERR_LAUNCH, "q8_gemm: no current device");
+    }
+    if (done_dev == dev) return Q8_OK;
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", bytes);
+    }
+    done_dev = dev;
+    return Q8_OK;
+}
+
 template <class C, int OUT, bool GELU>
 static int launch_gemm(const GemmParams& p, hipStream_t stream) {
     g_last_kernel = (C::BM == 256) ? Q8_GEMM_KERNEL_PLAIN256 : Q8_GEMM_KERNEL_TILE128;
     const int tiles_m = (p.M + C::BM - 1) / C::BM, tiles_n = (p.N + C::BN - 1) / C::BN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     auto kern = gemm_kernel<C, OUT, GELU>;
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                C::LDS_BYTES) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", C::LDS_BYTES);
-        }
-        attr_set = true;
-    }
+    static thread_local int lds_dev = -1;
+    if (int st = reserve_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES, lds_dev)) return st;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(C::NT), C::LDS_BYTES, stream, p);
     return launch_status("q8_gemm");
 }
@@ -190,15 +200,8 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     auto kern = gemm_pipe_kernel<IN, OUT, GELU>;
     g_last_kernel = Q8_GEMM_KERNEL_PIPE256;
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPipeLds) !=
-            hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", kPipeLds);
-        }
-        attr_set = true;
-    }
+    static thread_local int lds_dev = -1;
+    if (int st = reserve_lds(reinterpret_cast<const void*>(kern), kPipeLds, lds_dev)) return st;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(512), kPipeLds, stream, p);
     return launch_status("q8_gemm");
 }
@@ -208,14 +211,20 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
 // 20 % charged to the smaller tile (measured: a 192-row round takes 0.90 of a 256-row round, not 0.75: it moves 17 %
 // more operand bytes per flop and pays the same epilogue and barrier overheads).
 static int persist_cus() {
-    static thread_local int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    static thread_local int cus = 0, cus_dev = -1;  // of the device the count was read on
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (cus_dev != dev) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
             (void)hipGetLastError();
             n = 256;
         }
         cus = n >= 8 ? (n / 8) * 8 : 8;  // a multiple of the 8 XCDs keeps every workgroup's tiles on one XCD
+        cus_dev = dev;
     }
     return cus;
 }
@@ -229,15 +238,8 @@ static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
     auto kern = gemm_persist_kernel<IN, GELU, MT, RES>;
     g_last_kernel = (MT == 4 ? Q8_GEMM_KERNEL_PERSIST256 : Q8_GEMM_KERNEL_PERSIST192) | (RES ? Q8_GEMM_KERNEL_RESIDUAL : 0);
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kPersistLds) !=
-            hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8_ERR_LAUNCH, "q8_gemm: cannot reserve %d bytes of LDS", kPersistLds);
-        }
-        attr_set = true;
-    }
+    static thread_local int lds_dev = -1;
+    if (int st = reserve_lds(reinterpret_cast<const void*>(kern), kPersistLds, lds_dev)) return st;
     const int cus = persist_cus();
     const int grid = total < cus ? (int)total : cus;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), kPersistLds, stream, p, tiles_m, tiles_n, (int)total);
