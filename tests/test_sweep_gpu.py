@@ -1,0 +1,82 @@
+"""Seeded random sweep of the bit-exact row operators against the oracle: dimensions anywhere in the documented range
+(multiples of 8 up to 32768, most of them not powers of two), odd row counts, all-zero rows, amplitudes from 1e-3 to
+1e4, both code types and both rounding rules. The fixed lists of the other test files name their cases; this one
+covers the combinations between them. A failure message carries everything needed to rebuild the case."""
+import random
+
+import pytest
+import torch
+
+from oracle import q8_oracle as O
+from tests.util import E4M3, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+def _C():
+    from q8_kernels_amd import _C as C
+    return C
+
+
+def _dim(rnd):
+    kind = rnd.random()
+    if kind < 0.35:
+        return rnd.choice([8, 16, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, 32768])
+    if kind < 0.8:
+        return 8 * rnd.randint(1, 1100)
+    return 8 * rnd.randint(1100, 4096)
+
+
+@pytest.mark.parametrize("sweep_seed", [11, 12, 13])
+def test_row_operators_random_shapes(dev, sweep_seed):
+    rnd = random.Random(sweep_seed)
+    for case in range(40):
+        op = rnd.choice(["quant", "quant", "fht", "fht", "fht_quant", "rope", "fma", "rms_quant"])
+        dim = _dim(rnd)
+        if op in ("rope", "fma") and dim > 8192:
+            dim = 8 * rnd.randint(1, 1024)
+        rows = rnd.choice([1, 2, 3, 5, 7, 17, 63, 64, 65, 130, 257]) if dim <= 8192 else rnd.choice([1, 2, 3, 5, 9])
+        seed = rnd.randint(0, 1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        amp = rnd.choice([1e-3, 1.0, 30.0, 1e4])
+        x = (torch.randn(rows, dim, generator=g) * amp).to(BF16)
+        if rnd.random() < 0.15:
+            x[rnd.randrange(rows)] = 0
+        out_type = rnd.choice([torch.int8, E4M3])
+        what = "sweep %d case %d: %s rows=%d dim=%d seed=%d amp=%g out=%s" % (sweep_seed, case, op, rows, dim, seed, amp, out_type)
+        if op == "quant":
+            rhe = rnd.random() < 0.3
+            codes, scales = _C().tokenwise_quant(x.to(dev), out_type, round_half_even=rhe)
+            want_codes, want_scales = O.ref_quant(x, out_type, round_half_even=rhe)
+            assert_bit_equal(codes, want_codes, what + " rne=%s codes" % rhe)
+            assert_bit_equal(scales, want_scales, what + " scales")
+        elif op == "fht":
+            scale = rnd.choice([1.0, dim ** -0.5, 0.125])
+            to = rnd.choice([BF16, E4M3])
+            assert_bit_equal(_C().fast_hadamard_transform(x.to(dev), scale, to), O.ref_fht(x, scale, to), what + " scale=%g to=%s" % (scale, to))
+        elif op == "fht_quant":
+            codes, scales = _C().fht_quant(x.to(dev), dim ** -0.5, out_type, mid_type=BF16)
+            want_codes, want_scales = O.ref_quant(O.ref_fht(x, dim ** -0.5, BF16), out_type)
+            assert_bit_equal(codes, want_codes, what + " codes")
+            assert_bit_equal(scales, want_scales, what + " scales")
+        elif op == "rope":
+            cos, sin = torch.randn(rows, dim, generator=g), torch.randn(rows, dim, generator=g)
+            assert_bit_equal(_C().rope(x.to(dev), cos.to(dev), sin.to(dev), None), O.ref_rope(x, cos, sin, None), what)
+        elif op == "fma":
+            b = rnd.choice([1, 2]) if rows >= 2 else 1
+            t = max(1, rows // b)
+            x3 = x[:b * t].reshape(b, t, dim).contiguous()
+            tm = rnd.choice([1, t])
+            yt, zt = rnd.choice([BF16, torch.float32]), rnd.choice([BF16, torch.float32])
+            y = (torch.randn(b, tm, dim, generator=g) * 0.3).to(yt)
+            z = torch.randn(b, tm, dim, generator=g).to(zt)
+            scale_add = rnd.choice([0.0, 1.0])
+            got = _C().fma_8bit(x3.to(dev), y.to(dev), z.to(dev), scale_add)
+            assert_bit_equal(got, O.ref_fma(x3, y, z, scale_add), what + " y=%s z=%s mod_rows=%d add=%g" % (yt, zt, tm, scale_add))
+        else:  # rms_quant: against the two separate HIP kernels (same summation order), as in test_fused_gpu.py
+            w = 1 + 0.1 * torch.randn(dim, generator=g)
+            codes, scales, _ = _C().rms_norm_quant(x.to(dev), w.to(dev), out_type)
+            want_codes, want_scales = _C().tokenwise_quant(_C().rms_norm(x.to(dev), w.to(dev), BF16)[0], out_type)
+            assert_bit_equal(codes, want_codes, what + " codes")
+            assert_bit_equal(scales, want_scales, what + " scales")
