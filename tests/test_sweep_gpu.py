@@ -80,3 +80,61 @@ def test_row_operators_random_shapes(dev, sweep_seed):
             want_codes, want_scales = _C().tokenwise_quant(_C().rms_norm(x.to(dev), w.to(dev), BF16)[0], out_type)
             assert_bit_equal(codes, want_codes, what + " codes")
             assert_bit_equal(scales, want_scales, what + " scales")
+
+
+def _gemm_cfg(c):
+    from q8_kernels_amd import _lib
+    _lib.check(_lib.lib().q8_gemm_set_config(c))
+
+
+@pytest.mark.parametrize("sweep_seed", [21, 22])
+def test_gemm_random_shapes(dev, sweep_seed):
+    """int32 accumulators of random (M, N, K) under every kernel pin: bit-exact. The persistent kernel's bf16 path on
+    random shapes it takes (N % 8 == 0, K a multiple of 128 above 256), with batches, both tile heights, GELU and the
+    residual epilogue: at most one bf16 ulp from the oracle (int8 operands make the accumulators exact), the residual
+    form bit-equal to the separate addition, and the persistent kernel is the one that ran."""
+    from q8_kernels_amd import _lib
+    rnd = random.Random(sweep_seed)
+    for case in range(30):
+        seed = rnd.randint(0, 1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        if rnd.random() < 0.6:
+            m, n, k = rnd.randint(1, 700), rnd.randint(1, 700), 16 * rnd.randint(1, 80)
+            cfg = rnd.choice([0, 1, 2, 3, 4])
+            a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+            b = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int8)
+            _gemm_cfg(cfg)
+            try:
+                got = _C().q8_mm_i32(a.to(dev), b.to(dev))
+            finally:
+                _gemm_cfg(0)
+            assert_bit_equal(got, O.ref_gemm_i32(a, b), "sweep %d case %d: acc m=%d n=%d k=%d cfg=%d seed=%d" % (sweep_seed, case, m, n, k, cfg, seed))
+            continue
+        m, n, k = rnd.randint(1, 3000), 8 * rnd.randint(1, 400), 128 * rnd.randint(3, 10)
+        ba, bb = rnd.choice([(1, 1), (1, 1), (2, 1), (1, 2)])
+        rows, gelu, with_res = rnd.choice([40, 43, 44]), rnd.random() < 0.5, rnd.random() < 0.3
+        a = torch.randint(-128, 128, ((ba, m, k) if ba > 1 else (m, k)), generator=g, dtype=torch.int8).to(dev)
+        b = torch.randint(-128, 128, ((bb, n, k) if bb > 1 else (n, k)), generator=g, dtype=torch.int8).to(dev)
+        sa = torch.rand(ba * m, generator=g) * 2e-3 + 1e-4
+        sb = torch.rand(bb * n, generator=g) * 2e-2 + 1e-3
+        bias = torch.randn(n, generator=g)
+        what = "sweep %d case %d: persistent m=%d n=%d k=%d batches=%d,%d rows=%d gelu=%s seed=%d" % (sweep_seed, case, m, n, k, ba, bb, rows, gelu, seed)
+        _gemm_cfg(4)
+        _gemm_cfg(rows)
+        try:
+            got = _C().q8_mm_bias(a, b, bias.to(dev), sa.to(dev), sb.to(dev), gelu, BF16)
+            assert _lib.lib().q8_gemm_last_kernel() in (_lib.Q8_GEMM_KERNEL_PERSIST256, _lib.Q8_GEMM_KERNEL_PERSIST192), what
+            if with_res:
+                res = torch.randn(got.shape, generator=g).to(BF16).to(dev)
+                fused = _C().q8_mm_bias(a, b, bias.to(dev), sa.to(dev), sb.to(dev), gelu, BF16, residual=res)
+                assert _lib.lib().q8_gemm_last_kernel() & _lib.Q8_GEMM_KERNEL_RESIDUAL, what
+                assert_bit_equal(fused, got + res, what + " residual")
+        finally:
+            _gemm_cfg(40)
+            _gemm_cfg(0)
+        want = O.ref_q8_mm(a.cpu(), b.cpu(), bias, sa, sb, gelu, BF16)
+        assert got.shape == want.shape, what
+        diff = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        # far in GELU's negative tail the oracle's float64 1 + tanh cancels to zero while the kernel keeps the tiny value
+        diff = torch.where((got.cpu().float() - want.float()).abs() <= 1e-7, torch.zeros_like(diff), diff)
+        assert int(diff.max()) <= 1, what + ": %d ulp" % int(diff.max())
