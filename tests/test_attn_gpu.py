@@ -209,3 +209,44 @@ def test_attention_rejects_bad_arguments(dev):
     q32 = O.e4m3_c10(torch.zeros(1, 1, 16, 32))
     with pytest.raises(Q8Error):
         _C().flash_attention(q32.to(dev), q32.to(dev), O.e4m3_c10(torch.zeros(1, 1, 32, 16)).to(dev), 0.125, None)
+
+
+@pytest.mark.parametrize("sweep_seed", [31, 32])
+def test_attention_random_shapes(dev, sweep_seed):
+    """Seeded sweep between the fixed cases above: random query and key counts (ragged against the 32-query and
+    64-key tiles), batch and head counts, key-length masks including 0 and the full length, direct casts or per-token
+    scales, logit spreads, every workgroup shape; the same bounds as everywhere in this file."""
+    import random
+    from q8_kernels_amd import _lib
+    rnd = random.Random(sweep_seed)
+    for case in range(14):
+        b, h = rnd.choice([(1, 1), (1, 3), (2, 2), (3, 1)])
+        m, n = rnd.randint(1, 420), rnd.randint(1, 900)
+        cfg = rnd.choice([0, 1, 2])
+        scaled, masked = rnd.random() < 0.4, rnd.random() < 0.6
+        std = rnd.choice([0.5, 1.0, 2.0])
+        seed = rnd.randint(0, 1 << 30)
+        what = "sweep %d case %d: b=%d h=%d m=%d n=%d cfg=%d scaled=%s masked=%s std=%g seed=%d" % (
+            sweep_seed, case, b, h, m, n, cfg, scaled, masked, std, seed)
+        g = torch.Generator().manual_seed(seed)
+        lens = None
+        if masked:
+            lens = torch.tensor([rnd.choice([0, 1, n, rnd.randint(1, n)]) for _ in range(b)], dtype=torch.int32)
+        if scaled:
+            qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2) * std
+            kf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 4 + 0.2)
+            vf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 2 + 0.5)
+            (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+            sc = (sq, sk, sv)
+        else:
+            q, k, v = _inputs(seed, b, h, m, n, std)
+            sc = (None, None, None)
+        _lib.check(_lib.lib().q8_attn_set_config(cfg))
+        try:
+            got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None if lens is None else lens.to(dev),
+                                       out_dtype=torch.bfloat16,
+                                       **({"q_scales": sq.to(dev), "k_scales": sk.to(dev), "v_scales": sv.to(dev)} if scaled else {}))
+        finally:
+            _lib.check(_lib.lib().q8_attn_set_config(0))
+        assert got.shape == (b, h, m, 64), what
+        _check(got, q, k, v, 0.125, lens, sc, what=what)
