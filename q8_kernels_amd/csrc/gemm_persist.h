@@ -10,7 +10,8 @@
 //     stages of the next tile are already on their way, and they land while the epilogue of the finished tile runs.
 //   * The epilogue therefore may not touch the two stage buffers: every wave stages its results through 2 KiB of its
 //     own (16 rows x 128 B per round, two rounds per 32-row MFMA tile, chunks swizzled by (row >> 1) & 7) and writes
-//     8 complete 128-byte lines per store instruction. All LDS traffic of the epilogue is inline assembly with its own
+//     8 complete 128-byte lines per store instruction. (With GELU fused and no residual the lanes store their chunks
+//     directly instead, see the epilogue.) All LDS traffic of the epilogue is inline assembly with its own
 //     lgkmcnt waits; the stores are never waited for, they drain under the next tile's MFMAs.
 //   * sa / sb / bias of a tile are copied to LDS (double-buffered) when the copy side enters the tile.
 //   * Every wave issues the same number of copy instructions per stage (8, and 2 more in a stage where the copy
@@ -303,6 +304,22 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     }
                     outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
                 }
+            if constexpr (GELU && !RES) {
+                // With GELU the epilogue is bound by its arithmetic, and the round trips through the staging buffer
+                // below only add latency to it: the lane's four 16-byte chunks of row 32 i + r32 go straight to
+                // memory, 32 contiguous bytes per row and instruction (the four instructions complete the row's
+                // 128-byte line within a few hundred cycles, so the L2 merges them). Measured 2.5-3.3 % faster per
+                // launch than the staged form on the GELU shapes and 1-4 % slower without GELU, where the stores
+                // are what the epilogue waits for and whole lines per instruction pay off.
+                const int m = mw0 + 32 * i + r32;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int wp = 0; wp < 2; ++wp) {
+                        const int n = nw0 + 32 * t + 16 * wp + 8 * h;
+                        if (m < M && n < N) *reinterpret_cast<v4u*>(cbase + (size_t)m * N + n) = outc[t][wp];
+                    }
+            } else {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 // rows 16 half .. 16 half + 15 of the MFMA tile: their lanes write, then all lanes store 16 full rows
@@ -338,6 +355,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     const int n = nw0 + (lane_e & 7) * 8;
                     if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * N + n) = w[j];
                 }
+            }
             }
         }
         if (item + 1 < count) cur = item_of(item + 1);
