@@ -297,3 +297,38 @@ def test_mm_rejects_bad_arguments(dev):
     with pytest.raises(RuntimeError):
         _C().q8_mm(torch.zeros(2, 16, 32, dtype=torch.int8, device=dev), torch.zeros(3, 16, 32, dtype=torch.int8, device=dev),
                    torch.ones(32, device=dev), torch.ones(48, device=dev), False, torch.bfloat16)
+
+
+# ------------------------------------------------------------------ operand sizes around 4 GiB
+
+@pytest.mark.parametrize("rows_over", [-64, 64], ids=["just_below_4GiB_persistent", "above_4GiB_per_tile"])
+def test_operand_around_4_gib(dev, rows_over):
+    """A [M, 2048] int8 with M * K = 4 GiB -/+ 128 KiB. Below the limit the persistent kernel takes it and its 32-bit
+    byte offsets run up to just under 2^32 (far beyond 2^31: they have to be treated as unsigned); above it the
+    dispatcher has to fall back to the per-tile kernel with its 64-bit addresses. Rows at the start, around the 2 GiB
+    mark and at the end are checked against the oracle (int8 operands, exact accumulators: at most one bf16 ulp)."""
+    k, n = 2048, 256
+    m = (1 << 32) // k + rows_over
+    torch.manual_seed(3)
+    a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device=dev)
+    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device=dev)
+    sa = torch.rand(m, device=dev) * 2e-3 + 1e-4
+    sb = torch.rand(n, device=dev) * 2e-2 + 1e-3
+    bias = torch.randn(n, device=dev)
+    assert a.numel() == m * k and (a.numel() < (1 << 32)) == (rows_over < 0)
+    out = _C().q8_mm_bias(a, b, bias, sa, sb, False, torch.bfloat16)
+    kernel = _last_kernel()
+    torch.cuda.synchronize()
+    if rows_over < 0:
+        assert kernel in (K_PERSIST256, K_PERSIST192), kernel
+    else:
+        assert kernel == K_PIPE256, kernel
+    assert out.shape == (1, m, n)
+    half = (1 << 31) // k
+    for lo in (0, half - 150, m - 300):
+        rows = slice(lo, lo + 300)
+        want = O.ref_q8_mm(a[rows].cpu(), b.cpu(), bias.cpu(), sa[rows].cpu(), sb.cpu(), False, torch.bfloat16)
+        diff = (out[0, rows].cpu().view(torch.int16).int() - want[0].view(torch.int16).int()).abs()
+        assert int(diff.max()) <= 1, "rows %d..%d: %d ulp" % (lo, lo + 300, int(diff.max()))
+    del a, out
+    torch.cuda.empty_cache()
