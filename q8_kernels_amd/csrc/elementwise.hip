@@ -247,6 +247,7 @@ extern "C" int q8_rmsnorm_backward(const void* y, int y_dtype, const float* rstd
     const int N = pow2_ceil(dim);
     Q8_ROW_SHAPE_SWITCH(N, {
         const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+        if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_rmsnorm_backward: too many rows for one launch");
         hipLaunchKernelGGL((rmsnorm_backward_kernel<LANES, CH>), dim3((unsigned)grid), dim3(kBlock), 0, stream, y, y_dtype, rstd,
                            grad, grad_dtype, w, out, out_dtype, rows, dim);
     })

@@ -450,6 +450,7 @@ extern "C" int q8_fht_quant_rows(const void* x, int x_dtype, void* codes, int co
     Q8_FUSED_SWITCH(x_dtype, code_dtype, mid_dtype, {
         Q8_ROW_SHAPE_SWITCH(N, {
             const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_fht_quant_rows: too many rows for one launch");
             hipLaunchKernelGGL((fht_quant_kernel<LANES, CH, IN, OUT, MID>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
                                x, codes, scales, rows, dim, fht_scale, flags);
         })
@@ -469,6 +470,7 @@ extern "C" int q8_rmsnorm_quant_rows(const void* x, int x_dtype, const float* w,
     Q8_FUSED_SWITCH(x_dtype, code_dtype, mid_dtype, {
         Q8_ROW_SHAPE_SWITCH(N, {
             const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_rmsnorm_quant_rows: too many rows for one launch");
             hipLaunchKernelGGL((rmsnorm_quant_kernel<LANES, CH, IN, OUT, MID>), dim3((unsigned)grid), dim3(kBlock), 0,
                                stream, x, w, codes, scales, rstd, rows, dim, eps, flags);
         })
@@ -497,6 +499,7 @@ extern "C" int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, in
 #define NMQ_LAUNCH(OUT)                                                                                                  \
     Q8_ROW_SHAPE_SWITCH(N, {                                                                                             \
         const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);                                           \
+        if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_norm_mod_fht_quant_rows: too many rows for one launch"); \
         hipLaunchKernelGGL((norm_mod_fht_quant_kernel<LANES, CH, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, \
                            norm_w, apply_norm, mod_scale, mod_shift, mod_dtype, rpm, scale_add, apply_fht, fht_scale,    \
                            codes, scales, rows, dim, flags);                                                             \

@@ -209,6 +209,7 @@ extern "C" int q8_quant_rows(const void* x, int x_dtype, void* codes, int code_d
     Q8_ROW_SHAPE_SWITCH(N, {                                                                           \
         constexpr int RB = (kBlock / LANES) * RowsPerThread<LANES, CH>::value;                         \
         const int64_t grid = (rows + RB - 1) / RB;                                                     \
+        if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_quant_rows: too many rows for one launch"); \
         hipLaunchKernelGGL((quant_rows_kernel<LANES, CH, IN, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, \
                            codes, scales, rows, dim, x_row_stride, flags);                             \
     })
@@ -250,6 +251,7 @@ extern "C" int q8_fht(const void* x, int x_dtype, void* y, int y_dtype, int64_t 
     Q8_IO_SWITCH(x_dtype, y_dtype, {
         Q8_ROW_SHAPE_SWITCH(N, {
             const int64_t grid = (rows + (kBlock / LANES) - 1) / (kBlock / LANES);
+            if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_fht: too many rows for one launch");
             hipLaunchKernelGGL((fht_kernel<LANES, CH, IN, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, y, rows,
                                dim, scale);
         })
@@ -269,6 +271,7 @@ extern "C" int q8_rmsnorm(const void* x, int x_dtype, const float* w, void* y, i
         Q8_ROW_SHAPE_SWITCH(N, {
             constexpr int RB = (kBlock / LANES) * RowsPerThread<LANES, CH>::value;
             const int64_t grid = (rows + RB - 1) / RB;
+            if (grid > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "q8_rmsnorm: too many rows for one launch");
             hipLaunchKernelGGL((rmsnorm_kernel<LANES, CH, IN, OUT>), dim3((unsigned)grid), dim3(kBlock), 0, stream, x, w, y,
                                rstd, rows, dim, eps);
         })

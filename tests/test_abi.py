@@ -56,6 +56,11 @@ def test_strerror_and_argument_validation_without_gpu():
     assert L.q8_fht(16, _lib.Q8_F32, 16, _lib.Q8_BF16, 4, 64, 1.0, None) == -2
     assert L.q8_fht(16, _lib.Q8_BF16, 16, _lib.Q8_BF16, 4, 65536, 1.0, None) == -3
     assert L.q8_rope(16, _lib.Q8_BF16, None, None, 16, _lib.Q8_BF16, 4, 64, None) == -1
+    # more rows than one launch can cover (2^31 - 1 workgroups): refused, not truncated
+    assert L.q8_quant_rows(16, _lib.Q8_BF16, 16, _lib.Q8_I8, 16, 1 << 40, 32768, 32768, 0, None) == -3
+    assert b"too many rows" in L.q8_last_error()
+    assert L.q8_fht(16, _lib.Q8_BF16, 16, _lib.Q8_BF16, 1 << 40, 32768, 1.0, None) == -3
+    assert b"too many rows" in L.q8_last_error()
     assert L.q8_gemm(16, 16, None, 16, 16, 16, 1, 1, 8, 8, 24, _lib.Q8_I8, _lib.Q8_BF16, 0, None) == -3
     assert L.q8_gemm(16, 16, None, 16, 16, 16, 2, 3, 8, 8, 32, _lib.Q8_I8, _lib.Q8_BF16, 0, None) == -3
     assert L.q8_gemm(16, 16, None, 16, 16, 16, 1, 1, 8, 8, 32, _lib.Q8_BF16, _lib.Q8_BF16, 0, None) == -2

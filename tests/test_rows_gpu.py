@@ -219,3 +219,31 @@ def test_rope_rejects_bad_arguments(dev):
         _C().rope(x, torch.zeros(2, 8, device=dev), torch.zeros(2, 8, device=dev))
     with pytest.raises(RuntimeError):
         _C().rope(x, torch.zeros(2, 16, device=dev, dtype=torch.float64), torch.zeros(2, 16, device=dev))
+
+
+def test_rows_beyond_2_31_elements(dev):
+    """[1 100 000, 2048] bf16: 2.25e9 elements, 4.5 GB; element 2^31 and byte 2^32 fall into row 1 048 576. Quantizer,
+    FHT and the fused FHT + quantizer on rows at the start, around that row and at the end, against the oracle."""
+    from q8_kernels_amd import _C
+    rows, dim = 1_100_000, 2048
+    torch.manual_seed(4)
+    x = torch.randn(rows, dim, device=dev, dtype=torch.bfloat16)
+    assert x.numel() > (1 << 31)
+    codes, scales = _C.tokenwise_quant(x, torch.int8)
+    y = _C.fast_hadamard_transform(x, dim ** -0.5, torch.bfloat16)
+    fcodes, fscales = _C.fht_quant(x, dim ** -0.5, torch.int8, mid_type=torch.bfloat16)
+    torch.cuda.synchronize()
+    mark = (1 << 31) // dim
+    for lo in (0, mark - 32, rows - 64):
+        sl = slice(lo, lo + 64)
+        xs = x[sl].cpu()
+        want_codes, want_scales = O.ref_quant(xs, torch.int8)
+        assert_bit_equal(codes[sl], want_codes, "quantizer codes, rows from %d" % lo)
+        assert_bit_equal(scales[sl], want_scales, "quantizer scales, rows from %d" % lo)
+        want_y = O.ref_fht(xs, dim ** -0.5, torch.bfloat16)
+        assert_bit_equal(y[sl], want_y, "FHT, rows from %d" % lo)
+        want_fc, want_fs = O.ref_quant(want_y, torch.int8)
+        assert_bit_equal(fcodes[sl], want_fc, "FHT + quantizer codes, rows from %d" % lo)
+        assert_bit_equal(fscales[sl], want_fs, "FHT + quantizer scales, rows from %d" % lo)
+    del x, y, codes, fcodes
+    torch.cuda.empty_cache()
