@@ -169,8 +169,8 @@ extern "C" int q8_fma(const void* x, int x_dtype, const void* y, int y_dtype, co
                       q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (rows < 0 || dim <= 0 || dim % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_fma: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
+    if (rows == 0) return Q8_OK;  // (with no rows the broadcast periods mean nothing; a caller with zero tokens passes 0)
     if (y_rows_every <= 0 || z_rows_every <= 0) return fail(Q8_ERR_SHAPE, "q8_fma: broadcast periods must be positive");
-    if (rows == 0) return Q8_OK;
     if (!x || !y || !z || !out) return fail(Q8_ERR_NULL, "q8_fma: null pointer");
     if (!is_8or16(x_dtype) || !is_8or16(out_dtype) || !is_operand(y_dtype) || !is_operand(z_dtype))
         return fail(Q8_ERR_DTYPE, "q8_fma: dtypes x %d y %d z %d out %d", x_dtype, y_dtype, z_dtype, out_dtype);

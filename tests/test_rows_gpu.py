@@ -247,3 +247,27 @@ def test_rows_beyond_2_31_elements(dev):
         assert_bit_equal(fscales[sl], want_fs, "FHT + quantizer scales, rows from %d" % lo)
     del x, y, codes, fcodes
     torch.cuda.empty_cache()
+
+
+def test_zero_rows_everywhere(dev):
+    """Tensors without rows pass through every row operator (outputs of the matching empty shapes, no launch)."""
+    from q8_kernels_amd import _C
+    bf16 = torch.bfloat16
+    x = torch.zeros(0, 64, dtype=bf16, device=dev)
+    x3 = torch.zeros(2, 0, 64, dtype=bf16, device=dev)
+    w = torch.ones(64, device=dev)
+    tab = torch.zeros(0, 64, device=dev)
+    assert _C.fast_hadamard_transform(x, 1.0, None).shape == (0, 64)
+    y, rstd = _C.rms_norm(x, w, None)
+    assert y.shape == (0, 64) and rstd.shape == (0,)
+    assert _C.rope(x, tab, tab, None).shape == (0, 64)
+    codes, scales = _C.fht_quant(x, 0.125, torch.int8)
+    assert codes.shape == (0, 64) and scales.shape == (0,)
+    codes, scales, rstd = _C.rms_norm_quant(x, w, E4M3)
+    assert codes.shape == (0, 64) and scales.shape == (0,) and rstd.shape == (0,)
+    mod = torch.zeros(2, 1, 64, dtype=bf16, device=dev)
+    codes, scales = _C.norm_mod_fht_quant(x3, True, None, mod, mod, 1.0, 0.125, torch.int8)
+    assert codes.shape == (2, 0, 64) and scales.shape == (2, 0)
+    assert _C.fma_8bit(x3, mod, mod, 1.0).shape == (2, 0, 64)
+    assert _C.gelu_forward(x).shape == (0, 64)
+    torch.cuda.synchronize()
