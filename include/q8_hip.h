@@ -223,6 +223,8 @@ int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scal
  * in_dtype in {I8, E4M3}; out_dtype in {BF16, E4M3}; bias fp32 [N] or NULL.
  * K % 16 == 0 and A, B 16-byte aligned; M, N arbitrary (> 0); N % 8 == 0 for BF16 output rows to stay
  * 16-byte aligned, N % 16 == 0 for E4M3 output.
+ * M == 0 or N == 0 (no tokens, no output elements) returns Q8_OK without touching any pointer, also in
+ * q8_gemm_residual and q8_gemm_i32; negative sizes and K <= 0 are errors.
  */
 int q8_gemm(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C,
             int batch_a, int batch_b, int M, int N, int K, int in_dtype, int out_dtype, int fuse_gelu,
@@ -284,6 +286,7 @@ int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int 
  * q: [B,H,M,64] e4m3; k: [B,H,N,64] e4m3; v: e4m3 in v_layout; o: [B,H,M,64] of out_dtype.
  * kv_len: int32 [B] or NULL; sq: fp32 [B,H,M], sk, sv: fp32 [B,H,N] per-token dequantisation scales
  * or NULL (all three given or none). D must be 64. softmax_scale is the plain (natural-log) scale.
+ * B == 0 or M == 0 (no queries) returns Q8_OK without touching any pointer; N has to be positive.
  */
 int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int32_t* kv_len,
                 const float* sq, const float* sk, const float* sv,

@@ -342,9 +342,10 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
                            const float* sk, const float* sv, int B, int H, int M, int N, int D, int v_layout,
                            int64_t v_row_stride, float softmax_scale, int out_dtype, int flags, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (!q || !k || !v || !o) return fail(Q8_ERR_NULL, "q8_attn_fwd: null pointer");
     if (D != 64) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: head dim %d (only 64 is supported)", D);
-    if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
+    if (B < 0 || H <= 0 || M < 0 || N <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
+    if (B == 0 || M == 0) return Q8_OK;  // no queries: nothing to compute or to write
+    if (!q || !k || !v || !o) return fail(Q8_ERR_NULL, "q8_attn_fwd: null pointer");
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);
     if (out_dtype != Q8_BF16 && out_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_attn_fwd: output dtype %d", out_dtype);
     if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE | Q8_ATTN_O_TOKEN_MAJOR)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);

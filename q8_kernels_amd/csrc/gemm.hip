@@ -279,6 +279,12 @@ static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
     return launch_gemm<CfgSmall<IN>, OUT, GELU>(p, stream);
 }
 
+// An output without rows or columns (no tokens): nothing to compute or to write. Negative sizes, K <= 0 and bad batch
+// counts are still errors (check_gemm).
+static bool gemm_output_is_empty(int batch_a, int batch_b, int M, int N, int K) {
+    return (M == 0 || N == 0) && M >= 0 && N >= 0 && K > 0 && batch_a > 0 && batch_b > 0;
+}
+
 static int check_gemm(const char* who, const void* A, const void* B, const void* C, int batch_a, int batch_b, int M, int N,
                       int K) {
     if (!A || !B || !C) return fail(Q8_ERR_NULL, "%s: null pointer", who);
@@ -310,6 +316,7 @@ extern "C" int q8_gemm(const void* A, const void* B, const float* bias, const fl
                        int batch_a, int batch_b, int M, int N, int K, int in_dtype, int out_dtype, int fuse_gelu,
                        q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (gemm_output_is_empty(batch_a, batch_b, M, N, K)) return Q8_OK;
     if (int st = check_gemm("q8_gemm", A, B, C, batch_a, batch_b, M, N, K)) return st;
     if (!sa || !sb) return fail(Q8_ERR_NULL, "q8_gemm: scales are required");
     if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_gemm: input dtype %d", in_dtype);
@@ -331,6 +338,7 @@ extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias,
                                 const void* residual, void* C, int batch_a, int batch_b, int M, int N, int K, int in_dtype,
                                 int fuse_gelu, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (gemm_output_is_empty(batch_a, batch_b, M, N, K)) return Q8_OK;
     if (int st = check_gemm("q8_gemm_residual", A, B, C, batch_a, batch_b, M, N, K)) return st;
     if (!sa || !sb || !residual) return fail(Q8_ERR_NULL, "q8_gemm_residual: scales and residual are required");
     if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_gemm_residual: input dtype %d", in_dtype);
@@ -346,6 +354,7 @@ extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias,
 
 extern "C" int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int K, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;
     if (int st = check_gemm("q8_gemm_i32", A, B, C, 1, 1, M, N, K)) return st;
     if (!aligned16(C)) return fail(Q8_ERR_ALIGN, "q8_gemm_i32: C must be 16-byte aligned");
     GemmParams p{reinterpret_cast<const uint8_t*>(A), reinterpret_cast<const uint8_t*>(B), nullptr, nullptr, nullptr, C, 1, 1, M, N, K};

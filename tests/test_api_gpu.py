@@ -274,3 +274,25 @@ def test_ltx_block_replays_from_a_graph(dev):
                 (torch.randn(2, 1, 6 * dim, generator=g) * 0.3).to(dev))
 
     _replays_match_eager(lambda h, x, ts: blk(h, (cos, sin), None, x, lens, ts, attn_type="q8_kernels"), make(1), make)
+
+
+def test_no_tokens_give_empty_outputs(dev):
+    """Zero rows through the linears and zero queries through attention return empty tensors of the right shape, as
+    torch's own operators do, instead of an error."""
+    import q8_kernels_amd.functional as F
+    from q8_kernels_amd import _C
+    from q8_kernels_amd.modules import Q8Linear
+    g = torch.Generator().manual_seed(2)
+    w = (torch.randn(128, 256, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    x0 = torch.zeros(0, 256, dtype=torch.bfloat16, device=dev)
+    assert F.linear.q8_linear(x0, w, out_dtype=torch.bfloat16).shape == (1, 0, 128)
+    assert F.linear.fp8_linear(x0, w, out_dtype=torch.bfloat16).shape[-2:] == (0, 128)
+    lin = Q8Linear.from_linear(torch.nn.Linear(256, 128).to(dev).to(torch.bfloat16))
+    assert lin(torch.zeros(2, 0, 256, dtype=torch.bfloat16, device=dev), out_dtype=torch.bfloat16).shape == (2, 0, 128)
+    a = torch.zeros(0, 64, dtype=torch.int8, device=dev)
+    b = torch.zeros(8, 64, dtype=torch.int8, device=dev)
+    assert _C.q8_mm_i32(a, b).shape == (0, 8)
+    q = torch.zeros(1, 2, 0, 64, dtype=torch.bfloat16, device=dev)
+    kv = torch.randn(1, 2, 40, 64, generator=g).to(torch.bfloat16).to(dev)
+    assert F.flash_attention.flash_attn_func(q, kv, kv, out_dtype=torch.bfloat16).shape == (1, 2, 0, 64)
+    torch.cuda.synchronize()
