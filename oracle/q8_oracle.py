@@ -110,10 +110,15 @@ def ref_quant(x: torch.Tensor, out_type: Optional[torch.dtype] = None, round_hal
         e4m3: c10 cast;  stored scale = 1 / r.     QMAX = 127 / 448 (:10-12); out_type None -> int8
         (csrc/quantizer/tokenwise_quant.cpp:88-93).
     Deviations selected by flags: round_half_even (BASELINE config 2), scale_as_division
-    (scale = a / QMAX). A zero row gives codes 0 and scale 0 (the reference yields NaN codes there)."""
+    (scale = a / QMAX). A zero row gives codes 0 and scale 0 (the reference yields NaN codes there).
+    Non-finite input: the reference's row maximum is a chain of CUDA max(float, float), i.e. fmaxf (:115-132), which
+    skips NaN operands, so a NaN element leaves the scale and the other codes of its row alone and only becomes a NaN
+    code itself (e4m3; its int8 code is a C++ conversion of NaN, undefined); an infinite element makes the scale
+    infinite, the finite elements' codes zero and its own code NaN (inf * 0). A row of nothing but NaN is not modelled."""
     out_type = torch.int8 if out_type is None else out_type
     xf = x.to(torch.float32)
-    a = xf.abs().amax(dim=-1, keepdim=True)
+    ax = xf.abs()
+    a = torch.where(ax.isnan(), torch.zeros_like(ax), ax).amax(dim=-1, keepdim=True)
     qmax = torch.tensor(127.0 if out_type == torch.int8 else 448.0, dtype=torch.float32)
     nz = a > 0
     r = torch.where(nz, qmax / torch.where(nz, a, torch.ones_like(a)), torch.zeros_like(a))

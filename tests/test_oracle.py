@@ -434,3 +434,34 @@ def test_rms_norm_backward_against_autograd():
         # the oracle is called with out_type float32 on bf16-free data through its float path
         got = O.ref_rms_norm_backward(y.detach().float(), rstd.detach().float().squeeze(-1), go.float(), w, torch.float32)
         assert torch.allclose(got.double(), xd.grad, rtol=2e-5, atol=2e-6)
+
+
+def test_quant_nan_elements_do_not_touch_the_rest_of_the_row():
+    """fmaxf semantics of the reference's row maximum (csrc/quantizer/tokenwise_quant_cuda.cu:115-132), pinned without
+    the oracle's own formula: the row with its NaN elements replaced by zeros (which cannot be the maximum) must give the
+    same scale and the same codes everywhere else; the NaN elements themselves come out as e4m3 NaN codes. An infinite
+    element: infinite scale, zero codes for the finite elements, a NaN code for itself (inf * 0)."""
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn(6, 64, generator=g) * 3).to(torch.bfloat16)
+    nan_at = [(1, 5), (3, 0), (3, 63), (4, 17)]
+    for r, c in nan_at:
+        x[r, c] = float("nan")
+    clean = torch.where(x.isnan(), torch.zeros_like(x), x)
+    keep = ~x.isnan()
+    for out_type in (torch.int8, O.E4M3):
+        codes, scales = O.ref_quant(x, out_type)
+        want_codes, want_scales = O.ref_quant(clean, out_type)
+        assert torch.equal(scales, want_scales)
+        view = (lambda t: t.view(torch.uint8)) if out_type == O.E4M3 else (lambda t: t)
+        assert torch.equal(view(codes)[keep], view(want_codes)[keep])
+        if out_type == O.E4M3:
+            assert all((int(view(codes)[r, c]) & 0x7F) == 0x7F for r, c in nan_at)
+    y = (torch.randn(2, 32, generator=g)).to(torch.bfloat16)
+    y[0, 3] = float("inf")
+    y[1, 9] = float("-inf")
+    codes, scales = O.ref_quant(y, O.E4M3)
+    assert torch.isinf(scales).all()
+    u = codes.view(torch.uint8)
+    finite = ~y.isinf()
+    assert ((u[finite] & 0x7F) == 0).all()            # +-0
+    assert ((u[~finite] & 0x7F) == 0x7F).all()        # NaN

@@ -271,3 +271,29 @@ def test_zero_rows_everywhere(dev):
     assert _C.fma_8bit(x3, mod, mod, 1.0).shape == (2, 0, 64)
     assert _C.gelu_forward(x).shape == (0, 64)
     torch.cuda.synchronize()
+
+
+def test_quantizer_non_finite_elements(dev):
+    """A NaN element is skipped by the row maximum (the reference's fmaxf chain): scale and the other codes as without
+    it, itself an e4m3 NaN code (sign not compared; its int8 code is undefined in the reference and not compared).
+    An infinite element: infinite scale, zeros, NaN for itself. Kernel against the oracle."""
+    from q8_kernels_amd import _C
+    g = torch.Generator().manual_seed(22)
+    x = (torch.randn(8, 2048, generator=g) * 2).to(torch.bfloat16)
+    x[1, 5] = float("nan")
+    x[2, 3] = float("inf")
+    x[3, 7] = float("-inf")
+    x[4, 0] = float("nan")
+    x[4, 2047] = float("nan")
+    x[5, 100] = float("nan")
+    x[5, 200] = float("inf")
+    special = ~torch.isfinite(x)
+    for out_type in (torch.int8, E4M3):
+        codes, scales = _C.tokenwise_quant(x.to(dev), out_type)
+        want_codes, want_scales = O.ref_quant(x, out_type)
+        assert_bit_equal(scales, want_scales, "scales %s" % out_type)
+        got, want = codes.cpu(), want_codes
+        if out_type == E4M3:
+            got, want = got.view(torch.uint8), want.view(torch.uint8)
+            assert torch.equal(got[special] & 0x7F, want[special] & 0x7F), "codes of the non-finite elements"
+        assert torch.equal(got[~special], want[~special]), "codes of the finite elements, %s" % out_type
