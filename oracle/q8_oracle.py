@@ -17,6 +17,8 @@ Pinning status:
   parity unpinned (bit level) .. the low-order bits the reference gets from nvcc --use_fast_math
                                  (approximate division in the quantizer, tanhf / exp2f / rsqrtf) and the
                                  accumulation order inside mma.sync; unobservable without an sm_89 GPU.
+                                 Quantizer: the int8 code of a NaN element (an undefined C++ conversion in the
+                                 reference), a row of nothing but NaN, the sign of NaN codes.
 """
 import math
 from typing import Optional, Tuple
