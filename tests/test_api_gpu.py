@@ -296,3 +296,47 @@ def test_no_tokens_give_empty_outputs(dev):
     kv = torch.randn(1, 2, 40, 64, generator=g).to(torch.bfloat16).to(dev)
     assert F.flash_attention.flash_attn_func(q, kv, kv, out_dtype=torch.bfloat16).shape == (1, 2, 0, 64)
     torch.cuda.synchronize()
+
+
+def test_concurrent_threads_on_their_own_streams(dev):
+    """Four host threads, each on a stream of its own, run quantizer -> GEMM (+GELU) -> attention on their own data 30
+    times while the others do the same (ctypes releases the GIL during the calls); every result has to equal the one
+    computed alone beforehand. The library's per-call state (error text, last-kernel record, per-kernel set-up) is
+    thread-local and its kernels use no shared scratch memory."""
+    from concurrent.futures import ThreadPoolExecutor
+    from q8_kernels_amd import _C
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(700 + 64 * seed, 512, generator=g).to(torch.bfloat16).to(dev)
+        w = (torch.randn(384, 512, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+        bias = torch.randn(384, generator=g).to(dev)
+        q = torch.randn(1, 2, 208 + 16 * seed, 64, generator=g).to(torch.bfloat16).to(dev)
+        return x, w, bias, q
+
+    def step(x, w, bias, q):
+        xq, sx = _C.tokenwise_quant(x, E4M3)
+        wq, sw = _C.tokenwise_quant(w, E4M3)
+        y = _C.fp8_mm_bias(xq, wq, bias, sx, sw, True, torch.bfloat16)
+        q8 = _C.fast_hadamard_transform(q, 0.125, E4M3)
+        o = _C.flash_attention(q8, q8, q8.transpose(2, 3).contiguous(), 1.0, None, out_dtype=torch.bfloat16)
+        return y, o
+
+    data = [make(s) for s in range(4)]
+    want = [step(*d) for d in data]
+    torch.cuda.synchronize()
+
+    def worker(i):
+        stream = torch.cuda.Stream()
+        bad = 0
+        with torch.cuda.stream(stream):
+            for _ in range(30):
+                y, o = step(*data[i])
+                stream.synchronize()
+                bad += int(not torch.equal(y.view(torch.int16), want[i][0].view(torch.int16)))
+                bad += int(not torch.equal(o.view(torch.int16), want[i][1].view(torch.int16)))
+        return bad
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        results = list(pool.map(worker, range(4)))
+    assert results == [0, 0, 0, 0], results
