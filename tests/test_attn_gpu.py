@@ -250,3 +250,30 @@ def test_attention_random_shapes(dev, sweep_seed):
             _lib.check(_lib.lib().q8_attn_set_config(0))
         assert got.shape == (b, h, m, 64), what
         _check(got, q, k, v, 0.125, lens, sc, what=what)
+
+
+def test_workgroup_shapes_give_identical_bits(dev):
+    """A query row meets the same 64-key tiles in the same order whatever the workgroup shape, so the three shapes
+    of q8_attn_set_config have to agree bit for bit (direct casts with a mask, and per-token scales)."""
+    from q8_kernels_amd import _lib
+    g = torch.Generator().manual_seed(77)
+    b, h, m, n = 2, 3, 333, 517
+    q, k, v = _inputs(77, b, h, m, n)
+    lens = torch.tensor([517, 130], dtype=torch.int32)
+    qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)
+    kf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 4 + 0.2)
+    vf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 2 + 0.5)
+    (q2, sq), (k2, sk), (v2, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+    outs = {}
+    try:
+        for cfg in (0, 1, 2):
+            _lib.check(_lib.lib().q8_attn_set_config(cfg))
+            plain = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16)
+            scaled = _C().flash_attention(q2.to(dev), k2.to(dev), _vt(v2).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
+                                          q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+            outs[cfg] = (plain.cpu().view(torch.int16), scaled.cpu().view(torch.int16))
+    finally:
+        _lib.check(_lib.lib().q8_attn_set_config(0))
+    for cfg in (1, 2):
+        assert torch.equal(outs[cfg][0], outs[0][0]), "direct casts, shape %d" % cfg
+        assert torch.equal(outs[cfg][1], outs[0][1]), "per-token scales, shape %d" % cfg
