@@ -236,7 +236,7 @@ def ref_fp8_linear(a, b, bias=None, scale_a=None, scale_b=None, use_hadamard=Fal
 def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                   kv_len: Optional[torch.Tensor] = None, sq=None, sk=None, sv=None,
                   round_p: bool = True, out_dtype: Optional[torch.dtype] = None, return_weighted_abs: bool = False,
-                  p_scale: float = 256.0):
+                  p_scale: float = 1.0):
     """Attention on e4m3 operands as the reference kernel defines it (csrc/flash_attention/
     flash_attention_cuda.cu:171-248,437,487-497; mask: flash_attention_cuda_mask.cu:244,319):
         s_ij = (q_i . k_j) * scale (* sq_i sk_j);  keys j >= kv_len[b] masked;
@@ -247,8 +247,9 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
     q [B,H,M,D], k, v [B,H,N,D] (v NOT transposed here). With round_p=False this is plain fp32-style
     softmax attention on the dequantised inputs (evaluated in float64), the accuracy target of the
     BASELINE configs. out_dtype None returns float64; bf16 -> RNE; e4m3 -> saturating cast.
-    p_scale: the probabilities are rounded as e4m3_sat(p_scale * p); the reference has p_scale = 1 (weights
-    below 2^-10 flush to zero), the HIP kernel defaults to 2^8, which cancels in o / l.
+    p_scale: the probabilities are rounded as e4m3_sat(p_scale * p). The default 1 is the reference (weights below
+    2^-10 flush to zero); the HIP kernel's own default is 2^8, which cancels in o / l, and the tests of that default
+    pass p_scale=256 explicitly.
     The online kernel rounds p against the running maximum, so its P-hat differs from this one in the
     last e4m3 bit here and there: comparisons carry a tolerance. With return_weighted_abs the function also
     returns W = sum_j p_ij |v_j| / l_i and U = sum_j |v_j| / l_i: rounding every weight with relative error eps
@@ -293,11 +294,12 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
 
 
 def ref_flash_attn_func(q, k, v, softmax_scale=None, batch_mask=None, apply_qk_hadamard=False, out_dtype=None,
-                        round_p=True):
+                        round_p=True, p_scale=1.0):
     """FlashAttnFunc.forward, q8_kernels/functional/flash_attention.py:18-61: head dim padded to a multiple of
     32, V cast straight to e4m3, Q and K either cast straight (kernel scale = softmax_scale) or rotated by the
     FHT with sqrt(softmax_scale)/sqrt(D) folded into both (kernel scale = 1). Output e4m3 like the
-    reference unless out_dtype says otherwise; sliced back to the original head dim."""
+    reference unless out_dtype says otherwise; sliced back to the original head dim. p_scale as in ref_attention
+    (1 = the reference's rounding of the probabilities)."""
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     d_og = q.shape[-1]
@@ -318,7 +320,7 @@ def ref_flash_attn_func(q, k, v, softmax_scale=None, batch_mask=None, apply_qk_h
             k = e4m3_c10(k)
         kernel_scale = softmax_scale
     o = ref_attention(q, k, v, kernel_scale, batch_mask, round_p=round_p,
-                      out_dtype=E4M3 if out_dtype is None else out_dtype)
+                      out_dtype=E4M3 if out_dtype is None else out_dtype, p_scale=p_scale)
     return o[..., :d_og]
 
 
@@ -435,7 +437,7 @@ def ref_rms_norm_backward(x_normed: torch.Tensor, x_norms: torch.Tensor, grad_ou
 # ------------------------------------------------------------------------------------------- block composition
 
 
-def ref_dit_block(hidden, text, freqs_cis, text_lens, params, num_heads, head_dim=64):
+def ref_dit_block(hidden, text, freqs_cis, text_lens, params, num_heads, head_dim=64, p_scale=1.0):
     """The simplified LTX-style fp8 block of the benchmark configuration, composed from the functions above
     (op order as q8_kernels/modules/attention.py:45-106 and q8_kernels/modules/ffn.py:10-17 chain them):
     RMSNorm -> fp8 QKV -> RoPE(q, k) -> fp8 Hadamard self-attention -> out projection (+res) -> RMSNorm ->
@@ -458,18 +460,18 @@ def ref_dit_block(hidden, text, freqs_cis, text_lens, params, num_heads, head_di
     h, _ = ref_rms_norm(hidden, params["norm1"])
     q, k, v = lin("to_qkv", h).split(dim, dim=-1)
     q, k = ref_rope(q, *freqs_cis), ref_rope(k, *freqs_cis)
-    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, None, True, out_dtype=bf16)
+    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, None, True, out_dtype=bf16, p_scale=p_scale)
     hidden = hidden + lin("to_out", merge(a))
     h, _ = ref_rms_norm(hidden, params["norm2"])
     a = ref_flash_attn_func(heads(lin("to_q2", h)), heads(lin("to_k2", text)), heads(lin("to_v2", text)), None, text_lens, True,
-                            out_dtype=bf16)
+                            out_dtype=bf16, p_scale=p_scale)
     hidden = hidden + lin("to_out2", merge(a))
     h, _ = ref_rms_norm(hidden, params["norm3"])
     return hidden + lin("ff_down", lin("ff_up", h, gelu=True))
 
 
 def ref_attention_module(p, prefix, x, num_heads, head_dim, freqs_cis=None, context=None, lens=None,
-                         non_mm=torch.bfloat16, mm_out=torch.bfloat16):
+                         non_mm=torch.bfloat16, mm_out=torch.bfloat16, p_scale=1.0):
     """q8_kernels/modules/attention.py:45-106 with attn_type 'q8_kernels': int8 projections, qk-RMSNorm over the
     full inner dim, RoPE on self-attention, fp8 flash attention with Hadamard (e4m3 output), output projection.
     p[prefix + name] = (int8 weight, fp32 scales, fp32 bias or None); p[prefix + 'q_norm' / 'k_norm'] = fp32 [inner]."""
@@ -488,12 +490,12 @@ def ref_attention_module(p, prefix, x, num_heads, head_dim, freqs_cis=None, cont
     k, _ = ref_rms_norm(k, p[prefix + "k_norm"], non_mm)
     if context is None and freqs_cis is not None:
         q, k = ref_rope(q, freqs_cis[0], freqs_cis[1], non_mm), ref_rope(k, freqs_cis[0], freqs_cis[1], non_mm)
-    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, lens, True)
+    a = ref_flash_attn_func(heads(q), heads(k), heads(v), None, lens, True, p_scale=p_scale)
     a = a.transpose(1, 2).reshape(b, -1, num_heads * head_dim)
     return lin("to_out", a).to(non_mm)
 
 
-def ref_ltx_block(p, hidden, freqs_cis, context, context_lens, timestep, num_heads, head_dim):
+def ref_ltx_block(p, hidden, freqs_cis, context, context_lens, timestep, num_heads, head_dim, p_scale=1.0):
     """q8_kernels/blocks/ltx_transformer_block.py:21-58 with bfloat16 activations; the modulations and gated
     residuals are evaluated as fused multiply-adds (ref_fma). p['scale_shift_table'] fp32 [6, dim],
     p['norm1'] / p['norm2'] = fp32 [dim] or None, attention parameters under 'attn1.' / 'attn2.',
@@ -504,9 +506,9 @@ def ref_ltx_block(p, hidden, freqs_cis, context, context_lens, timestep, num_hea
     shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (t.to(bf16) for t in ada.unbind(dim=2))
     h, _ = ref_rms_norm(hidden, p["norm1"], bf16)
     h = ref_fma(h, scale_msa, shift_msa, 1.0)
-    a = ref_attention_module(p, "attn1.", h, num_heads, head_dim, freqs_cis)
+    a = ref_attention_module(p, "attn1.", h, num_heads, head_dim, freqs_cis, p_scale=p_scale)
     hidden = ref_fma(a, gate_msa, hidden, 0.0)
-    a = ref_attention_module(p, "attn2.", hidden, num_heads, head_dim, None, context, context_lens)
+    a = ref_attention_module(p, "attn2.", hidden, num_heads, head_dim, None, context, context_lens, p_scale=p_scale)
     hidden = a + hidden
     h, _ = ref_rms_norm(hidden, p["norm2"], bf16)
     h = ref_fma(h, scale_mlp, shift_mlp, 1.0)

@@ -65,7 +65,8 @@ def main():
     lens = torch.tensor([50], dtype=torch.int32)
     out["attn_q"], out["attn_k"], out["attn_v"], out["attn_len"] = u8(q), u8(k), u8(v), lens.numpy()
     out["attn_exact_f64"] = O.ref_attention(q, k, v, 0.125, lens, round_p=False).numpy()
-    out["attn_rounded_f64"] = O.ref_attention(q, k, v, 0.125, lens, round_p=True).numpy()
+    out["attn_rounded_f64"] = O.ref_attention(q, k, v, 0.125, lens, round_p=True, p_scale=256.0).numpy()
+    out["attn_rounded_unit_f64"] = O.ref_attention(q, k, v, 0.125, lens, round_p=True, p_scale=1.0).numpy()
     # RMSNorm / RoPE
     xn = torch.randn(5, 64, generator=g).to(torch.bfloat16)
     w = torch.rand(64, generator=g) + 0.5

@@ -42,7 +42,8 @@ def test_oracle_reproduces_fixture():
     q, k, v = e4m3("attn_q"), e4m3("attn_k"), e4m3("attn_v")
     lens = torch.from_numpy(G["attn_len"].copy())
     assert np.allclose(O.ref_attention(q, k, v, 0.125, lens, round_p=False).numpy(), G["attn_exact_f64"], atol=1e-12)
-    assert np.allclose(O.ref_attention(q, k, v, 0.125, lens, round_p=True).numpy(), G["attn_rounded_f64"], atol=1e-12)
+    assert np.allclose(O.ref_attention(q, k, v, 0.125, lens, round_p=True, p_scale=256.0).numpy(), G["attn_rounded_f64"], atol=1e-12)
+    assert np.allclose(O.ref_attention(q, k, v, 0.125, lens, round_p=True).numpy(), G["attn_rounded_unit_f64"], atol=1e-12)
     xn = bf16("rms_x_bf16")
     y, r = O.ref_rms_norm(xn, torch.from_numpy(G["rms_w"].copy()))
     assert np.array_equal(y.view(torch.int16).numpy(), G["rms_y_bf16"]) and np.array_equal(r.numpy(), G["rms_rstd"])

@@ -265,12 +265,14 @@ def test_attention_rounded_p_invariants():
     k = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
     v = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
     lens = torch.tensor([41], dtype=torch.int32)
-    o = O.ref_attention(q, k, v, 0.125, lens)
+    o = O.ref_attention(q, k, v, 0.125, lens)  # the reference's grid: p <= 1
     exact, wabs, uabs = O.ref_attention(q, k, v, 0.125, lens, round_p=False, return_weighted_abs=True)
-    # e4m3 rounding of p is a <= 2^-4 relative (normal range) / 2^-18 absolute (below it) perturbation of each weight
-    assert ((o - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -18 * uabs + 1e-12).all()
-    o1 = O.ref_attention(q, k, v, 0.125, lens, p_scale=1.0)
-    assert ((o1 - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -10 * uabs + 1e-12).all()
+    # e4m3 rounding of p is a <= 2^-4 relative (normal range) / 2^-10 absolute (below it) perturbation of each weight
+    assert ((o - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -10 * uabs + 1e-12).all()
+    assert torch.equal(o, O.ref_attention(q, k, v, 0.125, lens, p_scale=1.0)), "the default is the reference's p_scale = 1"
+    # probabilities scaled by 2^8 before the cast (the HIP kernel's default): the subnormal floor drops to 2^-18
+    o256 = O.ref_attention(q, k, v, 0.125, lens, p_scale=256.0)
+    assert ((o256 - exact).abs() <= 2.0 ** -4 * wabs + 2.0 ** -18 * uabs + 1e-12).all()
     # masked keys carry no weight: changing them changes nothing
     v2 = v.clone().view(torch.uint8)
     v2[:, :, 41:, :] = 0x7E
@@ -465,3 +467,204 @@ def test_quant_nan_elements_do_not_touch_the_rest_of_the_row():
     finite = ~y.isinf()
     assert ((u[finite] & 0x7F) == 0).all()            # +-0
     assert ((u[~finite] & 0x7F) == 0x7F).all()        # NaN
+
+
+# ------------------------------------------------------------------ block compositions against dense float64
+#
+# ref_attention_module, ref_ltx_block and ref_dit_block chain the operators above; what they decide is ORDER:
+# which modulation row is the shift and which the scale, which residual is gated, whether the qk-norm comes before
+# the rotation, which attention is rotated at all. They are pinned here against a dense float64 evaluation written
+# from the text of q8_kernels/blocks/ltx_transformer_block.py:21-58, q8_kernels/modules/attention.py:45-106 and
+# q8_kernels/modules/ffn.py:10-17 with the ORIGINAL (unquantized) weights: plain x @ W.T, softmax, no rotation, no
+# quantization. Every mutant of that evaluation (swapped shift / scale, a missing gate, ...) must be rejected.
+
+def _cos(a, b):
+    return torch.nn.functional.cosine_similarity(a.double().flatten(), b.double().flatten(), dim=0).item()
+
+
+def _dense_rms(x, w=None):
+    y = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True))
+    return y if w is None else y * w.double()
+
+
+def _dense_rope(x, cos, sin):
+    """Pairs (x[2i], x[2i+1]) as complex numbers times exp(i phi); the tables repeat every value twice."""
+    z = torch.view_as_complex(x.reshape(x.shape[:-1] + (-1, 2)).contiguous())
+    rot = torch.complex(cos[..., 0::2].double(), sin[..., 0::2].double())
+    return torch.view_as_real(z * rot).reshape(x.shape)
+
+
+def _dense_mha(q, k, v, heads, hd, lens=None):
+    b = q.shape[0]
+    split = lambda t: t.reshape(b, -1, heads, hd).transpose(1, 2)  # noqa: E731
+    q, k, v = split(q), split(k), split(v)
+    s = q @ k.transpose(-1, -2) / math.sqrt(hd)
+    if lens is not None:
+        keep = torch.arange(k.shape[2])[None, :] < lens.to(torch.int64)[:, None]
+        s = s.masked_fill(~keep[:, None, None, :], float("-inf"))
+    return (torch.softmax(s, dim=-1) @ v).transpose(1, 2).reshape(b, -1, heads * hd)
+
+
+def _dense_attention_module(W, prefix, x, heads, hd, freqs=None, ctx=None, lens=None, mutate=""):
+    """modules/attention.py:45-106: projections, qk-RMSNorm over the whole inner dim, rotation of q and k in
+    self-attention only, softmax attention with the valid-length mask, output projection."""
+    lin = lambda n, t: t @ W[prefix + n][0].double().T + W[prefix + n][1].double()  # noqa: E731
+    src = x if ctx is None else ctx
+    q, k, v = lin("to_q", x), lin("to_k", src), lin("to_v", src)
+    if mutate == "norm_after_rope" and ctx is None:
+        q, k = _dense_rope(q, *freqs), _dense_rope(k, *freqs)
+    q, k = _dense_rms(q, W[prefix + "q_norm"]), _dense_rms(k, W[prefix + "k_norm"])
+    if mutate == "no_qk_norm_weight":
+        q, k = _dense_rms(lin("to_q", x)), _dense_rms(lin("to_k", src))
+    rope_here = (ctx is None and mutate != "norm_after_rope" and mutate != "no_rope") or (ctx is not None and mutate == "rope_cross")
+    if rope_here:
+        q = _dense_rope(q, *freqs)
+        if ctx is None:
+            k = _dense_rope(k, *freqs)
+    if mutate == "swap_kv":
+        k, v = v, k
+    return lin("to_out", _dense_mha(q, k, v, heads, hd, None if mutate == "no_mask" else lens))
+
+
+def _dense_ltx_block(W, hidden, freqs, ctx, lens, timestep, heads, hd, mutate=""):
+    """blocks/ltx_transformer_block.py:21-58 in float64."""
+    b = hidden.shape[0]
+    ada = W["scale_shift_table"].double()[None, None] + timestep.double().reshape(b, timestep.shape[1], 6, -1)
+    shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada.unbind(dim=2)
+    if mutate == "swap_shift_scale":
+        shift_msa, scale_msa, shift_mlp, scale_mlp = scale_msa, shift_msa, scale_mlp, shift_mlp
+    if mutate == "swap_msa_mlp":
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = shift_mlp, scale_mlp, gate_mlp, shift_msa, scale_msa, gate_msa
+    one = 0.0 if mutate == "scale_without_one" else 1.0
+    h = hidden.double()
+    n = _dense_rms(h) * (one + scale_msa) + shift_msa
+    a = _dense_attention_module(W, "attn1.", n, heads, hd, freqs, mutate=mutate)
+    h = (a if mutate == "no_gate_msa" else gate_msa * a) + h
+    a = _dense_attention_module(W, "attn2.", h, heads, hd, freqs, ctx.double(), lens, mutate=mutate)
+    h = (gate_msa * a if mutate == "gate_on_cross" else a) + h
+    n = _dense_rms(h) * (one + scale_mlp) + shift_mlp
+    up = torch.nn.functional.gelu(n @ W["ff.up"][0].double().T + W["ff.up"][1].double(), approximate="none" if mutate == "no_gelu" else "tanh")
+    if mutate == "no_gelu":
+        up = n @ W["ff.up"][0].double().T + W["ff.up"][1].double()
+    ff = up @ W["ff.down"][0].double().T + W["ff.down"][1].double()
+    return (ff if mutate == "no_gate_mlp" else gate_mlp * ff) + h
+
+
+def _ltx_case(seed=71, dim=256, heads=4, hd=64, kv_dim=128, s_tok=48, s_txt=24):
+    """Dense weights W[name] = (weight, bias), and the quantized parameter dict the oracle block takes: int8 codes of
+    the rotated weight with per-row scales, as Q8Linear.from_linear stores them (modules/linear.py:36-49)."""
+    g = torch.Generator().manual_seed(seed)
+    bf16 = torch.bfloat16
+    W, P = {}, {}
+    shapes = {"to_q": (dim, dim), "to_k": (dim, kv_dim), "to_v": (dim, kv_dim), "to_out": (dim, dim)}
+    for a in ("attn1.", "attn2."):
+        for n, (o, i) in shapes.items():
+            i = dim if (a == "attn1." or n in ("to_q", "to_out")) else i
+            W[a + n] = ((torch.randn(o, i, generator=g) / math.sqrt(i)).to(bf16), torch.randn(o, generator=g) * 0.1)
+        for n in ("q_norm", "k_norm"):
+            W[a + n] = P[a + n] = torch.rand(dim, generator=g) * 1.6 + 0.2  # uneven inside a rotated pair: the norm does not commute with the rotation
+    W["ff.up"] = ((torch.randn(4 * dim, dim, generator=g) / math.sqrt(dim)).to(bf16), torch.randn(4 * dim, generator=g) * 0.1)
+    W["ff.down"] = ((torch.randn(dim, 4 * dim, generator=g) / math.sqrt(4 * dim)).to(bf16), torch.randn(dim, generator=g) * 0.1)
+    for n, val in list(W.items()):
+        if isinstance(val, tuple):
+            codes, scales = O.ref_quant(O.ref_fht(val[0]))
+            P[n] = (codes, scales, val[1])
+    W["scale_shift_table"] = P["scale_shift_table"] = torch.randn(6, dim, generator=g) / dim ** 0.5
+    P["norm1"] = P["norm2"] = None
+    hidden = torch.randn(2, s_tok, dim, generator=g).to(bf16)
+    ctx = torch.randn(2, s_txt, kv_dim, generator=g).to(bf16)
+    timestep = torch.randn(2, 1, 6 * dim, generator=g) * 0.5
+    grid = torch.stack(torch.meshgrid(torch.arange(2), torch.arange(4), torch.arange(6), indexing="ij")).reshape(3, -1)
+    freqs = O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim)
+    lens = torch.tensor([24, 7], dtype=torch.int32)
+    return W, P, hidden, freqs, ctx, lens, timestep, heads, hd
+
+
+LTX_MUTANTS = ["swap_shift_scale", "swap_msa_mlp", "scale_without_one", "no_gate_msa", "gate_on_cross", "no_gate_mlp",
+               "no_gelu", "norm_after_rope", "no_rope", "rope_cross", "no_mask", "swap_kv", "no_qk_norm_weight"]
+
+
+def test_ltx_block_composition_against_dense_float64():
+    W, P, hidden, freqs, ctx, lens, timestep, heads, hd = _ltx_case()
+    got = O.ref_ltx_block(P, hidden, freqs, ctx, lens, timestep, heads, hd)
+    assert got.shape == hidden.shape and got.dtype == torch.bfloat16
+    want = _dense_ltx_block(W, hidden, freqs, ctx, lens, timestep, heads, hd)
+    clean = _cos(got, want)
+    assert clean >= 0.99, clean
+    rel = ((got.double() - want).norm() / want.norm()).item()
+    # every mutant of the dense evaluation is further from the oracle than the 8-bit noise of the clean one
+    for mut in LTX_MUTANTS:
+        bad = _dense_ltx_block(W, hidden, freqs, ctx, lens, timestep, heads, hd, mutate=mut)
+        rel_bad = ((got.double() - bad).norm() / bad.norm()).item()
+        assert rel_bad > 1.5 * rel and _cos(got, bad) < clean, (mut, rel_bad, rel, _cos(got, bad), clean)
+
+
+def test_attention_module_composition_against_dense_float64():
+    W, P, hidden, freqs, ctx, lens, timestep, heads, hd = _ltx_case(seed=72)
+    for prefix, kw_o, kw_d in (("attn1.", dict(freqs_cis=freqs), dict(freqs=freqs)),
+                               ("attn2.", dict(context=ctx, lens=lens), dict(freqs=freqs, ctx=ctx.double(), lens=lens))):
+        got = O.ref_attention_module(P, prefix, hidden, heads, hd, **kw_o)
+        want = _dense_attention_module(W, prefix, hidden.double(), heads, hd, **kw_d)
+        assert got.shape == want.shape and got.dtype == torch.bfloat16
+        clean = _cos(got, want)
+        assert clean >= 0.99, (prefix, clean)
+        rel = ((got.double() - want).norm() / want.norm()).item()
+        muts = ["norm_after_rope", "no_rope", "swap_kv", "no_qk_norm_weight"] if prefix == "attn1." else ["rope_cross", "no_mask", "swap_kv", "no_qk_norm_weight"]
+        for mut in muts:
+            bad = _dense_attention_module(W, prefix, hidden.double(), heads, hd, mutate=mut, **kw_d)
+            rel_bad = ((got.double() - bad).norm() / bad.norm()).item()
+            assert rel_bad > 2.0 * rel, (prefix, mut, rel_bad, rel)
+
+
+def _dense_dit_block(W, hidden, text, freqs, lens, heads, hd, mutate=""):
+    """RMSNorm -> QKV -> rotation of q, k -> self-attention -> out projection (+ residual) -> RMSNorm -> cross-attention
+    with valid lengths (+ residual) -> RMSNorm -> FFN with tanh-GELU (+ residual), all in float64 on dense weights."""
+    lin = lambda n, t: t @ W[n][0].double().T + W[n][1].double()  # noqa: E731
+    dim = heads * hd
+    h = hidden.double()
+    q, k, v = lin("to_qkv", _dense_rms(h, W["norm1"])).split(dim, dim=-1)
+    if mutate == "qkv_order":
+        k, q, v = q, k, v
+    if mutate != "no_rope":
+        q, k = _dense_rope(q, *freqs), _dense_rope(k, *freqs)
+    a = lin("to_out", _dense_mha(q, k, v, heads, hd))
+    h = a if mutate == "no_residual1" else h + a
+    n = _dense_rms(h, W["norm2"])
+    t = text.double()
+    a = _dense_mha(lin("to_q2", n), lin("to_k2", t), lin("to_v2", t), heads, hd, None if mutate == "no_mask" else lens)
+    h = h + lin("to_out2", a)
+    n = _dense_rms(h, W["norm1" if mutate == "wrong_norm" else "norm3"])
+    up = lin("ff_up", n)
+    if mutate != "no_gelu":
+        up = torch.nn.functional.gelu(up, approximate="tanh")
+    ff = lin("ff_down", up)
+    return ff if mutate == "no_residual3" else h + ff
+
+
+def test_dit_block_composition_against_dense_float64():
+    g = torch.Generator().manual_seed(73)
+    bf16 = torch.bfloat16
+    dim, heads, hd, ffn, s_tok, s_txt = 256, 4, 64, 512, 48, 24
+    W, P = {}, {}
+    for n, (o, i) in {"to_qkv": (3 * dim, dim), "to_out": (dim, dim), "to_q2": (dim, dim), "to_k2": (dim, dim), "to_v2": (dim, dim),
+                      "to_out2": (dim, dim), "ff_up": (ffn, dim), "ff_down": (dim, ffn)}.items():
+        W[n] = ((torch.randn(o, i, generator=g) / math.sqrt(i)).to(bf16), torch.randn(o, generator=g) * 0.1)
+        codes, scales = O.ref_quant(W[n][0], E4M3)
+        P[n] = (codes, scales, W[n][1])
+    for n in ("norm1", "norm2", "norm3"):
+        W[n] = P[n] = torch.rand(dim, generator=g) + 0.5
+    hidden = torch.randn(2, s_tok, dim, generator=g).to(bf16)
+    text = torch.randn(2, s_txt, dim, generator=g).to(bf16)
+    grid = torch.stack(torch.meshgrid(torch.arange(2), torch.arange(4), torch.arange(6), indexing="ij")).reshape(3, -1)
+    freqs = O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim)
+    lens = torch.tensor([24, 5], dtype=torch.int32)
+    got = O.ref_dit_block(hidden, text, freqs, lens, P, heads, hd)
+    want = _dense_dit_block(W, hidden, text, freqs, lens, heads, hd)
+    assert got.shape == hidden.shape and got.dtype == bf16
+    clean = _cos(got, want)
+    assert clean >= 0.99, clean
+    rel = ((got.double() - want).norm() / want.norm()).item()
+    for mut in ("qkv_order", "no_rope", "no_residual1", "no_mask", "wrong_norm", "no_gelu", "no_residual3"):
+        bad = _dense_dit_block(W, hidden, text, freqs, lens, heads, hd, mutate=mut)
+        rel_bad = ((got.double() - bad).norm() / bad.norm()).item()
+        assert rel_bad > 2.0 * rel and _cos(got, bad) < clean, (mut, rel_bad, rel)
