@@ -119,7 +119,6 @@ def _cpu_blas_gemm(x, w, bias):
 def _extras(dev, steps, warmup):
     from q8_kernels_amd import _C
     from q8_kernels_amd.blocks import Fp8DiTBlock
-    from oracle import q8_oracle as O
     out = {}
     g = torch.Generator().manual_seed(1)
     # fp8 self-attention with Hadamard, per-token e4m3 (config 3) and reference-style direct casts
@@ -185,9 +184,8 @@ def _extras(dev, steps, warmup):
     blk = Fp8DiTBlock(device=dev).init_random()
     hidden = torch.randn(2, 6144, 2048, generator=g).to(torch.bfloat16).to(dev)
     text = torch.randn(2, 128, 2048, generator=g).to(torch.bfloat16).to(dev)
-    f, hh, ww = 16, 16, 24
-    grid = torch.stack(torch.meshgrid(torch.arange(f), torch.arange(hh), torch.arange(ww), indexing="ij")).reshape(3, -1)
-    cosf, sinf = (t_.to(dev) for t_ in O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), 2048))
+    from q8_kernels_amd.functional.rope import precompute_freqs_cis, video_index_grid
+    cosf, sinf = precompute_freqs_cis(video_index_grid(16, 16, 24, batch=2, device=dev), 2048)
     with torch.no_grad():
         t, _ = _time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
     out["dit_block"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12, "shape": "tokens [2,6144,2048], text [2,128,2048]"}

@@ -14,6 +14,10 @@ Pinning status:
                                  ref_epilogue, ref_rms_norm, ref_rope, ref_attention, ref_freqs_cis,
                                  ref_fma (exact rational arithmetic), ref_gelu_backward, ref_rms_norm_backward,
                                  ref_rope_backward (float64 autograd of the forward formulas, adjoint identity)
+  pinned by a dense evaluation . ref_attention_module, ref_ltx_block, ref_dit_block: float64 x @ W.T / softmax /
+                                 modulation on the unquantized weights, written from the reference's module text;
+                                 mutants of it (swapped shift and scale, a missing gate, norm after the rotation,
+                                 rotation in the cross-attention, no mask ...) are each rejected
   parity unpinned (bit level) .. the low-order bits the reference gets from nvcc --use_fast_math
                                  (approximate division in the quantizer, tanhf / exp2f / rsqrtf) and the
                                  accumulation order inside mma.sync; unobservable without an sm_89 GPU.

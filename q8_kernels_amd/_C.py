@@ -393,9 +393,10 @@ def norm_mod_fht_quant(x: torch.Tensor, norm: bool = True, norm_weight: Optional
                 raise RuntimeError("norm_mod_fht_quant: mod_scale / mod_shift must be [B, 1 or T, dim], both bfloat16 or float32")
         mod_scale, mod_shift = mod_scale.contiguous(), mod_shift.contiguous()
         rows_per_mod, mod_dt = shape[1] // mod_scale.shape[1], _DT[mod_scale.dtype]
+    norm_w = None if norm_weight is None else norm_weight.contiguous()  # bound to a name: alive across the launch
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().q8_norm_mod_fht_quant_rows(
-            x2.data_ptr(), _ptr(None if norm_weight is None else norm_weight.contiguous()), int(norm), _ptr(mod_scale),
+            x2.data_ptr(), _ptr(norm_w), int(norm), _ptr(mod_scale),
             _ptr(mod_shift), mod_dt, rows_per_mod, float(scale_add), int(fht_scale is not None),
             float(fht_scale if fht_scale is not None else 1.0), out.data_ptr(), _DT[out_type], scales.data_ptr(), rows, dim,
             0, _stream(x)))
@@ -595,8 +596,9 @@ def rms_norm_backward(x_normed: torch.Tensor, x_norms: torch.Tensor, grad_out: t
     if weights is not None and (weights.dtype != torch.float32 or not weights.is_cuda or weights.numel() != dim):
         raise RuntimeError("rms_norm_backward: weights error")
     out = torch.empty((rows, dim), dtype=out_type, device=x_normed.device)
+    norms, w = x_norms.contiguous(), (None if weights is None else weights.contiguous())  # alive across the launch
     with torch.cuda.device(x_normed.device):
-        _lib.check(_lib.lib().q8_rmsnorm_backward(y2.data_ptr(), _DT[y2.dtype], x_norms.contiguous().data_ptr(), g2.data_ptr(),
-                                                  _DT[g2.dtype], _ptr(None if weights is None else weights.contiguous()),
+        _lib.check(_lib.lib().q8_rmsnorm_backward(y2.data_ptr(), _DT[y2.dtype], norms.data_ptr(), g2.data_ptr(),
+                                                  _DT[g2.dtype], _ptr(w),
                                                   out.data_ptr(), _DT[out_type], rows, dim, _stream(x_normed)))
     return out.reshape(x_normed.shape)

@@ -17,6 +17,10 @@ from ..modules.rms_norm import RMSNorm
 
 
 class Fp8DiTBlock(nn.Module):
+    # True (default): RMSNorm + quantizer, the attention prologues and the residual additions run fused into their
+    # neighbours; False: one operator per step of the docstring's sequence. Both give the same bits.
+    fuse = True
+
     def __init__(self, dim: int = 2048, num_heads: int = 32, head_dim: int = 64, ffn_dim: int = 8192,
                  text_dim: int = 2048, device=None):
         super().__init__()
@@ -52,7 +56,27 @@ class Fp8DiTBlock(nn.Module):
         return Q8F.linear.fp8_linear(codes, layer.weight.data, layer.bias.data, scales, layer.scales, False, x.dtype,
                                      fuse_gelu=fuse_gelu)
 
+    def _forward_by_operator(self, hidden, text, freqs_cis, text_lens):
+        bf16 = torch.bfloat16
+        d, h = self.dim, self.num_heads
+        b = hidden.shape[0]
+        heads = lambda t: t.reshape(b, -1, h, self.head_dim).transpose(1, 2)  # noqa: E731
+        merge = lambda t: t.transpose(1, 2).reshape(b, -1, d)  # noqa: E731
+        lin = lambda layer, x, gelu=False: Q8F.linear.fp8_linear(  # noqa: E731
+            x, layer.weight.data, layer.bias.data, None, layer.scales, False, bf16, fuse_gelu=gelu).reshape(b, -1, layer.out_features)
+        q, k, v = lin(self.to_qkv, self.norm1(hidden)).split(d, dim=-1)
+        q, k = Q8F.rope.apply_rope(q.contiguous(), *freqs_cis), Q8F.rope.apply_rope(k.contiguous(), *freqs_cis)
+        a = Q8F.flash_attention.flash_attn_func(heads(q), heads(k), heads(v), None, None, True, out_dtype=bf16)
+        hidden = hidden + lin(self.to_out, merge(a))
+        n = self.norm2(hidden)
+        a = Q8F.flash_attention.flash_attn_func(heads(lin(self.to_q2, n)), heads(lin(self.to_k2, text)), heads(lin(self.to_v2, text)),
+                                                None, text_lens, True, out_dtype=bf16)
+        hidden = hidden + lin(self.to_out2, merge(a))
+        return hidden + lin(self.ff_down, lin(self.ff_up, self.norm3(hidden), True))
+
     def forward(self, hidden, text, freqs_cis, text_lens):
+        if not self.fuse:
+            return self._forward_by_operator(hidden, text, freqs_cis, text_lens)
         bf16 = torch.bfloat16
         d, h = self.dim, self.num_heads
         # self-attention: q, k, v are read in place from the fused projection by the attention prologue kernels

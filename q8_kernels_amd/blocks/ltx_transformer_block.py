@@ -35,7 +35,7 @@ class LTXTransformerBlock(nn.Module):
                 and not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad or z.requires_grad))):
             bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
             return Q8F.fma.multiply_add(x.contiguous(), bf(y), bf(z), add)
-        return x * (y + add) + z
+        return (x * (y + add) + z).to(x.dtype)  # differentiable; in x's dtype like the kernel's result
 
     def forward(self, hidden_states, freqs_cis, attention_mask, encoder_hidden_states, encoder_attention_mask,
                 timestep, mm_out_dtype=torch.bfloat16, non_mm_precision=torch.bfloat16, attn_type="torch"):
@@ -44,9 +44,11 @@ class LTXTransformerBlock(nn.Module):
             hidden_states.shape[0], timestep.shape[1], num_ada_params, -1)
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada_values.unbind(dim=2)
 
+        # the fused prologue goes through the C ABI and carries no gradient: it is taken only when neither the input nor
+        # the modulation (scale_shift_table is a parameter, timestep may be the output of a trained embedding) needs one
         fuse = (self.fuse_prologue and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16
                 and non_mm_precision == torch.bfloat16 and hidden_states.dim() == 3 and hidden_states.shape[-1] % 8 == 0
-                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or timestep.requires_grad)))
+                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or ada_values.requires_grad)))
         bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
 
         if fuse:  # (int8 codes, row scales) of the rotated, modulated norm: what attn1's projections would compute

@@ -82,7 +82,9 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         const v4i* src = reinterpret_cast<const v4i*>(Qg + (size_t)row * 64 + 32 * h);
         const v4i a = src[0], c = src[1];
         qf[t] = v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
-        sqc[t] = SCALED ? p.sq[(size_t)bh * M + row] * p.scale_log2 : p.scale_log2;
+        // an all-zero query row has scale 0: kept strictly positive, so that a masked key's -inf times it stays -inf
+        // instead of becoming NaN (the row then weighs its valid keys uniformly, as zero logits do)
+        sqc[t] = SCALED ? fmaxf(p.sq[(size_t)bh * M + row] * p.scale_log2, 1.17549435e-38f) : p.scale_log2;
     }
 
     // copy plan: wave w fills LDS rows 16w .. 16w+15 of both tiles (64-byte rows, 4 chunks of 16 bytes,

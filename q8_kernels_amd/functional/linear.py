@@ -33,6 +33,22 @@ def _needs_grad(t) -> bool:
     return torch.is_grad_enabled() and isinstance(t, torch.Tensor) and t.requires_grad
 
 
+class GeluFn(torch.autograd.Function):
+    """tanh-GELU on the gelu_forward / gelu_backward kernels (csrc/ops/gelu_forward_cuda.cu, gelu_backward_cuda.cu of the
+    reference): what a fused-GELU linear falls back to when its input needs a gradient."""
+
+    @staticmethod
+    def forward(ctx, x, out_dtype):
+        ctx.save_for_backward(x)
+        ctx.out_dtype = out_dtype
+        return _C.gelu_forward(x.contiguous(), out_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        return _C.gelu_backward(x.contiguous(), grad_output.to(x.dtype).contiguous(), ctx.out_dtype).to(x.dtype), None
+
+
 # ----------------------------------------------------------------------------- int8
 
 def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=None):
@@ -89,7 +105,12 @@ def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = N
     `residual` (bfloat16, the output's shape, out_dtype bfloat16) returns `residual + linear(a)` with the addition done
     in the GEMM's epilogue: the bits of the separate bfloat16 addition."""
     if _needs_grad(a):
-        out = Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
+        if fuse_gelu and out_dtype is not None and is_16bit(out_dtype):
+            # the reference's backward ignores a fused GELU (functional/linear.py:44-52); here the activation follows as
+            # its own differentiable step
+            out = GeluFn.apply(Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, False, out_dtype), out_dtype)
+        else:
+            out = Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
         return out if residual is None else out + residual.reshape(out.shape)
     return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual)[0]
 
@@ -147,8 +168,11 @@ def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = 
 
     Keyword-only extensions (defaults = the reference's behaviour): `fuse_gelu` applies tanh-GELU in the epilogue;
     `residual` (bfloat16, the output's shape) returns `residual + linear(a)` with the addition done in the epilogue."""
-    if _needs_grad(a) and not fuse_gelu and residual is None:
-        return FP8LinearFunc.apply(a, b, bias, scale_a, scale_b, out_dtype, use_hadamard)
+    if _needs_grad(a):  # the fused epilogues carry no gradient: GELU and the residual addition follow as separate steps
+        out = FP8LinearFunc.apply(a, b, bias, scale_a, scale_b, out_dtype, use_hadamard)
+        if fuse_gelu:
+            out = GeluFn.apply(out, out_dtype)
+        return out if residual is None else out + residual.reshape(out.shape)
     return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual)[0]
 
 
@@ -169,9 +193,12 @@ class Q8LinearLora(torch.autograd.Function):
         assert is_16bit(lora_a) and is_16bit(lora_b), "Q8LinearFuncLora: lora_a and lora_b must be in 16bit"
         assert lora_a.shape[0] == lora_b.shape[-1], "Q8LinearFuncLora: lora_a and lora_b shape missmatch"
         assert out_dtype is not None and is_16bit(out_dtype), "Q8LinearFuncLora: out_dtype must be float16 or bfloat16"
-        a_q, sa = _rotate_quant(a) if use_hadamard else quantize(a)
+        # the forward always rotates both operands (q8_kernels/functional/linear.py:74-77): an int8 weight is taken to
+        # hold the rotated matrix, as Q8Linear.from_linear and convert_state_dict store it; use_hadamard only says
+        # whether the backward rotates the gradient back (:115-128)
+        a_q, sa = _rotate_quant(a)
         if b.dtype != torch.int8:
-            b, scale_b = _rotate_quant(b) if use_hadamard else quantize(b)
+            b, scale_b = _rotate_quant(b)
         if bias is not None:
             base = _C.q8_mm_bias(a_q, b, bias, sa, scale_b, False, out_dtype)
         else:

@@ -30,3 +30,49 @@ def apply_rope(x: torch.Tensor, cos_freqs: torch.Tensor, sin_freqs: torch.Tensor
     if torch.is_grad_enabled() and x.requires_grad:
         return ROPE.apply(x, cos_freqs, sin_freqs, out_type)
     return rope(x, cos_freqs, sin_freqs, out_type)
+
+
+def video_index_grid(frames: int, height: int, width: int, batch: int = 1, device=None) -> torch.Tensor:
+    """Integer (t, y, x) coordinates of a frames x height x width latent grid, token order t-major: float32
+    [batch, 3, frames * height * width], the `indices_grid` that precompute_freqs_cis takes."""
+    axes = [torch.arange(n, dtype=torch.float32, device=device) for n in (frames, height, width)]
+    t, y, x = torch.meshgrid(*axes, indexing="ij")
+    return torch.stack((t, y, x)).reshape(1, 3, -1).expand(batch, -1, -1)
+
+
+def precompute_freqs_cis(indices_grid: torch.Tensor, dim: int, theta: float = 10000.0,
+                         max_pos=(20, 2048, 2048), spacing: str = "exp"):
+    """The 3-D fractional rotary tables of the LTX-Video transformer (q8_kernels/models/LTXVideo.py:85-148):
+    indices_grid [B, 3, T] -> (cos, sin), float32 [B, T, dim], in the layout apply_rope takes.
+
+    Each of the dim // 6 frequencies w_f is applied to the three coordinates c_a / max_pos[a] mapped to [-1, 1]
+    ('exp', 'linear', 'sqrt') or left in [0, 1] ('exp_2'); column 6 f + 2 a (+ 1) of the tables holds the angle
+    w_f * position_a, every angle twice (the two members of a rotated pair), and the dim % 6 left-over columns in front
+    are the identity rotation."""
+    import math
+    n = dim // 6
+    dev = indices_grid.device
+    if spacing == "exp":
+        w = theta ** torch.linspace(0.0, 1.0, n, device=dev, dtype=torch.float32)
+    elif spacing == "exp_2":
+        w = (1.0 / theta ** (torch.arange(0, dim, 6, device=dev) / dim)).to(torch.float32)
+    elif spacing == "linear":
+        w = torch.linspace(1.0, theta, n, device=dev, dtype=torch.float32)
+    elif spacing == "sqrt":
+        w = torch.linspace(1.0, theta ** 2, n, device=dev, dtype=torch.float32).sqrt()
+    else:
+        raise ValueError("precompute_freqs_cis: spacing %r" % (spacing,))
+    w = w * (math.pi / 2)
+    scale = torch.tensor([1.0 / m for m in max_pos], dtype=torch.float32, device=dev)
+    pos = indices_grid.to(torch.float32) * scale[None, :, None]     # [B, 3, T] fractional positions
+    if spacing != "exp_2":
+        pos = pos * 2 - 1
+    ang = pos.transpose(1, 2)[:, :, None, :] * w[None, None, :, None]  # [B, T, n, 3]: frequency-major, axis-minor
+    ang = ang.reshape(ang.shape[0], ang.shape[1], 3 * n)
+    b, t = ang.shape[:2]
+    cos = torch.ones(b, t, dim, dtype=torch.float32, device=dev)
+    sin = torch.zeros(b, t, dim, dtype=torch.float32, device=dev)
+    lead = dim - 6 * n
+    cos[:, :, lead:] = ang.cos().repeat_interleave(2, dim=-1)
+    sin[:, :, lead:] = ang.sin().repeat_interleave(2, dim=-1)
+    return cos, sin

@@ -74,7 +74,8 @@ class Attention(nn.Module):
             would do exactly that to the same x on its own)."""
             if isinstance(x, tuple):  # already (int8 codes, row scales)
                 return [layer(x[0], x[1], out_dtype=mm_out_dtype) for layer in layers]
-            if self.fuse_prologue and len(layers) > 1 and x.is_cuda and Q8F.fused.can_fuse_hadamard_quantize(x):
+            if (self.fuse_prologue and len(layers) > 1 and x.is_cuda and Q8F.fused.can_fuse_hadamard_quantize(x)
+                    and not (torch.is_grad_enabled() and x.requires_grad)):  # the shared codes carry no gradient
                 xq, xs = Q8F.fused.hadamard_quantize(x)
                 return [layer(xq, xs, out_dtype=mm_out_dtype) for layer in layers]
             return [layer(x, out_dtype=mm_out_dtype) for layer in layers]
@@ -88,7 +89,8 @@ class Attention(nn.Module):
         if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64
                 and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
                 and non_mm_precision == torch.bfloat16 and query.dim() == 3
-                and all(t.dtype == torch.bfloat16 for t in (query, key, value))):
+                and all(t.dtype == torch.bfloat16 for t in (query, key, value))
+                and not (torch.is_grad_enabled() and any(t.requires_grad for t in (query, key, value)))):
             # qk-RMSNorm, RoPE, head split, Hadamard and the e4m3 cast in one prologue kernel, head-merged attention
             # output: the same bits as the sequence below
             hidden_states = Q8F.fused.flash_attn_token_major(

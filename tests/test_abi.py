@@ -194,3 +194,19 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode == 2
     assert "one GPU" in r.stderr and "--gpus 2" in r.stderr
     assert r.stdout.strip() == ""
+
+
+def test_precompute_freqs_cis_matches_the_oracle_tables():
+    """The package's own builder of the 3-D rotary tables against the oracle's restatement of
+    q8_kernels/models/LTXVideo.py:85-148 (itself pinned by explicit loops over frequency and axis)."""
+    import torch
+    from oracle import q8_oracle as O
+    from q8_kernels_amd.functional.rope import precompute_freqs_cis, video_index_grid
+    grid = video_index_grid(3, 4, 5, batch=2)
+    assert grid.shape == (2, 3, 60) and grid[0, :, 27].tolist() == [1.0, 1.0, 2.0]
+    for dim in (2048, 256, 100):
+        cos, sin = precompute_freqs_cis(grid, dim)
+        want_cos, want_sin = O.ref_freqs_cis(grid, dim)
+        assert cos.dtype == torch.float32 and cos.shape == (2, 60, dim)
+        assert torch.allclose(cos, want_cos, atol=1e-6) and torch.allclose(sin, want_sin, atol=1e-6)
+        assert torch.equal(cos[..., 0::2], cos[..., 1::2]) and torch.equal(sin[..., 0::2], sin[..., 1::2])

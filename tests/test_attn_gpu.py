@@ -277,3 +277,24 @@ def test_workgroup_shapes_give_identical_bits(dev):
     for cfg in (1, 2):
         assert torch.equal(outs[cfg][0], outs[0][0]), "direct casts, shape %d" % cfg
         assert torch.equal(outs[cfg][1], outs[0][1]), "per-token scales, shape %d" % cfg
+
+
+def test_zero_query_row_with_scales_and_masked_keys(dev, attn_cfg):
+    """An all-zero query row is quantized to scale 0. With a partial or masked tile its masked keys are -inf, and
+    -inf times that zero scale must not turn the row into NaN: zero logits weigh the valid keys uniformly, as the
+    oracle does."""
+    g = torch.Generator().manual_seed(15)
+    b, h, m, n = 2, 2, 70, 100
+    qf = torch.randn(b, h, m, 64, generator=g)
+    qf[0, 0, 3] = 0
+    qf[1, 1, 64:] = 0
+    kf, vf = torch.randn(b, h, n, 64, generator=g), torch.randn(b, h, n, 64, generator=g)
+    (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+    assert sq[0, 0, 3] == 0 and (sq[1, 1, 64:] == 0).all()
+    lens = torch.tensor([100, 37], dtype=torch.int32)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
+                               q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+    assert not torch.isnan(got).any()
+    _check(got, q, k, v, 0.125, lens, (sq, sk, sv), what="zero query rows")
+    mean_v = (v[1, 1, :37].double() * sv[1, 1, :37, None].double()).mean(dim=0)
+    assert (got[1, 1, 64:].cpu().double() - mean_v).abs().max() <= 0.07 * mean_v.abs().max() + 0.02

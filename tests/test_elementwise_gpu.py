@@ -175,6 +175,105 @@ def test_linear_backward_and_lora(dev):
         assert cosine(lora.lora_b.grad.cpu(), lb.grad.cpu()) > 0.99
 
 
+def test_gradients_reach_every_input_that_asks_for_one(dev):
+    """Three places where a gradient used to be dropped without an error: a bare hadamard_transform, fp8_linear with a
+    fused GELU or residual, q8_linear with a fused GELU. Each against float64 autograd of the dense formula."""
+    import scipy.linalg
+    import q8_kernels_amd.functional as Q8F
+    g = torch.Generator().manual_seed(50)
+    x = torch.randn(3, 17, 256, generator=g).to(BF16)
+    go = torch.randn(3, 17, 256, generator=g).to(BF16)
+    # hadamard_transform: y = x H / 16, dy/dx = H / 16 (symmetric)
+    xd = x.to(dev).requires_grad_(True)
+    y = Q8F.fast_hadamard.hadamard_transform(xd)
+    assert y.requires_grad and y.grad_fn is not None
+    y.backward(go.to(dev))
+    H = torch.tensor(scipy.linalg.hadamard(256), dtype=torch.float64) / 16.0
+    assert xd.grad.dtype == BF16 and cosine(xd.grad.cpu(), go.double() @ H) > 0.99999
+    # linears with fused epilogues
+    w = (torch.randn(128, 256, generator=g) / 16).to(BF16)
+    bias = torch.randn(128, generator=g) * 0.1
+    res = torch.randn(3, 17, 128, generator=g).to(BF16)
+    go2 = torch.randn(3, 17, 128, generator=g).to(BF16)
+    for kind in ("fp8_gelu", "fp8_residual", "fp8_gelu_residual", "q8_gelu"):
+        xd = x.to(dev).requires_grad_(True)
+        rd = res.to(dev).requires_grad_(True)
+        if kind.startswith("fp8"):
+            out = Q8F.linear.fp8_linear(xd, w.to(dev), bias.to(dev), out_dtype=BF16, fuse_gelu="gelu" in kind,
+                                        residual=rd if "residual" in kind else None)
+        else:
+            out = Q8F.linear.q8_linear(xd, w.to(dev), bias.to(dev), fuse_gelu=True, out_dtype=BF16)
+        assert out.grad_fn is not None, kind
+        out.reshape(3, 17, 128).backward(go2.to(dev))
+        xr = x.double().requires_grad_(True)
+        rr = res.double().requires_grad_(True)
+        pre = xr @ w.double().T + bias.double()
+        want = torch.nn.functional.gelu(pre, approximate="tanh") if "gelu" in kind else pre
+        if "residual" in kind:
+            want = want + rr
+        want.backward(go2.double())
+        assert cosine(out.detach().cpu(), want.detach()) > 0.998, kind
+        assert cosine(xd.grad.cpu(), xr.grad) > 0.99, kind
+        if "residual" in kind:
+            assert cosine(rd.grad.cpu(), rr.grad) > 0.99999, kind
+
+
+def test_ltx_block_modulation_table_gets_its_gradient(dev):
+    """scale_shift_table is a parameter. With gradients enabled and an input that does not need one, the block must
+    not take the fused prologue (which carries no gradient): the table's gradient through scale and shift, not only
+    through the gates, is compared with float64 autograd of the dense block on the dequantized weights."""
+    import scipy.linalg
+    import torch.nn as nn
+    from q8_kernels_amd.blocks import LTXTransformerBlock
+    from q8_kernels_amd.modules import Q8Linear
+    from tests.test_oracle import _dense_ltx_block
+    torch.manual_seed(51)
+    dim, heads, hd, kv_dim, s_tok, s_txt = 256, 4, 64, 128, 48, 24
+    blk = LTXTransformerBlock(dim, heads, hd, kv_dim, bias=True, use_rope=True, norm_affine=False).to(dev)
+    W = {}
+    for name, m in blk.named_modules():
+        if isinstance(m, Q8Linear):
+            src = nn.Linear(m.in_features, m.out_features).to(dev).to(BF16)
+            q = Q8Linear.from_linear(src)
+            m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+            key = {"ff.act.proj": "ff.up", "ff.proj_down": "ff.down"}.get(name, name)
+            W[key] = (src.weight.data.cpu(), src.bias.data.float().cpu())
+    for a in ("attn1", "attn2"):
+        W[a + ".q_norm"] = getattr(blk, a).q_norm.weight.data.cpu()
+        W[a + ".k_norm"] = getattr(blk, a).k_norm.weight.data.cpu()
+    g = torch.Generator().manual_seed(52)
+    hidden = torch.randn(2, s_tok, dim, generator=g).to(BF16)
+    text = torch.randn(2, s_txt, kv_dim, generator=g).to(BF16)
+    timestep = torch.randn(2, 1, 6 * dim, generator=g) * 0.3
+    go = torch.randn(2, s_tok, dim, generator=g).to(BF16)
+    grid = torch.stack(torch.meshgrid(torch.arange(2), torch.arange(4), torch.arange(6), indexing="ij")).reshape(3, -1)
+    cos, sin = O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim)
+    lens = torch.tensor([24, 9], dtype=torch.int32)
+    impl, calls = _C().norm_mod_fht_quant, []
+    def counted(*a, **k):
+        calls.append(1)
+        return impl(*a, **k)
+    try:
+        _C().norm_mod_fht_quant = counted
+        out = blk(hidden.to(dev), (cos.to(dev), sin.to(dev)), None, text.to(dev), lens.to(dev), timestep.to(dev),
+                  attn_type="torch")  # the differentiable attention (the fp8 kernel is forward-only, as in the reference)
+    finally:
+        _C().norm_mod_fht_quant = impl
+    assert not calls, "the fused prologue ran although scale_shift_table needs a gradient"
+    out.backward(go.to(dev))
+    got = blk.scale_shift_table.grad
+    assert got is not None and torch.isfinite(got).all()
+    Wd = dict(W)
+    table = blk.scale_shift_table.data.cpu().double().requires_grad_(True)
+    Wd["scale_shift_table"] = table
+    want_out = _dense_ltx_block(Wd, hidden, (cos, sin), text, lens, timestep, heads, hd)
+    want_out.backward(go.double())
+    assert cosine(out.detach().cpu(), want_out.detach()) > 0.995
+    for row, name in enumerate(("shift_msa", "scale_msa", "gate_msa", "shift_mlp", "scale_mlp", "gate_mlp")):
+        assert got[row].abs().max() > 0, name
+        assert cosine(got[row].cpu(), table.grad[row]) > 0.97, (name, cosine(got[row].cpu(), table.grad[row]))
+
+
 # ------------------------------------------------------------------ LTX transformer block
 
 def test_ltx_transformer_block_matches_oracle(dev):

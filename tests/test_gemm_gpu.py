@@ -24,6 +24,9 @@ from q8_kernels_amd._lib import (Q8_GEMM_KERNEL_PERSIST192 as K_PERSIST192, Q8_G
                                  Q8_GEMM_KERNEL_TILE128 as K_TILE128)
 
 
+PERSISTENT_KERNELS = {K_PERSIST256, K_PERSIST192}  # the workgroup-per-CU kernels that walk over several tiles
+
+
 def _last_kernel():
     from q8_kernels_amd import _lib
     return _lib.lib().q8_gemm_last_kernel()
@@ -332,3 +335,33 @@ def test_operand_around_4_gib(dev, rows_over):
         assert int(diff.max()) <= 1, "rows %d..%d: %d ulp" % (lo, lo + 300, int(diff.max()))
     del a, out
     torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------ the block's M = 12288 GEMM shapes
+
+@pytest.mark.parametrize("nk", [(2048, 2048), (2048, 8192)], ids=["projection_K2048", "ffn_down_K8192"])
+def test_fp8_linear_block_shapes_m12288(dev, nk):
+    """The fp8 linears of the DiT block at their real size, tokens [12288, K] x weight [2048, K] + bias -> bf16, against
+    the float64 oracle on row blocks from the start, the middle (across a tile boundary) and the end of M. The kernel
+    that ran must be one of the persistent family (the large-problem path these shapes are timed on)."""
+    n, k = nk
+    m = 12288
+    g = torch.Generator().manual_seed(12 + k)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=g) * 0.02).to(torch.bfloat16).float()
+    xq, sx = _C().tokenwise_quant(x.to(dev), E4M3)
+    wq, sw = _C().tokenwise_quant(w.to(dev), E4M3)
+    out = _C().fp8_mm_bias(xq, wq, bias.to(dev), sx, sw, False, torch.bfloat16)
+    kernel = _last_kernel()
+    assert kernel in PERSISTENT_KERNELS, kernel
+    assert out.shape == (1, m, n)
+    owq, osw = O.ref_quant(w, E4M3)
+    assert_bit_equal(wq, owq, "W codes")
+    for lo in (0, 6144 - 160, m - 320):
+        rows = slice(lo, lo + 320)
+        oxq, osx = O.ref_quant(x[rows], E4M3)
+        assert_bit_equal(xq[rows], oxq, "X codes")
+        v = O.ref_gemm_fp8_acc(oxq, owq) * (osx[:, None] * osw[None, :]).double() + bias.double()
+        _check_float_out(out[0, rows], v, "M=12288 N=%d K=%d rows %d.." % (n, k, lo))
+    assert torch.isfinite(out.float()).all()
