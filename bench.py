@@ -159,6 +159,14 @@ def _extras(dev, steps, warmup):
         gb = gb.to(dev)
         t, _ = _time(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, False, torch.bfloat16), steps, warmup)
         out[name] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12, "frac_of_fp8_peak": 2.0 * mm * nn * kk / t / 1e12 / FP8_PEAK_TFLOPS}
+        if kk == 2048:
+            # the reference's default output type: out_type None -> e4m3 (csrc/gemm/q8_gemm_api.cpp:82-87), fp8 and int8 operands
+            t, _ = _time(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, False, None), steps, warmup)
+            out[name + "_e4m3_out"] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12,
+                                       "frac_of_fp8_peak": 2.0 * mm * nn * kk / t / 1e12 / FP8_PEAK_TFLOPS}
+            ai, bi = gxq.view(torch.int8), gwq.view(torch.int8)  # any int8 codes do for timing
+            t, _ = _time(lambda: _C.q8_mm_bias(ai, bi, gb, gsx, gsw, False, None), steps, warmup)
+            out["int8_gemm_%dx%dx%d_e4m3_out" % (mm, nn, kk)] = {"ms": t * 1e3, "tops": 2.0 * mm * nn * kk / t / 1e12}
         del gxq, gwq
     # row kernels on [12288, 2048] tokens
     x = torch.randn(12288, 2048, generator=g).to(torch.bfloat16).to(dev)

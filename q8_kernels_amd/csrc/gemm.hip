@@ -206,7 +206,7 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
     return launch_status("q8_gemm");
 }
 
-// One workgroup per CU walking over the tiles (gemm_persist.h); bf16 output, N % 8 == 0, K a multiple of 128 above 256.
+// One workgroup per CU walking over the tiles (gemm_persist.h); bf16 or e4m3 output, N % 8 == 0, K a multiple of 128 above 256.
 // The tile height is 256 or 192 rows, whichever gives the shorter schedule: work per CU = rounds x tile height, with
 // 20 % charged to the smaller tile (measured: a 192-row round takes 0.90 of a 256-row round, not 0.75: it moves 17 %
 // more operand bytes per flop and pays the same epilogue and barrier overheads).
@@ -229,14 +229,14 @@ static int persist_cus() {
     return cus;
 }
 
-template <int IN, bool GELU, int MT, bool RES>
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT>
 static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     constexpr int BM = 64 * MT;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     const long total = (long)tiles_m * tiles_n * batch;
     if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
-    auto kern = gemm_persist_kernel<IN, GELU, MT, RES>;
+    auto kern = gemm_persist_kernel<IN, GELU, MT, RES, E4M3OUT>;
     g_last_kernel = (MT == 4 ? Q8_GEMM_KERNEL_PERSIST256 : Q8_GEMM_KERNEL_PERSIST192) | (RES ? Q8_GEMM_KERNEL_RESIDUAL : 0);
     static thread_local int lds_dev = -1;
     if (int st = reserve_lds(reinterpret_cast<const void*>(kern), kPersistLds, lds_dev)) return st;
@@ -248,7 +248,7 @@ static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
 
 static int g_persist_mt = 0;  // 0 = choose, 3 / 4 = forced tile height 192 / 256 (tuning)
 
-template <int IN, bool GELU>
+template <int IN, bool GELU, bool E4M3OUT = false>
 static int launch_persist(const GemmParams& p, hipStream_t stream) {
     const long batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     const long tn = (p.N + kPipeBN - 1) / kPipeBN, cus = persist_cus();
@@ -257,12 +257,14 @@ static int launch_persist(const GemmParams& p, hipStream_t stream) {
         return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? 1.0 : 1.2);
     };
     const bool small = g_persist_mt == 3 || (g_persist_mt == 0 && cost(192) < cost(256));
-    if (p.residual != nullptr)
-        return small ? launch_persist_mt<IN, GELU, 3, true>(p, stream) : launch_persist_mt<IN, GELU, 4, true>(p, stream);
-    return small ? launch_persist_mt<IN, GELU, 3, false>(p, stream) : launch_persist_mt<IN, GELU, 4, false>(p, stream);
+    if constexpr (!E4M3OUT) {
+        if (p.residual != nullptr)
+            return small ? launch_persist_mt<IN, GELU, 3, true, false>(p, stream) : launch_persist_mt<IN, GELU, 4, true, false>(p, stream);
+    }
+    return small ? launch_persist_mt<IN, GELU, 3, false, E4M3OUT>(p, stream) : launch_persist_mt<IN, GELU, 4, false, E4M3OUT>(p, stream);
 }
 
-// shapes the persistent kernel takes (its output is bf16)
+// shapes the persistent kernel takes (bf16 or e4m3 output)
 static bool persist_eligible(const GemmParams& p) {
     return (p.N % 8) == 0 && p.K > 256 && (p.K % 128) == 0 && (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32);
 }
@@ -271,8 +273,8 @@ template <int IN, int OUT, bool GELU>
 static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
     const long big_tiles = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.batch_a > p.batch_b ? p.batch_a : p.batch_b);
     const bool big = g_force_cfg == 1 || g_force_cfg == 4 || (g_force_cfg == 0 && big_tiles >= 192);
-    if constexpr (OUT == Q8_BF16) {
-        if (big && g_force_cfg != 1 && persist_eligible(p)) return launch_persist<IN, GELU>(p, stream);
+    if constexpr (OUT == Q8_BF16 || OUT == Q8_E4M3) {
+        if (big && g_force_cfg != 1 && persist_eligible(p)) return launch_persist<IN, GELU, OUT == Q8_E4M3>(p, stream);
     }
     if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
     if (g_force_cfg == 3) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);

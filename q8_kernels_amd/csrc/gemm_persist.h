@@ -47,14 +47,17 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 }
 
 // Requirements checked by the host: K % 128 == 0 and K > 256 (at least 3 whole stages per tile), N % 8 == 0,
-// M * K and N * K below 2^32 (32-bit source offsets), OUT == Q8_BF16.
+// M * K and N * K below 2^32 (32-bit source offsets).
+// E4M3OUT: the output is e4m3 (saturating cast, the reference's default output type, csrc/gemm/q8_gemm_api.cpp:82-87) instead
+// of bf16: every lane stores its 8-byte chunks straight from the MFMA layout (no residual form).
 // MT = 32-row MFMA tiles per wave along M: the tile is 64 MT x 256, i.e. 256 x 256 (MT = 4) or 192 x 256 (MT = 3, for
 // problems whose 256-row tiles do not divide evenly over the CUs).
 // RES: C = bf16(bf16(result) + residual), the residual connection around a projection (two roundings, as the separate
 // element-wise addition of the two bf16 tensors gives).
-template <int IN, bool GELU, int MT, bool RES>
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    static_assert(!(RES && E4M3OUT), "the residual epilogue writes bf16");
     constexpr int BM = 64 * MT, BN = kPipeBN;
     constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
     const int tid = threadIdx.x, lane = tid & 63;
@@ -302,9 +305,18 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         if constexpr (GELU) x = gelu_tanh_fast(x);
                         v[e] = x;
                     }
-                    outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
+                    if constexpr (E4M3OUT) {
+                        // 8 codes of row 32 i + r32; the two lane halves write 16 contiguous bytes of the row
+                        const int m = mw0 + 32 * i + r32, n = nw0 + 32 * t + 16 * wp + 8 * h;
+                        const v2i w = v2i{(int)pack4_e4m3_sat(v[0], v[1], v[2], v[3]), (int)pack4_e4m3_sat(v[4], v[5], v[6], v[7])};
+                        if (m < M && n < N) *reinterpret_cast<v2i*>(reinterpret_cast<uint8_t*>(p.C) + zc + (size_t)m * N + n) = w;
+                    } else {
+                        outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
+                    }
                 }
-            if constexpr (GELU && !RES) {
+            if constexpr (E4M3OUT) {
+                continue;
+            } else if constexpr (GELU && !RES) {
                 // With GELU the epilogue is bound by its arithmetic, and the round trips through the staging buffer
                 // below only add latency to it: the lane's four 16-byte chunks of row 32 i + r32 go straight to
                 // memory, 32 contiguous bytes per row and instruction (the four instructions complete the row's

@@ -34,7 +34,7 @@ def _last_kernel():
 
 def _kernels_for(cfg, n, k, bf16_out=True):
     """The kernels a call may launch under q8_gemm_set_config(cfg): the pins 1 and 2 always hold; 4 means the
-    persistent kernel for the shapes it takes (bf16 output, N % 8 == 0, K a multiple of 128 above 256) and the
+    persistent kernel for the shapes it takes (bf16 or e4m3 output, N % 8 == 0, K a multiple of 128 above 256) and the
     per-tile pipelined kernel otherwise. Asserted after the calls below so that a test of a pinned kernel cannot
     pass on a silent fall-back to another one."""
     if cfg == 1:
@@ -133,6 +133,7 @@ def test_mm_epilogue_vs_oracle(dev, tile_cfg, in_dtype, fuse_gelu, with_bias):
     _check_float_out(got[0], want64, "%s gelu=%s bias=%s" % (in_dtype, fuse_gelu, with_bias))
     # e4m3 output (the reference's default out_type): saturating cast of the same value
     got8 = fn(*args, None)
+    assert _last_kernel() in _kernels_for(tile_cfg, n, k), "e4m3 output: kernel %d under config %d" % (_last_kernel(), tile_cfg)
     assert got8.dtype == E4M3
     want8 = ref(a, b, bias, sa, sb, fuse_gelu, None)[0]
     g8, w8 = got8[0].cpu().float(), want8.float()
@@ -365,3 +366,20 @@ def test_fp8_linear_block_shapes_m12288(dev, nk):
         v = O.ref_gemm_fp8_acc(oxq, owq) * (osx[:, None] * osw[None, :]).double() + bias.double()
         _check_float_out(out[0, rows], v, "M=12288 N=%d K=%d rows %d.." % (n, k, lo))
     assert torch.isfinite(out.float()).all()
+    # the reference's default output type (out_type None -> e4m3, saturating cast) takes the same kernel family
+    out8 = _C().fp8_mm_bias(xq, wq, bias.to(dev), sx, sw, False, None)
+    assert _last_kernel() in PERSISTENT_KERNELS, _last_kernel()
+    assert out8.dtype == E4M3 and out8.shape == (1, m, n)
+    for lo in (0, m - 320):
+        rows = slice(lo, lo + 320)
+        oxq, osx = O.ref_quant(x[rows], E4M3)
+        v = O.ref_gemm_fp8_acc(oxq, owq) * (osx[:, None] * osw[None, :]).double() + bias.double()
+        want8 = O.e4m3_sat(v.float())
+        g8 = out8[0, rows].cpu()
+        assert not torch.isnan(g8.float()).any()
+        # fp32 accumulation order moves a value across an e4m3 rounding boundary now and then: never by more than one code
+        # (codes are sign-magnitude: taken as signed step counts, so that -0 = +0 and the smallest negative value is one
+        # step from zero)
+        steps = lambda c: (c & 0x7F) * (1 - 2 * (c >> 7))  # noqa: E731
+        diff = (steps(g8.view(torch.uint8).int()) - steps(want8.view(torch.uint8).int())).abs()
+        assert int(diff.max()) <= 1 and (diff > 0).float().mean() < 0.01, (int(diff.max()), (diff > 0).float().mean().item())
