@@ -47,6 +47,34 @@ constexpr int kStages = 4;      // LDS ring: one tile being read, up to three in
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Output stage shared by the attention kernels. The O^T accumulators of a 32-query tile: lane (q, h), tile d, register e
+// holds dim 32 d + 8 (e / 4) + 4 h + (e % 4) of query q, i.e. the two lanes of a query hold alternate groups of 4 dims.
+// One v_permlane32_swap per packed word hands every lane 8 consecutive dims (lane half 0 those of the even groups of 8,
+// lane half 1 the odd ones), so a lane stores 16 bytes of bf16 (8 bytes of e4m3) and the two lanes of a query 32 (16)
+// contiguous bytes per instruction: half as many, twice as large write requests as storing the groups of 4 directly.
+template <int OUT>
+__device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, const v16f (&o_acc)[2], float inv, bool live) {
+#pragma unroll
+    for (int d = 0; d < 2; ++d)
+#pragma unroll
+        for (int wp = 0; wp < 2; ++wp) {  // the pair of 8-dim groups 2 wp, 2 wp + 1 of this 32-dim tile
+            float a[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = o_acc[d][8 * wp + e] * inv;
+            // before: a[0..3] = dims 16 wp + 4 h + 0..3, a[4..7] = dims 16 wp + 8 + 4 h + 0..3 (relative to 32 d)
+            const int dim = 32 * d + 16 * wp + 8 * h;  // after: 8 consecutive dims from here
+            if constexpr (OUT == Q8_BF16) {
+                const auto s0 = __builtin_amdgcn_permlane32_swap(pack2_bf16(a[0], a[1]), pack2_bf16(a[4], a[5]), false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(pack2_bf16(a[2], a[3]), pack2_bf16(a[6], a[7]), false, false);
+                if (live) *reinterpret_cast<v4u*>(reinterpret_cast<uint16_t*>(o) + row_off + dim) = v4u{s0[0], s1[0], s0[1], s1[1]};
+            } else {
+                const auto s0 = __builtin_amdgcn_permlane32_swap(pack4_e4m3_sat(a[0], a[1], a[2], a[3]),
+                                                                 pack4_e4m3_sat(a[4], a[5], a[6], a[7]), false, false);
+                if (live) *reinterpret_cast<v2i*>(reinterpret_cast<uint8_t*>(o) + row_off + dim) = v2i{(int)s0[0], (int)s0[1]};
+            }
+        }
+}
+
 // kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
 template <int OUT, bool SCALED, int kQT, int kWaves>
 __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams p) {
@@ -305,25 +333,146 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         const int row = q0 + 32 * qt + ql;
         float l = l_run[qt] + lane_xor<32>(l_run[qt]);
         const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
-        if (row >= M) continue;
+        store_o_tile<OUT>(p.o, o_base + (size_t)row * o_rs, h, o_acc[qt], inv, row < M);
+    }
+}
+
+// Short key / value sequences (N <= 128: cross-attention to a text prompt, csrc/flash_attention/
+// flash_attention_cuda_mask.cu:254-535 in the reference). The whole K and V^T of a (batch, head) are 16 KiB: every wave
+// keeps them in registers as ready-made MFMA operands (64 registers, loaded once) and walks over many 32-query tiles with
+// them, so a tile costs one 2 KiB read of Q (requested one tile ahead) and one store of O and nothing else: no LDS, no
+// barrier, no running maximum (all keys of a query are present at once, the probabilities are rounded against the
+// final maximum like the oracle's). Operand layouts, masking, P rounding and the output stage are those of
+// attn_fwd_kernel; a 64-key block beyond the valid length is skipped. A workgroup belongs to one head and takes its
+// share of the queries of EVERY batch in turn: the valid lengths differ per batch, and with a workgroup per
+// (batch, head) the launch would last as long as its longest batch.
+template <int OUT>
+__global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int tiles_per_wave) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, h = lane >> 5;
+    const int M = p.M, N = p.N;
+    for (int b = 0; b < p.B; ++b) {
+        const int bh = b * p.H + blockIdx.y;
+        int valid = N;
+        if (p.kv_len) {
+            const int len = p.kv_len[b];
+            valid = len < N ? (len < 0 ? 0 : len) : N;
+        }
+        const uint8_t* Qg = p.q + (size_t)bh * M * 64;
+        const uint8_t* Kg = p.k + (size_t)bh * N * 64;
+        const uint8_t* Vg = p.v + (size_t)bh * 64 * p.v_row_stride;
+        const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
+        const size_t o_base = o_tok ? ((size_t)b * M * p.H + (size_t)(bh - b * p.H)) * 64 : (size_t)bh * M * 64;
+        const size_t o_rs = o_tok ? (size_t)p.H * 64 : 64;
+        const int n_blocks = (valid + 63) >> 6;  // 64-key blocks that hold valid keys: 0, 1 or 2
+
+        // K operand of block kb, tile t: lane (i, h) holds bytes 32 h .. 32 h + 31 of the key that comes out as row i of the
+        // S^T accumulator tile (lane half h then owns keys 32 h .. 32 h + 31 of the block in operand byte order);
+        // V^T operand of block kb, tile d: lane (i, h) holds keys 64 kb + 32 h .. + 31 of V^T row 32 d + i.
+        v8i kf[2][2], vf[2][2];
+        const v4i zero4 = v4i{0, 0, 0, 0};
 #pragma unroll
-        for (int d = 0; d < 2; ++d) {
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const int dim = 32 * d + 8 * w + 4 * h;
-                const float a0 = o_acc[qt][d][4 * w] * inv, a1 = o_acc[qt][d][4 * w + 1] * inv;
-                const float a2 = o_acc[qt][d][4 * w + 2] * inv, a3 = o_acc[qt][d][4 * w + 3] * inv;
-                if constexpr (OUT == Q8_BF16) {
-                    uint16_t* dst = reinterpret_cast<uint16_t*>(p.o) + o_base + (size_t)row * o_rs + dim;
-                    v2i wv;
-                    wv[0] = (int)pack2_bf16(a0, a1);
-                    wv[1] = (int)pack2_bf16(a2, a3);
-                    *reinterpret_cast<v2i*>(dst) = wv;
-                } else {
-                    uint8_t* dst = reinterpret_cast<uint8_t*>(p.o) + o_base + (size_t)row * o_rs + dim;
-                    *reinterpret_cast<uint32_t*>(dst) = pack4_e4m3_sat(a0, a1, a2, a3);
+            for (int t = 0; t < 2; ++t) {
+                int key = 64 * kb + 32 * ((ql >> 2) & 1) + 16 * t + 4 * (ql >> 3) + (ql & 3);
+                key = key < N ? key : N - 1;
+                const v4i* ks = reinterpret_cast<const v4i*>(Kg + (size_t)key * 64 + 32 * h);
+                v4i a = zero4, c = zero4, va = zero4, vc = zero4;
+                if (kb < n_blocks) {
+                    a = ks[0];
+                    c = ks[1];
+                    const int col = 64 * kb + 32 * h;
+                    const uint8_t* vs = Vg + (size_t)(32 * t + ql) * p.v_row_stride + col;
+                    if (col < p.v_row_stride) va = *reinterpret_cast<const v4i*>(vs);
+                    if (col + 16 < p.v_row_stride) vc = *reinterpret_cast<const v4i*>(vs + 16);
+                }
+                kf[kb][t] = v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
+                vf[kb][t] = v8i{va[0], va[1], va[2], va[3], vc[0], vc[1], vc[2], vc[3]};
+            }
+
+        const int q_tiles = (M + 31) >> 5;
+        const int wave_id = blockIdx.x * 8 + wave, waves = gridDim.x * 8;
+        auto load_q = [&](int tile) {  // Q^T operand: lane (q, h) holds bytes 32 h .. 32 h + 31 of query row q
+            int row = 32 * tile + ql;
+            row = row < M ? row : M - 1;
+            const v4i* src = reinterpret_cast<const v4i*>(Qg + (size_t)row * 64 + 32 * h);
+            const v4i a = src[0], c = src[1];
+            return v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
+        };
+        const float c = p.scale_log2;
+        int tile = wave_id;
+        v8i qf = load_q(tile < q_tiles ? tile : 0);
+        for (int it = 0; it < tiles_per_wave && tile < q_tiles; ++it, tile += waves) {
+            const int next = tile + waves;
+            const v8i qn = load_q(next < q_tiles ? next : tile);  // requested now, used in the next round
+            float x[2][32];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if (kb < n_blocks) {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        v16f z;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) z[e] = 0.f;
+                        const v16f s = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[kb][t], qf, z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) x[kb][16 * t + e] = s[e];
+                    }
+                    if (64 * kb + 64 > valid) {
+#pragma unroll
+                        for (int e = 0; e < 32; ++e)
+                            if (64 * kb + 32 * h + e >= valid) x[kb][e] = -INFINITY;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 32; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[kb][e]), x[kb][e + 1]);
                 }
             }
+            mx = fmaxf(mx, lane_xor<32>(mx));
+            // (no valid key at all: everything below is skipped and the output is zero)
+            const float m_sub = mx * c - p.p_shift;
+            float psum = 0.f;
+            v16f o_acc[2];
+#pragma unroll
+            for (int d = 0; d < 2; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o_acc[d][e] = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if (kb < n_blocks) {
+                    v8i pf;
+                    float pr[32];
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) {
+                        pr[e] = fast_exp2(fmaf(x[kb][e], c, -m_sub));
+                        psum += pr[e];
+                    }
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) {
+                        uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
+                        u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
+                        pf[w] = (int)u;
+                    }
+                    if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {
+#pragma unroll
+                        for (int e = 0; e < 32; ++e) psum -= pr[e];
+#pragma unroll
+                        for (int w = 0; w < 8; ++w)
+                            psum += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
+                    }
+#pragma unroll
+                    for (int d = 0; d < 2; ++d)
+                        o_acc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[kb][d], pf, o_acc[d], 0, 0, 0, 0, 0, 0);
+                }
+            }
+            // ---- O^T lane (q, h), tile d, register e holds dim 32 d + 8 (e/4) + 4 h + (e%4)
+            const int row = 32 * tile + ql;
+            const float l = psum + lane_xor<32>(psum);
+            const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
+            store_o_tile<OUT>(p.o, o_base + (size_t)row * o_rs, h, o_acc, inv, row < M);
+            qf = qn;
         }
     }
 }
@@ -332,10 +481,11 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
 
 using namespace q8;
 
-static int g_attn_cfg = 0;  // 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries
+static int g_attn_cfg = 0;  // 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries,
+                            // 3 = as 0 and without the register-resident path for N <= 128
 
 extern "C" int q8_attn_set_config(int cfg) {
-    if (cfg < 0 || cfg > 2) return fail(Q8_ERR_FLAGS, "q8_attn_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 3) return fail(Q8_ERR_FLAGS, "q8_attn_set_config: %d", cfg);
     g_attn_cfg = cfg;
     return Q8_OK;
 }
@@ -363,6 +513,19 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
                  (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
     if (!(softmax_scale > 0.f)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: softmax_scale must be positive");
     const int cfg = g_attn_cfg;
+    if (N <= 128 && !scaled && cfg != 3) {
+        // K and V^T stay in registers; enough waves to fill the device, each walking over several query tiles
+        // (tiles per wave and batch: about 2048 waves in all, one 8-wave workgroup per CU)
+        const long q_tiles = (M + 31) / 32;
+        long tpw = (q_tiles * H + 2047) / 2048;
+        tpw = tpw < 1 ? 1 : (tpw > 16 ? 16 : tpw);
+        const unsigned gx = (unsigned)((q_tiles + 8 * tpw - 1) / (8 * tpw));
+        if (out_dtype == Q8_BF16)
+            hipLaunchKernelGGL((attn_short_kernel<Q8_BF16>), dim3(gx, (unsigned)H), dim3(512), 0, stream, p, (int)tpw);
+        else
+            hipLaunchKernelGGL((attn_short_kernel<Q8_E4M3>), dim3(gx, (unsigned)H), dim3(512), 0, stream, p, (int)tpw);
+        return launch_status("q8_attn_fwd");
+    }
 #define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV)                                                                         \
     hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
                                                                   (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
