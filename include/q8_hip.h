@@ -11,7 +11,8 @@
  *     default stream) and the call returns without synchronising;
  *   - the return value is Q8_OK (0) or a negative Q8_ERR_* code; on error no
  *     kernel has been launched; q8_last_error() returns a thread-local text;
- *   - no global mutable state: calls are re-entrant and thread-safe per stream.
+ *   - no global mutable state: calls are re-entrant and thread-safe per stream. (The error text, the last-kernel
+ *     record and the two *_set_config overrides for tests and tuning are per-thread.)
  *
  * Each entry point cites the interface of the reference implementation
  * (KONAKONA666/q8_kernels, paths relative to its root) that it replaces.
@@ -242,10 +243,10 @@ int q8_gemm_residual(const void* A, const void* B, const float* bias, const floa
 
 /*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with
- * one tile per workgroup, 2 = 128x128 tiles, 3 = plain 256x256 tiles, 4 = persistent pipelined 256x256 tiles (bf16
- * output, N % 8 == 0, K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's
- * tile to 192 / 256 rows / back to automatic. Process-wide; meant for tests and tuning, it has no counterpart in the reference
- * (whose tile is fixed at 128x128x64, csrc/gemm/fp8_matmul_bias.cu:426-429).
+ * one tile per workgroup, 2 = 128x128 tiles, 4 = persistent pipelined 256x256 tiles (bf16 or e4m3 output, N % 8 == 0,
+ * K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's tile to 192 / 256 rows /
+ * back to automatic. It holds for the calling thread only; meant for tests and tuning, it has no counterpart in the
+ * reference (whose tile is fixed at 128x128x64, csrc/gemm/fp8_matmul_bias.cu:426-429).
  */
 int q8_gemm_set_config(int cfg);
 
@@ -258,7 +259,6 @@ int q8_gemm_set_config(int cfg);
 enum {
     Q8_GEMM_KERNEL_PIPE256 = 1,    /* pipelined 256x256 tiles, one tile per workgroup */
     Q8_GEMM_KERNEL_TILE128 = 2,    /* 128x128 tiles                                    */
-    Q8_GEMM_KERNEL_PLAIN256 = 3,   /* plain 256x256 tiles                              */
     Q8_GEMM_KERNEL_PERSIST256 = 4, /* persistent, 256-row tiles                        */
     Q8_GEMM_KERNEL_PERSIST192 = 5, /* persistent, 192-row tiles                        */
     Q8_GEMM_KERNEL_RESIDUAL = 16
@@ -295,7 +295,8 @@ int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int3
 
 /*
  * Workgroup-shape override for q8_attn_fwd: 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries,
- * 2 = 4 waves x 32 queries. Process-wide; meant for tests and tuning, no counterpart in the reference (whose
+ * 2 = 4 waves x 32 queries, 3 = as 0 without the register-resident kernel that otherwise takes N <= 128 with unit
+ * scales. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
  * workgroup is fixed at 4 warps x 16 queries, csrc/flash_attention/flash_attention_cuda.cu:279-287).
  */
 int q8_attn_set_config(int cfg);

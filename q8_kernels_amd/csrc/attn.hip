@@ -1,7 +1,8 @@
 // FP8 FlashAttention-2 forward for gfx950, head dim 64, non-causal, optional per-batch KV length.
 //
-// One workgroup = 4 waves = 4 x 64 query rows of one (batch, head); KV is walked forward in tiles of
-// 64 keys that all four waves share through LDS (two stages, filled by global_load_lds_dwordx4).
+// One workgroup = 8 waves x 32 query rows of one (batch, head) (4 x 64 and 4 x 32 are instantiated as well); KV is
+// walked forward in tiles of 64 keys that all waves share through a four-stage LDS ring filled by
+// global_load_lds_dwordx4. Key / value sequences of at most 128 tokens with unit scales take attn_short_kernel instead.
 //
 // Everything is computed transposed so that no operand ever passes through LDS or a cross-lane
 // shuffle between the two matrix products:
@@ -481,7 +482,7 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
 
 using namespace q8;
 
-static int g_attn_cfg = 0;  // 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries,
+static thread_local int g_attn_cfg = 0;  // per thread: 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries,
                             // 3 = as 0 and without the register-resident path for N <= 128
 
 extern "C" int q8_attn_set_config(int cfg) {

@@ -174,7 +174,7 @@ static int reserve_lds(const void* kern, int bytes, int& done_dev) {
 
 template <class C, int OUT, bool GELU>
 static int launch_gemm(const GemmParams& p, hipStream_t stream) {
-    g_last_kernel = (C::BM == 256) ? Q8_GEMM_KERNEL_PLAIN256 : Q8_GEMM_KERNEL_TILE128;
+    g_last_kernel = Q8_GEMM_KERNEL_TILE128;
     const int tiles_m = (p.M + C::BM - 1) / C::BM, tiles_n = (p.N + C::BN - 1) / C::BN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     auto kern = gemm_kernel<C, OUT, GELU>;
@@ -184,15 +184,14 @@ static int launch_gemm(const GemmParams& p, hipStream_t stream) {
     return launch_status("q8_gemm");
 }
 
-// Tile selection: 256x256 (8 waves of 128x64) for large problems, 128x128 (4 waves of 64x64) when the
-// large tile would leave most of the 256 CUs idle.
-template <int IN>
-using CfgBig = GemmCfg<IN, 2, 4, 8, 4>;
+// Tile selection: pipelined 256x256 tiles (gemm_pipe.h / gemm_persist.h) for large problems, this file's 128x128 tiles
+// (4 waves of 64x64) when the large tile would leave most of the 256 CUs idle.
 template <int IN>
 using CfgSmall = GemmCfg<IN, 2, 2, 4, 4>;
 
-static int g_force_cfg = 0;  // 0 = auto, 1 = pipelined 256x256 (one tile per workgroup), 2 = 128x128, 3 = plain 256x256,
-                             // 4 = persistent pipelined 256x256 where eligible (see q8_gemm_set_config)
+// per-thread override (q8_gemm_set_config): 0 = auto, 1 = pipelined 256x256 (one tile per workgroup), 2 = 128x128,
+// 4 = persistent pipelined 256x256 where eligible
+static thread_local int g_force_cfg = 0;
 
 template <int IN, int OUT, bool GELU>
 static int launch_pipe(const GemmParams& p, hipStream_t stream) {
@@ -246,7 +245,7 @@ static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     return launch_status("q8_gemm");
 }
 
-static int g_persist_mt = 0;  // 0 = choose, 3 / 4 = forced tile height 192 / 256 (tuning)
+static thread_local int g_persist_mt = 0;  // 0 = choose, 3 / 4 = forced tile height 192 / 256 (tuning, per thread)
 
 template <int IN, bool GELU, bool E4M3OUT = false>
 static int launch_persist(const GemmParams& p, hipStream_t stream) {
@@ -277,7 +276,6 @@ static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
         if (big && g_force_cfg != 1 && persist_eligible(p)) return launch_persist<IN, GELU, OUT == Q8_E4M3>(p, stream);
     }
     if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
-    if (g_force_cfg == 3) return launch_gemm<CfgBig<IN>, OUT, GELU>(p, stream);
     return launch_gemm<CfgSmall<IN>, OUT, GELU>(p, stream);
 }
 
@@ -309,7 +307,7 @@ extern "C" int q8_gemm_last_kernel(void) { return g_last_kernel; }
 
 extern "C" int q8_gemm_set_config(int cfg) {
     if (cfg == 43 || cfg == 44 || cfg == 40) { g_persist_mt = cfg - 40; return Q8_OK; }  // tuning: persistent tile height
-    if (cfg < 0 || cfg > 4) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 4 || cfg == 3) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
     g_force_cfg = cfg;
     return Q8_OK;
 }

@@ -176,7 +176,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
     }
     auto read_half = [&](PipeFragsT<MT>& f, int stage, int s) {
         const unsigned so = (stage & 1) * kPipeStageBytes;
-        pipe_read_frags<0, MT>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+        pipe_read_frags<MT>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
     };
 
     using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;

@@ -38,29 +38,21 @@ using PipeFrags = PipeFragsT<4>;
 
 // a0/a1 (b0/b1): byte address of the lane's low/high 16-byte chunk in row (lane % 32) of the wave's first A (B)
 // tile; the following 32-row tiles are 4096 bytes apart.
-template <int SKIP = 0, int MT = 4>  // SKIP (tuning builds): 1 = leave the B fragments, 2 = leave the A fragments as they are
+template <int MT = 4>
 __device__ __forceinline__ void pipe_read_frags(PipeFragsT<MT>& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
-    if constexpr (SKIP != 1) {
-        f.b[0][0] = lds_read_b128<0>(b0);
-        f.b[0][1] = lds_read_b128<0>(b1);
-    }
-    if constexpr (SKIP != 2) {
-        f.a[0][0] = lds_read_b128<0>(a0);
-        f.a[0][1] = lds_read_b128<0>(a1);
-    }
-    if constexpr (SKIP != 1) {
-        f.b[1][0] = lds_read_b128<4096>(b0);
-        f.b[1][1] = lds_read_b128<4096>(b1);
-    }
-    if constexpr (SKIP != 2) {
-        f.a[1][0] = lds_read_b128<4096>(a0);
-        f.a[1][1] = lds_read_b128<4096>(a1);
-        f.a[2][0] = lds_read_b128<8192>(a0);
-        f.a[2][1] = lds_read_b128<8192>(a1);
-        if constexpr (MT == 4) {
-            f.a[3][0] = lds_read_b128<12288>(a0);
-            f.a[3][1] = lds_read_b128<12288>(a1);
-        }
+    f.b[0][0] = lds_read_b128<0>(b0);
+    f.b[0][1] = lds_read_b128<0>(b1);
+    f.a[0][0] = lds_read_b128<0>(a0);
+    f.a[0][1] = lds_read_b128<0>(a1);
+    f.b[1][0] = lds_read_b128<4096>(b0);
+    f.b[1][1] = lds_read_b128<4096>(b1);
+    f.a[1][0] = lds_read_b128<4096>(a0);
+    f.a[1][1] = lds_read_b128<4096>(a1);
+    f.a[2][0] = lds_read_b128<8192>(a0);
+    f.a[2][1] = lds_read_b128<8192>(a1);
+    if constexpr (MT == 4) {
+        f.a[3][0] = lds_read_b128<12288>(a0);
+        f.a[3][1] = lds_read_b128<12288>(a1);
     }
 }
 
@@ -123,9 +115,7 @@ __device__ __forceinline__ void pipe_mfma(const PipeFragsT<MT>& f, ACC (&acc)[MT
     }
 }
 
-// DBG (tuning builds only): bit 0 = no HBM->LDS loads, 1 = no LDS reads, 2 = no MFMA, 3 = no stores, 4 = no barrier,
-// 6 = no vmcnt wait, 7 = no B fragment reads, 8 = no A fragment reads in the loop
-template <int IN, int OUT, bool GELU, int DBG = 0>
+template <int IN, int OUT, bool GELU>
 __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     constexpr int BM = kPipeBM, BN = kPipeBN;
@@ -165,7 +155,6 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     }
     const int KT = (K + 127) >> 7;
     auto issue_load = [&](int stage, int i) {  // copy instruction i (0..7) of this wave for `stage`
-        if constexpr (DBG & 1) return;
         uint8_t* base = lds + (stage & 1) * kPipeStageBytes;
         const int k0 = stage << 7;
         const int q = (i < 4 ? 0 : 32) + wave + 8 * (i & 3);
@@ -191,10 +180,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
         pc[s][1] = pc[s][0] ^ 16;
     }
     auto read_half = [&](PipeFrags& f, int stage, int s) {
-        if constexpr (DBG & 2) return;
         const unsigned so = (stage & 1) * kPipeStageBytes;
-        pipe_read_frags<(DBG & 128) ? 1 : ((DBG & 256) ? 2 : 0)>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0],
-                                                                   b_row + so + pc[s][1]);
+        pipe_read_frags(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
     };
 
     using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
@@ -232,20 +219,8 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     PipeFrags f0, f1;
     issue_loads(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_barrier();
     issue_loads(1);
-    if constexpr (DBG & 2) {  // fragments of stage 0 are read once and reused for every stage
-        pipe_read_frags(f0, a_row + pc[0][0], a_row + pc[0][1], b_row + pc[0][0], b_row + pc[0][1]);
-        pipe_read_frags(f1, a_row + pc[1][0], a_row + pc[1][1], b_row + pc[1][0], b_row + pc[1][1]);
-        pipe_wait_frags(f0);
-        pipe_wait_frags(f1);
-    }
-    if constexpr ((DBG & (128 | 256)) != 0) {  // the fragments that the loop leaves alone get real data once
-        pipe_read_frags(f0, a_row + pc[0][0], a_row + pc[0][1], b_row + pc[0][0], b_row + pc[0][1]);
-        pipe_read_frags(f1, a_row + pc[1][0], a_row + pc[1][1], b_row + pc[1][0], b_row + pc[1][1]);
-        pipe_wait_frags(f0);
-        pipe_wait_frags(f1);
-    }
     read_half(f0, 0, 0);
 
     for (int k = 0; k < KT; ++k) {
@@ -255,39 +230,27 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
         pipe_pin(f0);
         // First half. Once the second half of stage k is in registers everywhere (barrier 1, after the 4th MFMA
         // tile), buffer k & 1 is free and the copies of stage k+2 start to trickle out, one per MFMA tile.
-        if constexpr (!(DBG & 4)) {
-            pipe_mfma<IN, 4>(f0, acc, [&](int j) {
-                if (j == 3) {
-                    pipe_wait_frags(f1);
-                    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
-                }
-                if (j >= 4) issue_load(k + 2, j - 4);
-            });
-        } else {
-            pipe_wait_frags(f1);
-            if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
-            issue_loads(k + 2);
-        }
+        pipe_mfma<IN, 4>(f0, acc, [&](int j) {
+            if (j == 3) {
+                pipe_wait_frags(f1);
+                __builtin_amdgcn_s_barrier();
+            }
+            if (j >= 4) issue_load(k + 2, j - 4);
+        });
         __builtin_amdgcn_sched_barrier(0);
         pipe_pin(f1);
         // Second half. After the last copy of stage k+2 is out, everything older (stage k+1) must have landed
         // (vmcnt counts in order); barrier 2 makes that true for every wave's copies, and the first half of
         // stage k+1 is fetched under the remaining MFMA tiles. A copy has between 1 and 1.5 stages of MFMA
         // time to land.
-        if constexpr (!(DBG & 4)) {
-            pipe_mfma<IN, 4>(f1, acc, [&](int j) {
-                if (j < 4) issue_load(k + 2, 4 + j);
-                if (j == 4) {
-                    if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-                    if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
-                    read_half(f0, k + 1, 0);
-                }
-            });
-        } else {
-            if constexpr (!(DBG & 64)) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-            if constexpr (!(DBG & 16)) __builtin_amdgcn_s_barrier();
-            read_half(f0, k + 1, 0);
-        }
+        pipe_mfma<IN, 4>(f1, acc, [&](int j) {
+            if (j < 4) issue_load(k + 2, 4 + j);
+            if (j == 4) {
+                asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                read_half(f0, k + 1, 0);
+            }
+        });
         __builtin_amdgcn_sched_barrier(0);
     }
     // drain: the look-ahead loads and fragment reads past the last stage target LDS / registers that nobody uses
@@ -302,7 +265,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
     // Interior tiles with bf16 output go through LDS: every wave lays its 128 x 64 results out as 128 rows of 128
     // bytes (16-byte chunks swizzled by (row >> 1) & 7, conflict-free both ways) and then writes 8 full rows of 128
     // contiguous bytes per instruction, i.e. whole cache lines instead of 32-byte pieces.
-    const bool staged = (OUT == Q8_BF16) && !(DBG & 8) && (m0 + BM <= M) && (n0 + BN <= N) && ((N & 7) == 0);
+    const bool staged = (OUT == Q8_BF16) && (m0 + BM <= M) && (n0 + BN <= N) && ((N & 7) == 0);
     uint8_t* stage_out = lds + wave * 16384;
     if (staged) __builtin_amdgcn_s_barrier();  // every wave has finished reading the operand stages
 #pragma unroll
@@ -342,8 +305,7 @@ __global__ __launch_bounds__(512) void gemm_pipe_kernel(const GemmParams p) {
                         continue;
                     }
                 }
-                if constexpr (DBG & 8) { if (a8[0] == (elem_t)12345.678f) finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv); }
-                else finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv);
+                finish8<OUT, GELU>(p, zc, sam, m, n, a8, sbv, bv);
             }
         }
     }

@@ -298,3 +298,32 @@ def test_zero_query_row_with_scales_and_masked_keys(dev, attn_cfg):
     _check(got, q, k, v, 0.125, lens, (sq, sk, sv), what="zero query rows")
     mean_v = (v[1, 1, :37].double() * sv[1, 1, :37, None].double()).mean(dim=0)
     assert (got[1, 1, 64:].cpu().double() - mean_v).abs().max() <= 0.07 * mean_v.abs().max() + 0.02
+
+
+@pytest.mark.parametrize("n,lens", [(128, [128, 16]), (100, [37, 100]), (64, [64, 1]), (17, [0, 17]), (1, [1, 1])])
+def test_register_resident_path_for_short_kv(dev, n, lens):
+    """N <= 128 with unit scales takes the kernel that keeps K and V^T in registers (single-pass softmax, no LDS). Same
+    bars as the general kernel, which is forced for comparison (config 3): both against the oracle, and against each
+    other within twice the rounding bound (they round P against different maxima)."""
+    from q8_kernels_amd import _lib
+    b, h, m = 2, 3, 1000
+    q, k, v = _inputs(7000 + n, b, h, m, n)
+    l = torch.tensor(lens, dtype=torch.int32)
+    args = (q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, l.to(dev))
+    short = _C().flash_attention(*args, out_dtype=torch.bfloat16)
+    try:
+        _lib.check(_lib.lib().q8_attn_set_config(3))
+        general = _C().flash_attention(*args, out_dtype=torch.bfloat16)
+    finally:
+        _lib.check(_lib.lib().q8_attn_set_config(0))
+    _check(short, q, k, v, 0.125, l, what="register-resident N=%d" % n)
+    _check(general, q, k, v, 0.125, l, what="general N=%d" % n)
+    assert not torch.equal(short, general) or n <= 64, "both calls took the same kernel"
+    # token-major output, e4m3 output and the reference's P grid through the same path
+    tok = _C().flash_attention(*args, out_dtype=torch.bfloat16, token_major_out=True)
+    assert_equal = torch.equal(tok.view(b, m, h, 64).transpose(1, 2), short)
+    assert assert_equal, "token-major output differs"
+    o8 = _C().flash_attention(*args)
+    assert o8.dtype == E4M3 and ((o8.cpu().float() - short.cpu().float()).abs() <= 0.07 * short.cpu().float().abs() + 0.02).all()
+    unit = _C().flash_attention(*args, out_dtype=torch.bfloat16, p_unit_range=True)
+    _check(unit, q, k, v, 0.125, l, what="register-resident, p <= 1", p_scale=1.0)
