@@ -116,37 +116,54 @@ def _cpu_blas_gemm(x, w, bias):
             "what": "fp32 torch.matmul on dequantised e4m3 codes + bias + tanh-GELU -> bf16, full size; not the oracle"}
 
 
-def _extras(dev, steps, warmup):
+def _attn_inputs(dev, g, B=2, H=32, S=6144):
     from q8_kernels_amd import _C
-    from q8_kernels_amd.blocks import Fp8DiTBlock
-    out = {}
-    g = torch.Generator().manual_seed(1)
-    # fp8 self-attention with Hadamard, per-token e4m3 (config 3) and reference-style direct casts
-    B, H, S = 2, 32, 6144
     q, k, v = (torch.randn(B, H, S, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
     qr, kr = _C.fast_hadamard_transform(q, 0.125, torch.bfloat16), _C.fast_hadamard_transform(k, 0.125, torch.bfloat16)
     (q8, sq), (k8, sk), (v8, sv) = _C.tokenwise_quant(qr, E4M3), _C.tokenwise_quant(kr, E4M3), _C.tokenwise_quant(v, E4M3)
     vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
-    flop = 4.0 * B * H * S * S * 64
-    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk,
-                                            v_scales=sv), steps, warmup)
-    out["attn_self_fp8_per_token_scales"] = {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS,
-                                             "shape": "B2 H32 S6144 D64"}
     s = (1 / 64) ** 0.5 * (0.125 ** 0.5)
     qd, kd = _C.fast_hadamard_transform(q, s, E4M3), _C.fast_hadamard_transform(k, s, E4M3)
+    return {"scaled": (q8, k8, vt, sq, sk, sv), "direct": (qd, kd, vt), "fold": s}
+
+
+def _extras_attn(dev, steps, warmup, g, out):
+    """fp8 self-attention with Hadamard at S = 6144: per-token e4m3 (config 3) and reference-style direct casts; the
+    cross-attention with a padding mask (config 4). Each entry carries the quantities a roofline needs: flop, the number
+    of exponentials (one per score; the kernel is bound by them), average launch time."""
+    from q8_kernels_amd import _C
+    B, H, S = 2, 32, 6144
+    a = _attn_inputs(dev, g, B, H, S)
+    q8, k8, vt, sq, sk, sv = a["scaled"]
+    qd, kd, _ = a["direct"]
+    flop = 4.0 * B * H * S * S * 64
+
+    def entry(t, kernel):
+        return {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS, "shape": "B2 H32 S6144 D64",
+                "roofline": {"bound": "mfma", "achieved": flop / t / 1e12, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": flop / t / 1e12 / FP8_PEAK_TFLOPS, "kernel": kernel, "flop_per_launch": flop,
+                             "exp2_per_launch": float(B * H) * S * S, "avg_launch_us": t * 1e6}}
+
+    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk,
+                                            v_scales=sv), steps, warmup)
+    out["attn_self_fp8_per_token_scales"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 8 waves x 32 queries>")
     t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16), steps, warmup)
-    out["attn_self_fp8_reference_casts"] = {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS,
-                                            "shape": "B2 H32 S6144 D64"}
+    out["attn_self_fp8_reference_casts"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>")
     # cross-attention with a padding mask (config 4): HBM-bound
     N = 128
     kx, vx = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
     lens = torch.randint(16, 129, (B,), generator=g, dtype=torch.int32).to(dev)
-    kx8 = _C.fast_hadamard_transform(kx, s, E4M3)
+    kx8 = _C.fast_hadamard_transform(kx, a["fold"], E4M3)
     vxt = vx.to(E4M3).view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
     t, _ = _time(lambda: _C.flash_attention(qd, kx8, vxt, 1.0, lens, out_dtype=torch.bfloat16), steps, warmup)
     byts = B * H * (S * 64 + 2 * N * 64 + S * 64 * 2)
     out["attn_cross_fp8_masked"] = {"ms": t * 1e3, "gbs": byts / t / 1e9, "frac_of_hbm_peak": byts / t / 1e9 / HBM_PEAK_GBS,
-                                    "tflops": 4.0 * B * H * S * N * 64 / t / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64"}
+                                    "tflops": 4.0 * B * H * S * N * 64 / t / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64",
+                                    "valid_lengths": lens.tolist(), "kernel": "attn_short_kernel<bf16>"}
+
+
+def _extras_gemm(dev, steps, warmup, g, out):
+    from q8_kernels_amd import _C
     # int8 GEMM (config 2)
     a = torch.randint(-127, 128, (6144, 2048), generator=g, dtype=torch.int8).to(dev)
     b = torch.randint(-127, 128, (2048, 2048), generator=g, dtype=torch.int8).to(dev)
@@ -168,6 +185,10 @@ def _extras(dev, steps, warmup):
             t, _ = _time(lambda: _C.q8_mm_bias(ai, bi, gb, gsx, gsw, False, None), steps, warmup)
             out["int8_gemm_%dx%dx%d_e4m3_out" % (mm, nn, kk)] = {"ms": t * 1e3, "tops": 2.0 * mm * nn * kk / t / 1e12}
         del gxq, gwq
+
+
+def _extras_rows(dev, steps, warmup, g, out):
+    from q8_kernels_amd import _C
     # row kernels on [12288, 2048] tokens
     x = torch.randn(12288, 2048, generator=g).to(torch.bfloat16).to(dev)
     n = x.numel()
@@ -188,11 +209,22 @@ def _extras(dev, steps, warmup):
                           ("attn_prep_v_fp8", lambda: _C.attn_prep_v(xs, 32), 3)):
         t, _ = _time(fn, steps, warmup)
         out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    del x, cos, sin
+    # the Hadamard rotation + int8 quantizer over the 8192-wide FFN hidden of the int8 block
+    xw = torch.randn(12288, 8192, generator=g).to(torch.bfloat16).to(dev)
+    t, _ = _time(lambda: _C.fht_quant(xw, 8192 ** -0.5, None), steps, warmup)
+    out["fht_quant_int8_fused_12288x8192"] = {"ms": t * 1e3, "gbs": xw.numel() * 3 / t / 1e9, "frac_of_hbm_peak": xw.numel() * 3 / t / 1e9 / HBM_PEAK_GBS}
+
+
+def _extras_blocks(dev, steps, warmup, g, out):
+    from q8_kernels_amd import _C
+    from q8_kernels_amd.blocks import Fp8DiTBlock
+    from q8_kernels_amd.functional.rope import precompute_freqs_cis, video_index_grid
     # the DiT block (config 5)
     blk = Fp8DiTBlock(device=dev).init_random()
     hidden = torch.randn(2, 6144, 2048, generator=g).to(torch.bfloat16).to(dev)
     text = torch.randn(2, 128, 2048, generator=g).to(torch.bfloat16).to(dev)
-    from q8_kernels_amd.functional.rope import precompute_freqs_cis, video_index_grid
+    lens = torch.randint(16, 129, (2,), generator=g, dtype=torch.int32).to(dev)
     cosf, sinf = precompute_freqs_cis(video_index_grid(16, 16, 24, batch=2, device=dev), 2048)
     with torch.no_grad():
         t, _ = _time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
@@ -214,6 +246,18 @@ def _extras(dev, steps, warmup):
                      max(3, steps // 4), max(1, warmup // 2))
     out["ltx_transformer_block_int8"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12,
                                          "shape": "tokens [2,6144,2048], text [2,128,2048], int8 linears, fp8 attention"}
+
+
+EXTRA_GROUPS = {"attn": _extras_attn, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks}
+
+
+def _extras(dev, steps, warmup, only=None):
+    """The other workloads of the metric. `only` (group names out of attn, gemm, rows, blocks) restricts the run to those
+    groups, e.g. for a counter-collection run of one kernel."""
+    out = {}
+    for name, fn in EXTRA_GROUPS.items():
+        if only is None or name in only:
+            fn(dev, steps, warmup, torch.Generator().manual_seed(1 + sorted(EXTRA_GROUPS).index(name)), out)
     return out
 
 
@@ -223,6 +267,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--only", default=None, help="comma-separated groups of the other workloads to run (attn, gemm, rows, blocks)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 512 MiB (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -279,11 +324,15 @@ def main():
     else:
         result["cpu_baseline"] = None
     if not args.no_extras:
-        result["extras"] = _extras(dev, args.steps, args.warmup)
-        a = result["extras"]["attn_self_fp8_per_token_scales"]
-        result["attn_tflops"] = a["tflops"]
-        result["attn_frac_of_fp8_peak"] = a["frac_of_fp8_peak"]
-        result["block_ms"] = result["extras"]["dit_block"]["ms"]
+        only = None if args.only is None else set(args.only.split(","))
+        result["extras"] = _extras(dev, args.steps, args.warmup, only)
+        a = result["extras"].get("attn_self_fp8_per_token_scales")
+        if a is not None:
+            result["attn_tflops"] = a["tflops"]
+            result["attn_frac_of_fp8_peak"] = a["frac_of_fp8_peak"]
+            result["attn_roofline"] = result["extras"]["attn_self_fp8_reference_casts"]["roofline"]
+        if "dit_block" in result["extras"]:
+            result["block_ms"] = result["extras"]["dit_block"]["ms"]
         if not args.no_cpu:
             result["extras"]["cpu_fp32_blas_linear_gelu"] = _cpu_blas_gemm(x, w, bias)
     print(json.dumps(result))

@@ -19,30 +19,20 @@ __global__ __launch_bounds__(kBlock) void fht_quant_kernel(const void* __restric
     constexpr int RPB = kBlock / LANES;
     constexpr int IN_B = (IN == Q8_E4M3) ? 1 : 2;
     __shared__ float red[4];
-    const int t = threadIdx.x % LANES;
+    const int t = row_thread<LANES>();
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
     const bool row_ok = row < rows;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPB <= rows;
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
 
     float v[CH][8];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<IN>(xr, e, v[c]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
-        }
-    }
-    fht_row<LANES, CH>(v, t);
+    load_row<IN, LANES, CH>(xr, t, row_ok, dim, full, v);
+    fht_row<LANES, CH>(v, t, fht_scale);
 
     float amax[1] = {0.f};
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int e = (c * LANES + t) * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[c][i] *= fht_scale;
         round_mid8<MID>(v[c]);
         if (e < dim) {  // outputs beyond dim are dropped
 #pragma unroll
@@ -74,19 +64,11 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
     const int t = threadIdx.x % LANES;
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
     const bool row_ok = row < rows;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPB <= rows;
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
 
     float v[CH][8];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<IN>(xr, e, v[c]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
-        }
-    }
+    load_row<IN, LANES, CH>(xr, t, row_ok, dim, full, v);
     float ss[1] = {0.f};
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -144,22 +126,14 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
                                                                     int flags) {
     constexpr int RPB = kBlock / LANES;
     __shared__ float red[4];
-    const int t = threadIdx.x % LANES;
+    const int t = row_thread<LANES>();
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
     const bool row_ok = row < rows;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPB <= rows;
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * 2;
 
     float v[CH][8];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<Q8_BF16>(xr, e, v[c]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
-        }
-    }
+    load_row<Q8_BF16, LANES, CH>(xr, t, row_ok, dim, full, v);
     if (apply_norm) {
         float ss[1] = {0.f};
 #pragma unroll
@@ -199,13 +173,9 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
         }
     }
     if (apply_fht) {
-        fht_row<LANES, CH>(v, t);
+        fht_row<LANES, CH>(v, t, fht_scale);
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] *= fht_scale;
-            round_mid8<Q8_BF16>(v[c]);
-        }
+        for (int c = 0; c < CH; ++c) round_mid8<Q8_BF16>(v[c]);
     }
     float amax[1] = {0.f};
 #pragma unroll
@@ -247,7 +217,7 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
                                                               int mid_bf16) {
     static_assert(LH <= LANES, "a head may not span tokens");
     constexpr int DIM = LANES * CH * 8, D = LH * 8, H = DIM / D, NT = PAIR ? 2 : 1;
-    const int t = threadIdx.x % LANES;
+    const int t = row_thread<LANES>();
     const int64_t tok = (int64_t)blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES;
     if (tok >= tokens) return;  // no barrier below; the lane exchanges stay inside a head, i.e. inside a token
     const int64_t b = tok / S, s = tok - b * S;
@@ -310,23 +280,7 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             if (apply_fht) {
-#pragma unroll
-                for (int st = 1; st < 8; st <<= 1) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        if ((i & st) == 0) {
-                            const float a0 = v[n][c][i], b0 = v[n][c][i + st];
-                            v[n][c][i] = a0 + b0;
-                            v[n][c][i + st] = a0 - b0;
-                        }
-                    }
-                }
-                fht_lane_stage<1>(v[n][c], (unsigned)(t & 1) << 31);
-                fht_lane_stage<2>(v[n][c], (unsigned)(t & 2) << 30);
-                fht_lane_stage<4>(v[n][c], 0u);
-                if constexpr (LH > 8) fht_lane_stage<8>(v[n][c], 0u);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[n][c][i] *= scale;
+                fht_head<LH>(v[n][c], t, scale);
             }
             const int h = (c * LANES + t) / LH;
             const int64_t orow = (b * H + h) * S + s;

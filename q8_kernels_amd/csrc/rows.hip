@@ -14,6 +14,7 @@ __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const void* __restri
     constexpr int ESZ = (IN == Q8_F32 ? 4 : (IN == Q8_E4M3 ? 1 : 2));
     __shared__ float red[RPT * 4];
     const int t = threadIdx.x % LANES;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPT * RPB <= rows;
     int64_t row[RPT];
     bool row_ok[RPT];
     float v[RPT][CH][8];
@@ -23,16 +24,7 @@ __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const void* __restri
         row[r] = ((int64_t)blockIdx.x * RPT + r) * RPB + threadIdx.x / LANES;
         row_ok[r] = row[r] < rows;
         const char* xr = reinterpret_cast<const char*>(x) + row[r] * x_row_stride * ESZ;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int e = (c * LANES + t) * 8;
-            if (row_ok[r] && e < dim) {
-                load8<IN>(xr, e, v[r][c]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[r][c][i] = 0.f;
-            }
-        }
+        load_row<IN, LANES, CH>(xr, t, row_ok[r], dim, full, v[r]);
     }
 #pragma unroll
     for (int r = 0; r < RPT; ++r) {
@@ -66,24 +58,16 @@ __global__ __launch_bounds__(kBlock) void fht_kernel(const void* __restrict__ x,
     constexpr int RPB = kBlock / LANES;
     constexpr int IN_B = (IN == Q8_E4M3) ? 1 : 2;
     constexpr int OUT_B = (OUT == Q8_E4M3) ? 1 : 2;
-    const int t = threadIdx.x % LANES;
+    const int t = row_thread<LANES>();
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LANES;
     const bool row_ok = row < rows;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPB <= rows;
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
 
     float v[CH][8];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (row_ok && e < dim) {
-            load8<IN>(xr, e, v[c]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
-        }
-    }
+    load_row<IN, LANES, CH>(xr, t, row_ok, dim, full, v);
 
-    fht_row<LANES, CH>(v, t);
+    fht_row<LANES, CH>(v, t, scale);
 
     if (!row_ok) return;
     char* yr = reinterpret_cast<char*>(y) + row * (int64_t)dim * OUT_B;
@@ -91,8 +75,6 @@ __global__ __launch_bounds__(kBlock) void fht_kernel(const void* __restrict__ x,
     for (int c = 0; c < CH; ++c) {
         const int e = (c * LANES + t) * 8;
         if (e >= dim) continue;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[c][i] *= scale;
         store8<OUT>(yr, e, v[c]);
     }
 }
@@ -108,6 +90,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const void* __restrict_
     constexpr int OUT_B = (OUT == Q8_E4M3) ? 1 : 2;
     __shared__ float red[RPT * 4];
     const int t = threadIdx.x % LANES;
+    const bool full = dim == 8 * LANES * CH && ((int64_t)blockIdx.x + 1) * RPT * RPB <= rows;
     int64_t row[RPT];
     bool row_ok[RPT];
     float v[RPT][CH][8];
@@ -117,16 +100,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const void* __restrict_
         row[r] = ((int64_t)blockIdx.x * RPT + r) * RPB + threadIdx.x / LANES;
         row_ok[r] = row[r] < rows;
         const char* xr = reinterpret_cast<const char*>(x) + row[r] * (int64_t)dim * IN_B;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int e = (c * LANES + t) * 8;
-            if (row_ok[r] && e < dim) {
-                load8<IN>(xr, e, v[r][c]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[r][c][i] = 0.f;
-            }
-        }
+        load_row<IN, LANES, CH>(xr, t, row_ok[r], dim, full, v[r]);
     }
 #pragma unroll
     for (int r = 0; r < RPT; ++r) {

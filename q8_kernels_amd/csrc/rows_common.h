@@ -57,161 +57,184 @@ __device__ __forceinline__ void row_reduce(float (&v)[RPT], float* red) {
 template <int LANES, int CH>
 struct RowsPerThread { static constexpr int value = (CH == 1) ? 4 : (CH == 2 ? 2 : 1); };
 
-// ---- Hadamard butterfly stages ------------------------------------------------------------------
+// ---- loading a row ----------------------------------------------------------------------------------
 
-// One butterfly stage across lanes l and l ^ MASK: y[l] = x[l] + x[l ^ MASK] in the lane with the bit clear,
-// x[l ^ MASK] - x[l] in the lane with the bit set (the same two roundings as the sequential butterfly).
-//
-// MASK 1, 2: the own value gets its sign flipped where the bit is set (one xor), then one add whose first
-//            operand comes through a DPP quad permutation.
-// MASK 4, 8: the lanes with the bit clear and the lanes with the bit set are whole DPP banks, so an add and a
-//            subtract with complementary bank masks do the stage in two instructions.
-// MASK 16, 32: two registers a, b at a time: a lane-half swap brings (a[l], a[l ^ MASK]) of the lower halves
-//            and (b[l], b[l ^ MASK]) of the upper halves into the same lanes, sum and difference are formed
-//            there, and a second swap puts them back. Four instructions per two values, no selects.
-template <int MASK>
-__device__ __forceinline__ void fht_lane_stage(float (&v)[8], unsigned sign_if_set) {
-    if constexpr (MASK == 1 || MASK == 2) {
+// v[c] = the 8 elements (c * LANES + t) * 8 + 0..7 of the row at xr as fp32, zeros beyond dim or when the row does
+// not exist. `full` (uniform over the block: every row of the block exists and dim == 8 * LANES * CH) selects a
+// branch-free path on which all CH loads of a thread are issued back to back; the guarded path waits for each
+// load inside its own branch.
+template <int IN, int LANES, int CH>
+__device__ __forceinline__ void load_row(const void* xr, int t, bool row_ok, int dim, bool full, float (&v)[CH][8]) {
+    if (full) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float own = __uint_as_float(__float_as_uint(v[i]) ^ sign_if_set);
-            const int o = __builtin_amdgcn_mov_dpp(__float_as_int(v[i]), MASK == 1 ? 0xB1 : 0x4E, 0xf, 0xf, true);
-            v[i] = __int_as_float(o) + own;
-        }
-    } else if constexpr (MASK == 4) {
-        float y[8];
-        // 2 wait states between a VALU write of a VGPR and a DPP read of it
-        asm volatile(
-            "s_nop 1\n"
-            "v_add_f32_dpp %0, %8, %8 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %1, %9, %9 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %2, %10, %10 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %3, %11, %11 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %4, %12, %12 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %5, %13, %13 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %6, %14, %14 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_add_f32_dpp %7, %15, %15 row_shl:4 row_mask:0xf bank_mask:0x5\n"
-            "v_sub_f32_dpp %0, %8, %8 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %1, %9, %9 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %2, %10, %10 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %3, %11, %11 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %4, %12, %12 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %5, %13, %13 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %6, %14, %14 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            "v_sub_f32_dpp %7, %15, %15 row_shr:4 row_mask:0xf bank_mask:0xa\n"
-            : "=&v"(y[0]), "=&v"(y[1]), "=&v"(y[2]), "=&v"(y[3]), "=&v"(y[4]), "=&v"(y[5]), "=&v"(y[6]), "=&v"(y[7])
-            : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]));
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = y[i];
-    } else if constexpr (MASK == 8) {
-        float y[8];
-        asm volatile(
-            "s_nop 1\n"
-            "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0x3\n"
-            "v_sub_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            "v_sub_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n"
-            : "=&v"(y[0]), "=&v"(y[1]), "=&v"(y[2]), "=&v"(y[3]), "=&v"(y[4]), "=&v"(y[5]), "=&v"(y[6]), "=&v"(y[7])
-            : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]));
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = y[i];
+        for (int c = 0; c < CH; ++c) load8<IN>(xr, (c * LANES + t) * 8, v[c]);
     } else {
-        static_assert(MASK == 16 || MASK == 32, "fht_lane_stage: mask must be 1..32");
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-            const unsigned a = __float_as_uint(v[i]), b = __float_as_uint(v[i + 1]);
-            // r[0] = a in the lanes with the bit clear, b[l ^ MASK] in the others; r[1] = a[l ^ MASK] | b
-            const auto r = (MASK == 16) ? __builtin_amdgcn_permlane16_swap(a, b, false, false)
-                                        : __builtin_amdgcn_permlane32_swap(a, b, false, false);
-            const float lo = __uint_as_float(r[0]), hi = __uint_as_float(r[1]);
-            const float sum = lo + hi, dif = lo - hi;
-            const auto w = (MASK == 16)
-                               ? __builtin_amdgcn_permlane16_swap(__float_as_uint(sum), __float_as_uint(dif), false, false)
-                               : __builtin_amdgcn_permlane32_swap(__float_as_uint(sum), __float_as_uint(dif), false, false);
-            v[i] = __uint_as_float(w[0]);
-            v[i + 1] = __uint_as_float(w[1]);
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (row_ok && e < dim) {
+                load8<IN>(xr, e, v[c]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+            }
         }
     }
 }
 
+// ---- Hadamard butterfly stages ------------------------------------------------------------------
+//
+// A butterfly stage over lane bit k replaces x by x + x[partner] in the thread whose element bit is clear and by
+// x[partner] - x in the thread whose bit is set. Here every such stage is ONE fused multiply-add per value,
+//     x <- x + s * x[partner],   s = +1 (bit clear) or -1 (bit set), a per-thread constant,
+// which is the exact sum (one rounding, like the addition) in the first kind of thread and the exact NEGATIVE of
+// the wanted difference in the second. The sign is not repaired stage by stage: negation commutes with every
+// later addition and rounding, so a thread simply carries all of its values with the sign
+// (-1)^popcount(thread bits processed), and the multiplication by the transform's scale that ends every
+// transform here takes that sign along (fht_row's last step). The only trace is the sign of exact zeros, which
+// that last step fixes to +0. The sequential network returns a zero other than +0 only when every input of the
+// transform is a zero (x + y = -0 needs x = y = -0 and x - y = -0 needs x = -0, y = +0, so a -0 has only zeros
+// beneath it): rows of zeros are detected before the transform and take the plain form of every stage
+// (fht_*_exact: partner + (own with its sign flipped where the bit is set), the reference's own additions), so
+// the signs of their zeros are the reference's too.
+//
+// The partner value arrives through the DPP operand of the multiply-add for thread bits 0..3 and through the
+// LDS crossbar (ds_swizzle / ds_bpermute, no LDS memory) for bits 4 and 5. DPP has no "lane ^ 4" or "lane ^ 8"
+// pattern but it has mirrors: row_half_mirror pairs lane l with l ^ 7 and row_mirror with l ^ 15. The threads of
+// a row therefore own the 16-byte chunks of 16 lanes in a permuted order (row_thread): chunk bits
+// (e0, e1, e2, e3) = (l0 ^ l2, l1 ^ l2, l2 ^ l3, l3) of lane bits l0..l3, under which flipping l0 flips e0 only,
+// l1 -> e1, half mirror -> e2 only and full mirror -> e3 only. 16 lanes still read and write the same 256
+// contiguous bytes; reductions over the lanes of a row pair the same elements as without the permutation.
 
-// All butterfly stages of one row held in registers as v[CH][8] (thread t of the row, element index
-// (c * LANES + t) * 8 + i): registers, lanes, waves (one exchange through LDS), chunks, in this order.
-template <int LANES, int CH>
-__device__ __forceinline__ void fht_row(float (&v)[CH][8], int t) {
-    // element bits 0..2: inside the 8 registers of a chunk
+// position of this thread among the LANES threads of its row (the "t" of the row mapping)
+template <int LANES>
+__device__ __forceinline__ int row_thread() {
+    const int l = threadIdx.x, p = l & 15;
+    const int e = p ^ (((p >> 2) & 1) * 3) ^ (((p >> 3) & 1) << 2);
+    return ((l & ~15) | e) & (LANES - 1);
+}
+
+// +1.0f or -1.0f: the factor s of the stage over thread bit `bit`
+__device__ __forceinline__ float fht_stage_sign(int t, int bit) {
+    return __uint_as_float(0x3f800000u | ((unsigned)((t >> bit) & 1) << 31));
+}
+
+#define Q8_FHT_DPP8(CTRL)                                                                                        \
+    asm volatile("s_nop 1\n" /* 2 wait states between a VALU write of a VGPR and a DPP read of it */             \
+                 "v_fmac_f32_dpp %0, %0, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %1, %1, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %2, %2, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %3, %3, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %4, %4, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %5, %5, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %6, %6, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 "v_fmac_f32_dpp %7, %7, %8 " CTRL " row_mask:0xf bank_mask:0xf\n"                               \
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]) \
+                 : "v"(s))
+
+// one stage over thread bit log2(MASK) for the 8 values of a chunk; s = fht_stage_sign of that bit
+template <int MASK>
+__device__ __forceinline__ void fht_lane_stage(float (&v)[8], float s) {
+    if constexpr (MASK == 1) {
+        Q8_FHT_DPP8("quad_perm:[1,0,3,2]");
+    } else if constexpr (MASK == 2) {
+        Q8_FHT_DPP8("quad_perm:[2,3,0,1]");
+    } else if constexpr (MASK == 4) {
+        Q8_FHT_DPP8("row_half_mirror");
+    } else if constexpr (MASK == 8) {
+        Q8_FHT_DPP8("row_mirror");
+    } else {
+        static_assert(MASK == 16 || MASK == 32, "fht_lane_stage: mask must be 1..32");
+        int p[8];
+        if constexpr (MASK == 16) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
+            for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_ds_swizzle(__float_as_int(v[i]), 0x401F);  // lane ^ 16
+        } else {
+            const int peer = (int)((threadIdx.x & 63) ^ 32) * 4;
 #pragma unroll
-        for (int s = 1; s < 8; s <<= 1) {
+            for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_ds_bpermute(peer, __float_as_int(v[i]));
+        }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if ((i & s) == 0) {
-                    const float a = v[c][i], b = v[c][i + s];
-                    v[c][i] = a + b;
-                    v[c][i + s] = a - b;
-                }
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(__int_as_float(p[i]), s, v[i]);
+    }
+}
+
+// the register stages (element bits 0..2) of one chunk
+__device__ __forceinline__ void fht_chunk_stages(float (&v)[8]) {
+#pragma unroll
+    for (int s = 1; s < 8; s <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if ((i & s) == 0) {
+                const float a = v[i], b = v[i + s];
+                v[i] = a + b;
+                v[i + s] = a - b;
             }
         }
     }
-    // lane bits
+}
+
+// True when some group of LANES threads handled by this wave (LANES <= 64; a group of inactive lanes counts) or
+// some wave of this block (LANES > 64, with a barrier: uniform over the block) holds only zeros in v.
+template <int LANES, int NV>
+__device__ __forceinline__ bool fht_zero_group(const float (&v)[NV]) {
+    unsigned acc = 0;
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if constexpr (LANES > 1) fht_lane_stage<1>(v[c], (unsigned)(t & 1) << 31);
-        if constexpr (LANES > 2) fht_lane_stage<2>(v[c], (unsigned)(t & 2) << 30);
-        if constexpr (LANES > 4) fht_lane_stage<4>(v[c], 0u);
-        if constexpr (LANES > 8) fht_lane_stage<8>(v[c], 0u);
-        if constexpr (LANES > 16) fht_lane_stage<16>(v[c], 0u);
-        if constexpr (LANES > 32) fht_lane_stage<32>(v[c], 0u);
-    }
-    // wave bits: one exchange through LDS per chunk, both stages evaluated from the 2 or 4 wave values
+    for (int i = 0; i < NV; ++i) acc |= __float_as_uint(v[i]);
+    unsigned long long m = __ballot((acc & 0x7fffffffu) != 0);
     if constexpr (LANES > 64) {
-        __shared__ v4f xch[2][kBlock];
-        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-        const unsigned m1 = (unsigned)(wave & 1) << 31, m2 = (unsigned)(wave & 2) << 30;
-        auto flip = [](float x, unsigned m) { return __uint_as_float(__float_as_uint(x) ^ m); };
+        return __syncthreads_or(m == 0) != 0;
+    } else if constexpr (LANES == 64) {
+        return m == 0;
+    } else {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            xch[0][threadIdx.x] = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
-            xch[1][threadIdx.x] = v4f{v[c][4], v[c][5], v[c][6], v[c][7]};
-            __syncthreads();
-            auto peer = [&](int w, float (&o)[8]) {
-                const v4f a = xch[0][w * 64 + lane], b = xch[1][w * 64 + lane];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
-            };
-            float p1[8];
-            peer(wave ^ 1, p1);
-            if constexpr (LANES == 128) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[c][i] = p1[i] + flip(v[c][i], m1);
-            } else {
-                float p2[8], p3[8];
-                peer(wave ^ 2, p2);
-                peer(wave ^ 3, p3);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float ya = p1[i] + flip(v[c][i], m1);
-                    const float yb = p3[i] + flip(p2[i], m1);
-                    v[c][i] = yb + flip(ya, m2);
-                }
-            }
-            __syncthreads();
-        }
+        for (int s = 1; s < LANES; s <<= 1) m |= m >> s;  // bit g * LANES = "group g has a non-zero"
+        constexpr unsigned long long low = LANES == 1 ? ~0ull : LANES == 2 ? 0x5555555555555555ull
+                                         : LANES == 4 ? 0x1111111111111111ull : LANES == 8 ? 0x0101010101010101ull
+                                         : LANES == 16 ? 0x0001000100010001ull : 0x0000000100000001ull;
+        return (~m & low) != 0;
     }
-    // chunk bits
+}
+
+// plain form of the stage over thread bit BIT: y = x[partner] + (bit set ? -x : x)
+template <int BIT>
+__device__ __forceinline__ void fht_lane_stage_exact(float (&v)[8], int t) {
+    constexpr int pm = BIT == 0 ? 1 : BIT == 1 ? 2 : BIT == 2 ? 7 : BIT == 3 ? 15 : BIT == 4 ? 16 : 32;
+    const int peer = (int)((threadIdx.x & 63) ^ pm) * 4;
+    const unsigned m = (unsigned)((t >> BIT) & 1) << 31;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float p = __int_as_float(__builtin_amdgcn_ds_bpermute(peer, __float_as_int(v[i])));
+        v[i] = p + __uint_as_float(__float_as_uint(v[i]) ^ m);
+    }
+}
+
+// D-point transform of the 8 * LH elements of a head held by LH threads (t = row_thread), times scale
+template <int LH>
+__device__ __forceinline__ void fht_head(float (&v)[8], int t, float scale) {
+    const bool zeros = fht_zero_group<LH, 8>(v);
+    fht_chunk_stages(v);
+    if (zeros) {
+        if constexpr (LH > 1) fht_lane_stage_exact<0>(v, t);
+        if constexpr (LH > 2) fht_lane_stage_exact<1>(v, t);
+        if constexpr (LH > 4) fht_lane_stage_exact<2>(v, t);
+        if constexpr (LH > 8) fht_lane_stage_exact<3>(v, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] *= scale;
+    } else {
+        if constexpr (LH > 1) fht_lane_stage<1>(v, fht_stage_sign(t, 0));
+        if constexpr (LH > 2) fht_lane_stage<2>(v, fht_stage_sign(t, 1));
+        if constexpr (LH > 4) fht_lane_stage<4>(v, fht_stage_sign(t, 2));
+        if constexpr (LH > 8) fht_lane_stage<8>(v, fht_stage_sign(t, 3));
+        const float ss = (__builtin_popcount(t & (LH - 1)) & 1) ? -scale : scale;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(v[i], ss, 0.f);
+    }
+}
+
+// the chunk stages (element bits above the thread bits)
+template <int CH>
+__device__ __forceinline__ void fht_upper_stages(float (&v)[CH][8]) {
 #pragma unroll
     for (int s = 1; s < CH; s <<= 1) {
 #pragma unroll
@@ -226,6 +249,102 @@ __device__ __forceinline__ void fht_row(float (&v)[CH][8], int t) {
             }
         }
     }
+}
+
+// the stages over the wave bits of the thread index (LANES = 128, 256): one exchange through LDS per chunk, both
+// stages evaluated from the 2 or 4 wave values. FMA: the one-instruction form with the carried sign.
+template <int LANES, int CH, bool FMA>
+__device__ __forceinline__ void fht_wave_stages(float (&v)[CH][8], int t) {
+    __shared__ v4f xch[2][kBlock];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const float s6 = fht_stage_sign(t, 6), s7 = fht_stage_sign(t, 7);
+    // y = b + (a with the sign of s): a + b or b - a
+    auto stage = [](float a, float s, float b) {
+        if constexpr (FMA) return __builtin_fmaf(b, s, a);  // a + s b
+        else return b + __uint_as_float(__float_as_uint(a) ^ (__float_as_uint(s) & 0x80000000u));
+    };
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        xch[0][threadIdx.x] = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
+        xch[1][threadIdx.x] = v4f{v[c][4], v[c][5], v[c][6], v[c][7]};
+        __syncthreads();
+        auto peer = [&](int w, float (&o)[8]) {
+            const v4f a = xch[0][w * 64 + lane], b = xch[1][w * 64 + lane];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
+        };
+        float p1[8];
+        peer(wave ^ 1, p1);
+        if constexpr (LANES == 128) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] = stage(v[c][i], s6, p1[i]);
+        } else {
+            float p2[8], p3[8];
+            peer(wave ^ 2, p2);
+            peer(wave ^ 3, p3);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float ya = stage(v[c][i], s6, p1[i]);  // this wave's value after the first stage
+                const float yb = stage(p2[i], s6, p3[i]);    // wave ^ 2's
+                v[c][i] = stage(ya, s7, yb);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// All butterfly stages of one row held in registers as v[CH][8] (thread t = row_thread<LANES>() of the row,
+// element index (c * LANES + t) * 8 + i): registers, lanes, waves, chunks, in this order, then the
+// multiplication by `scale`. Contains barriers when LANES > 64: every thread of the block must call it.
+template <int LANES, int CH>
+__device__ __forceinline__ void fht_row(float (&v)[CH][8], int t, float scale) {
+    const bool zeros = fht_zero_group<LANES, CH * 8>(reinterpret_cast<const float (&)[CH * 8]>(v));
+#pragma unroll
+    for (int c = 0; c < CH; ++c) fht_chunk_stages(v[c]);
+    if (zeros) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if constexpr (LANES > 1) fht_lane_stage_exact<0>(v[c], t);
+            if constexpr (LANES > 2) fht_lane_stage_exact<1>(v[c], t);
+            if constexpr (LANES > 4) fht_lane_stage_exact<2>(v[c], t);
+            if constexpr (LANES > 8) fht_lane_stage_exact<3>(v[c], t);
+            if constexpr (LANES > 16) fht_lane_stage_exact<4>(v[c], t);
+            if constexpr (LANES > 32) fht_lane_stage_exact<5>(v[c], t);
+        }
+        if constexpr (LANES > 64) fht_wave_stages<LANES, CH, false>(v, t);
+        fht_upper_stages<CH>(v);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[c][i] *= scale;
+        return;
+    }
+    const float s0 = fht_stage_sign(t, 0), s1 = fht_stage_sign(t, 1), s2 = fht_stage_sign(t, 2),
+                s3 = fht_stage_sign(t, 3), s4 = fht_stage_sign(t, 4), s5 = fht_stage_sign(t, 5);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if constexpr (LANES > 1) fht_lane_stage<1>(v[c], s0);
+        if constexpr (LANES > 2) fht_lane_stage<2>(v[c], s1);
+        if constexpr (LANES > 4) fht_lane_stage<4>(v[c], s2);
+        if constexpr (LANES > 8) fht_lane_stage<8>(v[c], s3);
+    }
+    // the two stages through the LDS crossbar, all chunks of a stage together so that many exchanges are in flight
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if constexpr (LANES > 16) fht_lane_stage<16>(v[c], s4);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if constexpr (LANES > 32) fht_lane_stage<32>(v[c], s5);
+    }
+    if constexpr (LANES > 64) fht_wave_stages<LANES, CH, true>(v, t);
+    fht_upper_stages<CH>(v);
+    // scale, the carried sign, and +0 for exact zeros (a product of -0 plus +0 is +0)
+    const float ss = (__builtin_popcount(t) & 1) ? -scale : scale;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[c][i] = __builtin_fmaf(v[c][i], ss, 0.f);
 }
 
 // ---- 8-element chunks with a run-time element type (uniform switch) ------------------------------------
@@ -289,12 +408,13 @@ __device__ __forceinline__ v2i quant_codes8(const float (&v)[8], float ratio, in
         // fp32 |q| < 2^22 (the sum rounds up to the next integer exactly for the ties and for nothing below them);
         // round half even = v_rndne. Two saturating 32->16 packs and one byte permute gather the 4 codes of a word.
         int qi[8];
+        if (flags & Q8_QUANT_RNE) {  // uniform
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float q = v[i] * ratio;
-            if (flags & Q8_QUANT_RNE) {
-                qi[i] = (int)rintf(q);
-            } else {
+            for (int i = 0; i < 8; ++i) qi[i] = (int)rintf(v[i] * ratio);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float q = v[i] * ratio;
                 const float half = __uint_as_float(0x3effffffu | (__float_as_uint(q) & 0x80000000u));
                 qi[i] = (int)(q + half);  // the conversion truncates
             }

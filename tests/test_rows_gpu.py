@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import q8_oracle as O
-from tests.util import E4M3, assert_bit_equal, bf16_ulp
+from tests.util import E4M3, assert_bit_equal, bf16_ulp, bits
 
 pytestmark = pytest.mark.gpu
 
@@ -140,6 +140,32 @@ def test_fht_fp8_input_and_head_dim_rows(dev):
     for scale in (0.125 * 0.125 ** 0.5, 40.0):
         got = _C().fast_hadamard_transform(q.to(dev), scale, E4M3)
         assert_bit_equal(got, O.ref_fht(q, scale, E4M3), "fht D=64 scale=%g" % scale)
+
+
+@pytest.mark.parametrize("dim", [8, 16, 64, 128, 512, 2048, 4096, 8192, 16384, 32768, 1536])
+def test_fht_signed_zeros_and_exact_cancellations(dev, dim):
+    """Rows of zeros of both signs keep the signs the sequential network gives them (a sum of -0 and -0 is -0),
+    rows with one or two non-zero entries produce exact cancellations (+0), and zero rows sit among non-zero rows
+    of the same wave and block."""
+    g = torch.Generator().manual_seed(1000 + dim)
+    rows = 13 if dim >= 8192 else 70
+    x = torch.randn(rows, dim, generator=g).to(torch.bfloat16)
+    neg_zero = torch.tensor(-0.0, dtype=torch.bfloat16)
+    x[1] = 0.0
+    x[2] = neg_zero
+    x[3] = torch.where(torch.rand(dim, generator=g) < 0.5, neg_zero, torch.tensor(0.0, dtype=torch.bfloat16))
+    x[4] = neg_zero
+    x[4, 0] = 0.0
+    x[5] = 0.0
+    x[5, dim // 2] = 1.5          # one non-zero: every output is +-1.5 * scale
+    x[6] = neg_zero
+    x[6, 1], x[6, dim - 1] = 2.0, 2.0   # half of the outputs cancel exactly
+    x[rows - 1] = torch.where(torch.rand(dim, generator=g) < 0.3, neg_zero, torch.tensor(0.0, dtype=torch.bfloat16))
+    for out_type in (torch.bfloat16, E4M3):
+        got = _C().fast_hadamard_transform(x.to(dev), dim ** -0.5, out_type)
+        want = O.ref_fht(x, dim ** -0.5, out_type)
+        assert (bits(want[2]) != bits(want[1])).any(), "the case needs negative zeros among the wanted outputs"
+        assert_bit_equal(got, want, "fht signed zeros dim=%d -> %s" % (dim, out_type))
 
 
 def test_fht_full_size_and_involution(dev):
