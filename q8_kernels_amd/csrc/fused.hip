@@ -26,8 +26,8 @@ __global__ __launch_bounds__(kBlock) void fht_quant_kernel(const void* __restric
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
 
     float v[CH][8];
-    load_row<IN, LANES, CH>(xr, t, row_ok, dim, full, v);
-    fht_row<LANES, CH>(v, t, fht_scale);
+    const bool nz = load_row<IN, LANES, CH, true>(xr, t, row_ok, dim, full, v);
+    fht_row<LANES, CH>(v, t, fht_scale, fht_zero_group<LANES>(nz));
 
     float amax[1] = {0.f};
 #pragma unroll
@@ -44,11 +44,7 @@ __global__ __launch_bounds__(kBlock) void fht_quant_kernel(const void* __restric
     const float ratio = quant_ratio<OUT>(amax[0]);
     if (t == 0) scales[row] = quant_scale<OUT>(amax[0], ratio, flags);
     uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
-    }
+    store_codes_row<OUT, LANES, CH>(out, t, dim, full, v, ratio, flags);
 }
 
 // ---- RMSNorm -> quantizer ----------------------------------------------------------------------------
@@ -103,11 +99,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(const void* __res
         if (rstd_out != nullptr) rstd_out[row] = rstd;
     }
     uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
-    }
+    store_codes_row<OUT, LANES, CH>(out, t, dim, full, v, ratio, flags);
 }
 
 // ---- RMSNorm -> AdaLN modulation -> FHT -> quantizer ---------------------------------------------------------
@@ -173,7 +165,8 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
         }
     }
     if (apply_fht) {
-        fht_row<LANES, CH>(v, t, fht_scale);
+        const bool nz = any_nonzero(reinterpret_cast<const float (&)[CH * 8]>(v));
+        fht_row<LANES, CH>(v, t, fht_scale, fht_zero_group<LANES>(nz));
 #pragma unroll
         for (int c = 0; c < CH; ++c) round_mid8<Q8_BF16>(v[c]);
     }
@@ -191,11 +184,7 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
     const float ratio = quant_ratio<OUT>(amax[0]);
     if (t == 0) scales[row] = quant_scale<OUT>(amax[0], ratio, flags);
     uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row * (int64_t)dim;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int e = (c * LANES + t) * 8;
-        if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
-    }
+    store_codes_row<OUT, LANES, CH>(out, t, dim, full, v, ratio, flags);
 }
 
 // ---- attention prologue for Q and K ---------------------------------------------------------------------

@@ -182,6 +182,31 @@ __device__ __forceinline__ void load8(const void* p, int64_t e, float (&v)[8]) {
     }
 }
 
+// The same, and the OR of the raw words read is accumulated into raw_or (BF16, E4M3): all of the 8 elements are
+// zeros of either sign exactly when (raw_or & sign_clear_mask<DT>()) == 0.
+template <int DT>
+__device__ __forceinline__ void load8(const void* p, int64_t e, float (&v)[8], unsigned& raw_or) {
+    if constexpr (DT == Q8_BF16) {
+        v4u w = *reinterpret_cast<const v4u*>(reinterpret_cast<const uint16_t*>(p) + e);
+        raw_or |= (w[0] | w[1]) | (w[2] | w[3]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = bf16_bits_to_f32(w[i] & 0xffffu);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    } else {
+        static_assert(DT == Q8_E4M3, "load8 with raw_or: unsupported element type");
+        v2i w = *reinterpret_cast<const v2i*>(reinterpret_cast<const uint8_t*>(p) + e);
+        raw_or |= (unsigned)(w[0] | w[1]);
+        v[0] = e4m3_to_f32<0>(w[0]); v[1] = e4m3_to_f32<1>(w[0]);
+        v[2] = e4m3_to_f32<2>(w[0]); v[3] = e4m3_to_f32<3>(w[0]);
+        v[4] = e4m3_to_f32<0>(w[1]); v[5] = e4m3_to_f32<1>(w[1]);
+        v[6] = e4m3_to_f32<2>(w[1]); v[7] = e4m3_to_f32<3>(w[1]);
+    }
+}
+template <int DT>
+__device__ __forceinline__ constexpr unsigned sign_clear_mask() { return DT == Q8_BF16 ? 0x7fff7fffu : 0x7f7f7f7fu; }
+
 // Store 8 fp32 values as `DT` (BF16: RNE; E4M3: c10 cast) at element index `e`.
 template <int DT>
 __device__ __forceinline__ void store8(void* p, int64_t e, const float (&v)[8]) {

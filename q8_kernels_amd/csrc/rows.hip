@@ -42,11 +42,7 @@ __global__ __launch_bounds__(kBlock) void quant_rows_kernel(const void* __restri
         const float ratio = quant_ratio<OUT>(amax[r]);
         if (t == 0) scales[row[r]] = quant_scale<OUT>(amax[r], ratio, flags);
         uint8_t* out = reinterpret_cast<uint8_t*>(codes) + row[r] * (int64_t)dim;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int e = (c * LANES + t) * 8;
-            if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[r][c], ratio, flags);
-        }
+        store_codes_row<OUT, LANES, CH>(out, t, dim, full, v[r], ratio, flags);
     }
 }
 
@@ -65,9 +61,8 @@ __global__ __launch_bounds__(kBlock) void fht_kernel(const void* __restrict__ x,
     const char* xr = reinterpret_cast<const char*>(x) + row * (int64_t)dim * IN_B;
 
     float v[CH][8];
-    load_row<IN, LANES, CH>(xr, t, row_ok, dim, full, v);
-
-    fht_row<LANES, CH>(v, t, scale);
+    const bool nz = load_row<IN, LANES, CH, true>(xr, t, row_ok, dim, full, v);
+    fht_row<LANES, CH>(v, t, scale, fht_zero_group<LANES>(nz));
 
     if (!row_ok) return;
     char* yr = reinterpret_cast<char*>(y) + row * (int64_t)dim * OUT_B;

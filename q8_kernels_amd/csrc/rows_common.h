@@ -62,24 +62,30 @@ struct RowsPerThread { static constexpr int value = (CH == 1) ? 4 : (CH == 2 ? 2
 // v[c] = the 8 elements (c * LANES + t) * 8 + 0..7 of the row at xr as fp32, zeros beyond dim or when the row does
 // not exist. `full` (uniform over the block: every row of the block exists and dim == 8 * LANES * CH) selects a
 // branch-free path on which all CH loads of a thread are issued back to back; the guarded path waits for each
-// load inside its own branch.
-template <int IN, int LANES, int CH>
-__device__ __forceinline__ void load_row(const void* xr, int t, bool row_ok, int dim, bool full, float (&v)[CH][8]) {
+// load inside its own branch. NZ: also returns whether this thread read anything but zeros (of either sign).
+template <int IN, int LANES, int CH, bool NZ = false>
+__device__ __forceinline__ bool load_row(const void* xr, int t, bool row_ok, int dim, bool full, float (&v)[CH][8]) {
+    unsigned raw_or = 0;
+    auto ld = [&](int e, float (&o)[8]) {
+        if constexpr (NZ) load8<IN>(xr, e, o, raw_or); else load8<IN>(xr, e, o);
+    };
     if (full) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) load8<IN>(xr, (c * LANES + t) * 8, v[c]);
+        for (int c = 0; c < CH; ++c) ld((c * LANES + t) * 8, v[c]);
     } else {
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int e = (c * LANES + t) * 8;
             if (row_ok && e < dim) {
-                load8<IN>(xr, e, v[c]);
+                ld(e, v[c]);
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
             }
         }
     }
+    if constexpr (NZ) return (raw_or & sign_clear_mask<IN>()) != 0;
+    else return true;
 }
 
 // ---- Hadamard butterfly stages ------------------------------------------------------------------
@@ -174,16 +180,27 @@ __device__ __forceinline__ void fht_chunk_stages(float (&v)[8]) {
     }
 }
 
-// True when some group of LANES threads handled by this wave (LANES <= 64; a group of inactive lanes counts) or
-// some wave of this block (LANES > 64, with a barrier: uniform over the block) holds only zeros in v.
-template <int LANES, int NV>
-__device__ __forceinline__ bool fht_zero_group(const float (&v)[NV]) {
+// whether any of the values is not a zero (of either sign)
+template <int NV>
+__device__ __forceinline__ bool any_nonzero(const float (&v)[NV]) {
     unsigned acc = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) acc |= __float_as_uint(v[i]);
-    unsigned long long m = __ballot((acc & 0x7fffffffu) != 0);
+    return (acc & 0x7fffffffu) != 0;
+}
+
+// nz: whether this thread holds a non-zero value. True when some group of LANES threads handled by this wave
+// (LANES <= 64; a group of inactive lanes counts) or some wave of this block (LANES > 64, with one barrier: every
+// thread of the block must call it, and the answer is uniform over the block) holds only zeros.
+template <int LANES>
+__device__ __forceinline__ bool fht_zero_group(bool nz) {
+    unsigned long long m = __ballot(nz);
     if constexpr (LANES > 64) {
-        return __syncthreads_or(m == 0) != 0;
+        __shared__ int wave_zero[kBlock / 64];
+        if ((threadIdx.x & 63) == 0) wave_zero[threadIdx.x >> 6] = (m == 0);
+        __syncthreads();
+        const v4i z = *reinterpret_cast<const v4i*>(wave_zero);
+        return ((z[0] | z[1]) | (z[2] | z[3])) != 0;
     } else if constexpr (LANES == 64) {
         return m == 0;
     } else {
@@ -212,7 +229,7 @@ __device__ __forceinline__ void fht_lane_stage_exact(float (&v)[8], int t) {
 // D-point transform of the 8 * LH elements of a head held by LH threads (t = row_thread), times scale
 template <int LH>
 __device__ __forceinline__ void fht_head(float (&v)[8], int t, float scale) {
-    const bool zeros = fht_zero_group<LH, 8>(v);
+    const bool zeros = fht_zero_group<LH>(any_nonzero(v));
     fht_chunk_stages(v);
     if (zeros) {
         if constexpr (LH > 1) fht_lane_stage_exact<0>(v, t);
@@ -251,11 +268,19 @@ __device__ __forceinline__ void fht_upper_stages(float (&v)[CH][8]) {
     }
 }
 
+// exchange buffer of the wave stages: two halves used by alternate chunks, each [2][kBlock] 16-byte slots
+__device__ __forceinline__ v4f* fht_exchange_buffer() {
+    __shared__ v4f xch[2 * 2 * kBlock];
+    return xch;
+}
+
 // the stages over the wave bits of the thread index (LANES = 128, 256): one exchange through LDS per chunk, both
-// stages evaluated from the 2 or 4 wave values. FMA: the one-instruction form with the carried sign.
+// stages evaluated from the 2 or 4 wave values. One barrier per chunk: chunk c + 1 writes the other half of the
+// buffer, and the half of chunk c is written again only behind the barrier of chunk c + 1, which no wave passes
+// before every wave has read chunk c. FMA: the one-instruction form with the carried sign.
 template <int LANES, int CH, bool FMA>
 __device__ __forceinline__ void fht_wave_stages(float (&v)[CH][8], int t) {
-    __shared__ v4f xch[2][kBlock];
+    v4f* const xch = fht_exchange_buffer();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const float s6 = fht_stage_sign(t, 6), s7 = fht_stage_sign(t, 7);
     // y = b + (a with the sign of s): a + b or b - a
@@ -265,11 +290,13 @@ __device__ __forceinline__ void fht_wave_stages(float (&v)[CH][8], int t) {
     };
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        xch[0][threadIdx.x] = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
-        xch[1][threadIdx.x] = v4f{v[c][4], v[c][5], v[c][6], v[c][7]};
+        v4f* const x0 = xch + (c & 1) * 2 * kBlock;
+        v4f* const x1 = x0 + kBlock;
+        x0[threadIdx.x] = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
+        x1[threadIdx.x] = v4f{v[c][4], v[c][5], v[c][6], v[c][7]};
         __syncthreads();
         auto peer = [&](int w, float (&o)[8]) {
-            const v4f a = xch[0][w * 64 + lane], b = xch[1][w * 64 + lane];
+            const v4f a = x0[w * 64 + lane], b = x1[w * 64 + lane];
 #pragma unroll
             for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
         };
@@ -289,16 +316,16 @@ __device__ __forceinline__ void fht_wave_stages(float (&v)[CH][8], int t) {
                 v[c][i] = stage(ya, s7, yb);
             }
         }
-        __syncthreads();
     }
+    __syncthreads();  // the buffer may be written again by a later call
 }
 
 // All butterfly stages of one row held in registers as v[CH][8] (thread t = row_thread<LANES>() of the row,
 // element index (c * LANES + t) * 8 + i): registers, lanes, waves, chunks, in this order, then the
-// multiplication by `scale`. Contains barriers when LANES > 64: every thread of the block must call it.
+// multiplication by `scale`. zeros = fht_zero_group<LANES>(...) of the values in v: selects the plain stage forms.
+// Contains barriers when LANES > 64: every thread of the block must call it.
 template <int LANES, int CH>
-__device__ __forceinline__ void fht_row(float (&v)[CH][8], int t, float scale) {
-    const bool zeros = fht_zero_group<LANES, CH * 8>(reinterpret_cast<const float (&)[CH * 8]>(v));
+__device__ __forceinline__ void fht_row(float (&v)[CH][8], int t, float scale, bool zeros) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) fht_chunk_stages(v[c]);
     if (zeros) {
@@ -439,6 +466,23 @@ __device__ __forceinline__ v2i quant_codes8(const float (&v)[8], float ratio, in
         w[1] = (int)p1;
     }
     return w;
+}
+
+// the codes of a row to out (the row's first byte); full: as in load_row, no guards
+template <int OUT, int LANES, int CH>
+__device__ __forceinline__ void store_codes_row(uint8_t* out, int t, int dim, bool full, const float (&v)[CH][8],
+                                                float ratio, int flags) {
+    if (full) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            *reinterpret_cast<v2i*>(out + (c * LANES + t) * 8) = quant_codes8<OUT>(v[c], ratio, flags);
+    } else {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int e = (c * LANES + t) * 8;
+            if (e < dim) *reinterpret_cast<v2i*>(out + e) = quant_codes8<OUT>(v[c], ratio, flags);
+        }
+    }
 }
 
 // ---- dispatch ------------------------------------------------------------------------------------
