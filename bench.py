@@ -149,6 +149,9 @@ def _extras_attn(dev, steps, warmup, g, out):
     out["attn_self_fp8_per_token_scales"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 8 waves x 32 queries>")
     t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16), steps, warmup)
     out["attn_self_fp8_reference_casts"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>")
+    v_tok = vt.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)  # [B,H,S,64]: V as the fused prologue leaves it
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, v_tok, 1.0, None, out_dtype=torch.bfloat16, v_token_major=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_token_major_v"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, token-major V>")
     # cross-attention with a padding mask (config 4): HBM-bound
     N = 128
     kx, vx = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
@@ -206,7 +209,9 @@ def _extras_rows(dev, steps, warmup, g, out):
     for name, fn, bpe in (("fht_quant_int8_fused", lambda: _C.fht_quant(x, 2048 ** -0.5, None), 3),
                           ("rmsnorm_quant_fp8_fused", lambda: _C.rms_norm_quant(x, w, E4M3), 3),
                           ("attn_prep_qk_rope_fht_fp8", lambda: _C.attn_prep_qk(xs, 32, cs3, sn3, True, 0.125), 11),
-                          ("attn_prep_v_fp8", lambda: _C.attn_prep_v(xs, 32), 3)):
+                          ("attn_prep_v_fp8", lambda: _C.attn_prep_v(xs, 32), 3),
+                          # Q, K, V of a self-attention in one pass: 3 x 2 B in, 8 B of tables (read once), 3 x 1 B out
+                          ("attn_prep_qkv_rope_fht_fp8", lambda: _C.attn_prep_qkv(xs, xs, xs, 32, cs3, sn3, True, 0.125), 17)):
         t, _ = _time(fn, steps, warmup)
         out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
     del x, cos, sin

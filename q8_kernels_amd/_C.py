@@ -259,7 +259,8 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
                     batch_mask: Optional[torch.Tensor] = None, *, out_dtype: Optional[torch.dtype] = None,
                     q_scales: Optional[torch.Tensor] = None, k_scales: Optional[torch.Tensor] = None,
                     v_scales: Optional[torch.Tensor] = None, sum_rounded_p: bool = False,
-                    p_unit_range: bool = False, token_major_out: bool = False) -> torch.Tensor:
+                    p_unit_range: bool = False, token_major_out: bool = False,
+                    v_token_major: bool = False) -> torch.Tensor:
     """csrc/flash_attention/flash_attention.cpp:18-48.
 
     q [B,H,M,64], k [B,H,N,64], v [B,H,64,Nv] (pre-transposed, Nv >= N, Nv % 16 == 0), all e4m3 and contiguous;
@@ -267,7 +268,8 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
     The keyword arguments are extensions: bf16 output, per-token dequantisation scales
     (q_scales [B,H,M], k_scales / v_scales [B,H,N], fp32), and p_unit_range=True to round the probabilities
     on the reference's grid (p <= 1) instead of the default 2^8 p, which does not flush small weights;
-    token_major_out=True returns [B,M,H*64], the transpose(1, 2).reshape the callers apply next.
+    token_major_out=True returns [B,M,H*64], the transpose(1, 2).reshape the callers apply next;
+    v_token_major=True takes v as [B,H,N,64] (k's layout): the kernel turns the tiles itself, no transposed copy.
     """
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
         _check_input(t, name)
@@ -277,7 +279,10 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
     n = k.shape[2]
     if k.shape[0] != bs or k.shape[1] != heads or k.shape[3] != d:
         raise RuntimeError("flash_attention: k shape mismatch")
-    if v.shape[0] != bs or v.shape[1] != heads or v.shape[2] != d or v.shape[3] < n:
+    if v_token_major:
+        if tuple(v.shape) != tuple(k.shape):
+            raise RuntimeError("flash_attention: a token-major v must have k's shape [B,H,N,D]")
+    elif v.shape[0] != bs or v.shape[1] != heads or v.shape[2] != d or v.shape[3] < n:
         raise RuntimeError("flash_attention: v must be [B,H,D,Nv] with Nv >= N")
     if batch_mask is not None:
         if batch_mask.dtype != torch.int32:
@@ -301,7 +306,8 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().q8_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(batch_mask),
                                           _ptr(q_scales), _ptr(k_scales), _ptr(v_scales), bs, heads, m, n, d,
-                                          _lib.Q8_V_DS, v.shape[3], float(softmax_scale), _DT[out_dtype],
+                                          _lib.Q8_V_SD if v_token_major else _lib.Q8_V_DS, v.shape[3],
+                                          float(softmax_scale), _DT[out_dtype],
                                           (_lib.Q8_ATTN_SUM_ROUNDED_P if sum_rounded_p else 0) |
                                           (_lib.Q8_ATTN_P_UNIT_RANGE if p_unit_range else 0) |
                                           (_lib.Q8_ATTN_O_TOKEN_MAJOR if token_major_out else 0), _stream(q)))
@@ -478,6 +484,37 @@ def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Opt
                                                    int(apply_fht), float(scale),
                                                    Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))
     return ((cq, sq), (ck, sk_)) if per_token_scales else (cq, ck)
+
+
+def attn_prep_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
+                  sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
+                  per_token_scales: bool = False, *, round_intermediate: bool = True,
+                  q_norm_weight: Optional[torch.Tensor] = None, k_norm_weight: Optional[torch.Tensor] = None):
+    """attn_prep_qk_pair, and the V projection of the same tokens is cast to e4m3 in the same pass, token-major per head
+    ([B, H, S, D], what flash_attention takes with v_token_major=True). Returns (q_out, k_out, v_out), each codes or
+    (codes, scales [B, H, S]) with per_token_scales."""
+    q, b, s, d = _token_major(q, num_heads, "attn_prep_qkv")
+    k, bk, sk, dk = _token_major(k, num_heads, "attn_prep_qkv")
+    v, bv, sv, dv = _token_major(v, num_heads, "attn_prep_qkv")
+    if (bk, sk, dk) != (b, s, d) or (bv, sv, dv) != (b, s, d):
+        raise RuntimeError("attn_prep_qkv: q, k and v must have the same shape")
+    if (cos is None) != (sin is None):
+        raise RuntimeError("attn_prep_qkv: cos and sin come together")
+    if cos is not None:
+        for t in (cos, sin):
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != q.numel():
+                raise RuntimeError("attn_prep_qkv: tables must be float32 CUDA tensors of q's shape")
+        cos, sin = cos.contiguous(), sin.contiguous()
+    mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=q.device)  # noqa: E731
+    mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=q.device) if per_token_scales else None  # noqa: E731
+    cq, ck, cv, sq, sk_, sv_ = mk(), mk(), mk(), mks(), mks(), mks()
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().q8_attn_prep_qkv(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), v.data_ptr(), v.stride(1),
+                                               _ptr(_norm_w(q_norm_weight, q)), _ptr(_norm_w(k_norm_weight, k)),
+                                               _ptr(cos), _ptr(sin), cq.data_ptr(), _ptr(sq), ck.data_ptr(), _ptr(sk_),
+                                               cv.data_ptr(), _ptr(sv_), b, s, num_heads, d, int(apply_fht), float(scale),
+                                               Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))
+    return ((cq, sq), (ck, sk_), (cv, sv_)) if per_token_scales else (cq, ck, cv)
 
 
 def attn_prep_v(x: torch.Tensor, num_heads: int, per_token_scales: bool = False):

@@ -3,6 +3,8 @@
 // One workgroup = 8 waves x 32 query rows of one (batch, head) (4 x 64 and 4 x 32 are instantiated as well); KV is
 // walked forward in tiles of 64 keys that all waves share through a four-stage LDS ring filled by
 // global_load_lds_dwordx4. Key / value sequences of at most 128 tokens with unit scales take attn_short_kernel instead.
+// V arrives either channel-major per head (V^T [B,H,64,Nv], Q8_V_DS) or token-major like K ([B,H,N,64], Q8_V_SD); the
+// token-major tile is turned while it is read from LDS (ds_read_b64_tr_b8), so no transposed copy of V exists in HBM.
 //
 // Everything is computed transposed so that no operand ever passes through LDS or a cross-lane
 // shuffle between the two matrix products:
@@ -34,7 +36,7 @@ struct AttnParams {
     const float* sk;
     const float* sv;
     int B, H, M, N;
-    int64_t v_row_stride;  // V^T row stride in bytes-elements (>= N, multiple of 16)
+    int64_t v_row_stride;  // V^T row stride in elements (>= N, multiple of 16); unused for token-major V
     float scale_log2;      // softmax_scale * log2(e)
     float p_shift;         // probabilities are formed as 2^(x - max + p_shift)
     int flags;
@@ -47,6 +49,16 @@ constexpr int kStage = 8192;    // K tile 4 KiB + V^T tile 4 KiB
 constexpr int kStages = 4;      // LDS ring: one tile being read, up to three in flight
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ds_read_b64_tr_b8: the 16 lanes of a group name an 8 x 16 byte matrix M (lane 2 r + c points at M[r][8 c .. 8 c + 7]) and
+// lane i of the group receives its column i, M[0..7][i]. Like lds_read_b128 the read is invisible to the compiler's
+// wait-count insertion: an s_waitcnt lgkmcnt that names the result must follow.
+template <int OFFSET>
+__device__ __forceinline__ v2i lds_read_tr_b64(unsigned addr) {
+    v2i r;
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET) : "memory");
+    return r;
+}
 
 // Output stage shared by the attention kernels. The O^T accumulators of a 32-query tile: lane (q, h), tile d, register e
 // holds dim 32 d + 8 (e / 4) + 4 h + (e % 4) of query q, i.e. the two lanes of a query hold alternate groups of 4 dims.
@@ -77,7 +89,8 @@ __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, con
 }
 
 // kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
-template <int OUT, bool SCALED, int kQT, int kWaves>
+// VTOK: V is token-major ([B,H,N,64])
+template <int OUT, bool SCALED, int kQT, int kWaves, bool VTOK = false>
 __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams p) {
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
@@ -94,7 +107,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     }
     const uint8_t* Qg = p.q + (size_t)bh * M * 64;
     const uint8_t* Kg = p.k + (size_t)bh * N * 64;
-    const uint8_t* Vg = p.v + (size_t)bh * 64 * p.v_row_stride;
+    const uint8_t* Vg = p.v + (size_t)bh * 64 * (VTOK ? (size_t)N : (size_t)p.v_row_stride);
     const int q0 = blockIdx.x * kBlockQ + wave * (kQT * 32);
     // output row r of this (batch, head): element offset o_base + r * o_rs
     const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
@@ -123,6 +136,9 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     const bool copy_k = (kWaves == 4) || wave < 4, copy_v = (kWaves == 4) || wave >= 4;
     const int crow = 16 * cw + (lane >> 2);
     const int cchunk = (lane & 3) ^ ((crow >> 2) & 3);
+    // token-major V tile: LDS row = key of the tile, physical chunk = logical chunk ^ (2 * ((row >> 2) & 1)), which keeps
+    // the 8 rows x 16 bytes that a 16-lane group of the transposing read touches on distinct banks
+    const int vchunk = (lane & 3) ^ (((crow >> 2) & 1) << 1);
     int k_src_row;  // key index inside the tile held by LDS row `crow`
     {
         const int t = crow >> 5, i = crow & 31;
@@ -140,8 +156,15 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         if (copy_k)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
                                              (__attribute__((address_space(3))) void*)(base + cw * 1024), 16, 0, 0);
-        const int col = kv0 + cchunk * 16;
-        const uint8_t* vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
+        const uint8_t* vs;
+        if constexpr (VTOK) {
+            int vr = kv0 + crow;
+            vr = vr < N ? vr : N - 1;  // rows past the end repeat the last key; their probabilities are zero
+            vs = real ? Vg + (size_t)vr * 64 + vchunk * 16 : zero;
+        } else {
+            const int col = kv0 + cchunk * 16;
+            vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
+        }
         if (copy_v)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
                                              (__attribute__((address_space(3))) void*)(base + 4096 + cw * 1024), 16, 0, 0);
@@ -162,6 +185,15 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
     // operand fetch: lane (i = lane%32, h) reads chunks 2h, 2h+1 of row (32 t + i)
     const unsigned fbase = lds_addr(lds) + ql * 64;
     const unsigned fpc0 = ((2 * h) ^ ((ql >> 2) & 3)) * 16, fpc1 = fpc0 ^ 16;
+    // token-major V: the 16-lane group (a = (lane / 16) % 2, h) turns, per read, keys 32 h + 8 j .. + 7 x channels
+    // 32 d + 16 a .. + 15; lane l of the group points at key row l / 2, half l % 2 of the 16 channel bytes
+    unsigned vtb[2];
+    {
+        const int l16 = lane & 15, a = (lane >> 4) & 1, f = ((l16 >> 3) & 1) << 1;  // f: swizzle of row l16 / 2 (+ multiples of 8)
+        const unsigned row_off = (unsigned)(32 * h + (l16 >> 1)) * 64 + (l16 & 1) * 8;
+        vtb[0] = lds_addr(lds) + 4096 + row_off + ((0 + a) ^ f) * 16;
+        vtb[1] = lds_addr(lds) + 4096 + row_off + ((2 + a) ^ f) * 16;
+    }
 
     v16f o_acc[kQT][2];
 #pragma unroll
@@ -215,27 +247,49 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         __builtin_amdgcn_s_barrier();
         issue_loads(it + 3, it + 3 < n_tiles);
         const unsigned st = fbase + (it & (kStages - 1)) * kStage;
-        v4i kl[2], kh[2], vl[2], vh[2];
+        v4i kl[2], kh[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             kl[t] = t ? lds_read_b128<2048>(st + fpc0) : lds_read_b128<0>(st + fpc0);
             kh[t] = t ? lds_read_b128<2048>(st + fpc1) : lds_read_b128<0>(st + fpc1);
         }
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            vl[t] = t ? lds_read_b128<4096 + 2048>(st + fpc0) : lds_read_b128<4096>(st + fpc0);
-            vh[t] = t ? lds_read_b128<4096 + 2048>(st + fpc1) : lds_read_b128<4096>(st + fpc1);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1])
-                     :
-                     : "memory");
         v8i kf[2], vf[2];
+        if constexpr (VTOK) {
+            const unsigned so = (it & (kStages - 1)) * kStage;
+            v2i r[2][4];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            kf[t] = v8i{kl[t][0], kl[t][1], kl[t][2], kl[t][3], kh[t][0], kh[t][1], kh[t][2], kh[t][3]};
-            vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
+            for (int d = 0; d < 2; ++d) {
+                r[d][0] = lds_read_tr_b64<0>(so + vtb[d]);
+                r[d][1] = lds_read_tr_b64<512>(so + vtb[d]);
+                r[d][2] = lds_read_tr_b64<1024>(so + vtb[d]);
+                r[d][3] = lds_read_tr_b64<1536>(so + vtb[d]);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]),
+                           "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int d = 0; d < 2; ++d)
+                vf[d] = v8i{r[d][0][0], r[d][0][1], r[d][1][0], r[d][1][1], r[d][2][0], r[d][2][1], r[d][3][0], r[d][3][1]};
+        } else {
+            v4i vl[2], vh[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                vl[t] = t ? lds_read_b128<4096 + 2048>(st + fpc0) : lds_read_b128<4096>(st + fpc0);
+                vh[t] = t ? lds_read_b128<4096 + 2048>(st + fpc1) : lds_read_b128<4096>(st + fpc1);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            kf[t] = v8i{kl[t][0], kl[t][1], kl[t][2], kl[t][3], kh[t][0], kh[t][1], kh[t][2], kh[t][3]};
 
         // per-key scales of this lane's 32 keys (key = kv0 + 32h + e): broadcast reads from the stage's scale rows
         float skv[SCALED ? 32 : 1], svv[SCALED ? 32 : 1];
@@ -502,8 +556,9 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);
     if (out_dtype != Q8_BF16 && out_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_attn_fwd: output dtype %d", out_dtype);
     if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE | Q8_ATTN_O_TOKEN_MAJOR)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
-    if (v_layout != Q8_V_DS) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V layout %d (only Q8_V_DS [B,H,64,Nv] is implemented)", v_layout);
-    if (v_row_stride < N || v_row_stride % 16 != 0)
+    if (v_layout != Q8_V_DS && v_layout != Q8_V_SD) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V layout %d", v_layout);
+    const bool vtok = v_layout == Q8_V_SD;
+    if (!vtok && (v_row_stride < N || v_row_stride % 16 != 0))
         return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V row stride %lld must be >= N and a multiple of 16", (long long)v_row_stride);
     const bool scaled = sq || sk || sv;
     if (scaled && !(sq && sk && sv)) return fail(Q8_ERR_NULL, "q8_attn_fwd: sq, sk, sv must be given together");
@@ -514,7 +569,9 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
                  (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
     if (!(softmax_scale > 0.f)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: softmax_scale must be positive");
     const int cfg = g_attn_cfg;
-    if (N <= 128 && !scaled && cfg != 3) {
+    if (vtok && (cfg == 1 || cfg == 2))
+        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4-wave tuning shapes read V^T only (Q8_V_DS)");
+    if (N <= 128 && !scaled && cfg != 3 && !vtok) {
         // K and V^T stay in registers; enough waves to fill the device, each walking over several query tiles
         // (tiles per wave and batch: about 2048 waves in all, one 8-wave workgroup per CU)
         const long q_tiles = (M + 31) / 32;
@@ -530,9 +587,12 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
 #define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV)                                                                         \
     hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
                                                                   (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
-#define Q8_ATTN_CFG(OUTT, SC)                                  \
-    if (cfg == 1) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4);               \
-    else if (cfg == 2) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4);          \
+#define Q8_ATTN_CFG(OUTT, SC)                                                                                     \
+    if (vtok)                                                                                                      \
+        hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, 1, 8, true>), dim3((unsigned)((M + 255) / 256), (unsigned)(B * H)), \
+                           dim3(512), 0, stream, p);                                                               \
+    else if (cfg == 1) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4);                                                             \
+    else if (cfg == 2) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4);                                                             \
     else Q8_ATTN_LAUNCH(OUTT, SC, 1, 8)
     if (out_dtype == Q8_BF16) {
         if (scaled) { Q8_ATTN_CFG(Q8_BF16, true); } else { Q8_ATTN_CFG(Q8_BF16, false); }

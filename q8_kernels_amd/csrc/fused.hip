@@ -194,7 +194,10 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
 // stages plus log2(LH) lane stages. Codes go to the head-major layout [B, H, S, D] the attention kernel reads.
 // The options are uniform branches: cs != NULL rotates, scales != NULL quantizes per (token, head).
 // PAIR: a second tensor (K next to Q of a self-attention) goes through the same steps with the same tables, which are
-// then read once: they are 8 of the 11 bytes per element that one tensor moves.
+// then read once: they are 8 of the 11 bytes per element that one tensor moves. xv != NULL (uniform): the V projection
+// of the same tokens is cast to e4m3 on the way (per (token, head) absmax scales when scales_v != NULL) and written
+// token-major per head, [B, H, S, D], the layout the attention kernel reads with Q8_V_SD
+// (the cast of q8_kernels/functional/flash_attention.py:38-45 without its transposed copy).
 template <int LANES, int CH, int LH, bool PAIR>
 __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __restrict__ x, int64_t x_row_stride,
                                                               const uint16_t* __restrict__ x2, int64_t x2_row_stride,
@@ -202,6 +205,8 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
                                                               const float* __restrict__ cs, const float* __restrict__ sn,
                                                               uint8_t* __restrict__ codes, float* __restrict__ scales,
                                                               uint8_t* __restrict__ codes2, float* __restrict__ scales2,
+                                                              const uint16_t* __restrict__ xv, int64_t xv_row_stride,
+                                                              uint8_t* __restrict__ codes_v, float* __restrict__ scales_v,
                                                               int64_t tokens, int S, int apply_fht, float scale,
                                                               int mid_bf16) {
     static_assert(LH <= LANES, "a head may not span tokens");
@@ -288,6 +293,30 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
                 w[1] = (int)pack4_e4m3_c10(v[n][c][4], v[n][c][5], v[n][c][6], v[n][c][7]);
             }
             *reinterpret_cast<v2i*>(cout + orow * D + (t % LH) * 8) = w;
+        }
+    }
+    if (xv != nullptr) {
+        float vv[CH][8];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) load8<Q8_BF16>(xv + tok * xv_row_stride, (c * LANES + t) * 8, vv[c]);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int h = (c * LANES + t) / LH;
+            const int64_t orow = (b * H + h) * S + s;
+            v2i w;
+            if (scales_v != nullptr) {
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(vv[c][i]));
+                amax = group_max<LH>(amax);
+                const float ratio = quant_ratio<Q8_E4M3>(amax);
+                if ((t % LH) == 0) scales_v[orow] = quant_scale<Q8_E4M3>(amax, ratio, 0);
+                w = quant_codes8<Q8_E4M3>(vv[c], ratio, 0);
+            } else {
+                w[0] = (int)pack4_e4m3_c10(vv[c][0], vv[c][1], vv[c][2], vv[c][3]);
+                w[1] = (int)pack4_e4m3_c10(vv[c][4], vv[c][5], vv[c][6], vv[c][7]);
+            }
+            *reinterpret_cast<v2i*>(codes_v + orow * D + (t % LH) * 8) = w;
         }
     }
 }
@@ -454,8 +483,8 @@ extern "C" int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, in
 
 static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_stride, const void* x2, int64_t x2_row_stride,
                              const float* norm_w, const float* norm_w2, const float* cos_t, const float* sin_t, void* codes, float* scales, void* codes2,
-                             float* scales2, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
-                             hipStream_t stream) {
+                             float* scales2, const void* xv, int64_t xv_row_stride, void* codes_v, float* scales_v, int B, int S,
+                             int H, int D, int apply_fht, float scale, int mid_dtype, hipStream_t stream) {
     const bool pair = x2 != nullptr;
     if (B < 0 || S < 0 || H <= 0) return fail(Q8_ERR_SHAPE, "%s: B %d S %d H %d", who, B, S, H);
     if (D != 64 && D != 128) return fail(Q8_ERR_SHAPE, "%s: head dim %d (want 64 or 128)", who, D);
@@ -475,6 +504,13 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
         (reinterpret_cast<uintptr_t>(codes) % 8) || (pair && (reinterpret_cast<uintptr_t>(codes2) % 8)))
         return fail(Q8_ERR_ALIGN, "%s: x and tables must be 16-byte aligned, codes 8-byte aligned", who);
     if (mid_dtype != Q8_BF16 && mid_dtype != Q8_F32) return fail(Q8_ERR_DTYPE, "%s: intermediate dtype %d", who, mid_dtype);
+    if (xv) {
+        if (!codes_v) return fail(Q8_ERR_NULL, "%s: null pointer", who);
+        if (xv_row_stride < dim || xv_row_stride % 8 != 0) return fail(Q8_ERR_SHAPE, "%s: V row stride %lld", who, (long long)xv_row_stride);
+        if (!aligned16(xv) || (reinterpret_cast<uintptr_t>(codes_v) % 8))
+            return fail(Q8_ERR_ALIGN, "%s: V must be 16-byte aligned, its codes 8-byte aligned", who);
+        if ((scales_v == nullptr) != (scales == nullptr)) return fail(Q8_ERR_NULL, "%s: all scale outputs or none", who);
+    }
     const int64_t tokens = (int64_t)B * S;
     const int lanes = small ? (int)(dim / 8) : 64;
     const int64_t grid = (tokens + (kBlock / lanes) - 1) / (kBlock / lanes);
@@ -482,8 +518,9 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
 #define PREP_ARGS                                                                                                        \
     static_cast<const uint16_t*>(x), x_row_stride, static_cast<const uint16_t*>(x2), x2_row_stride, norm_w, norm_w2,     \
         cos_t, sin_t,                                                                                                    \
-        static_cast<uint8_t*>(codes), scales, static_cast<uint8_t*>(codes2), scales2, tokens, S, apply_fht, scale,       \
-        mid_dtype == Q8_BF16 ? 1 : 0
+        static_cast<uint8_t*>(codes), scales, static_cast<uint8_t*>(codes2), scales2,                                    \
+        static_cast<const uint16_t*>(xv), xv_row_stride, static_cast<uint8_t*>(codes_v), scales_v, tokens, S, apply_fht, \
+        scale, mid_dtype == Q8_BF16 ? 1 : 0
 #define PREP_LAUNCH(LANES, CH, LH)                                                                                       \
     if (pair) hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH, true>), dim3((unsigned)grid), dim3(kBlock), 0, stream, PREP_ARGS); \
     else hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH, false>), dim3((unsigned)grid), dim3(kBlock), 0, stream, PREP_ARGS)
@@ -512,7 +549,8 @@ extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float*
                                const float* sin_t, void* codes, float* scales, int B, int S, int H, int D, int apply_fht,
                                float scale, int mid_dtype, q8_stream_t stream_) {
     return attn_prep_qk_impl("q8_attn_prep_qk", x, x_row_stride, nullptr, 0, norm_w, nullptr, cos_t, sin_t, codes, scales, nullptr,
-                             nullptr, B, S, H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
+                             nullptr, nullptr, 0, nullptr, nullptr, B, S, H, D, apply_fht, scale, mid_dtype,
+                             static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
@@ -521,7 +559,19 @@ extern "C" int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const
                                     int D, int apply_fht, float scale, int mid_dtype, q8_stream_t stream_) {
     if (!xk) return fail(Q8_ERR_NULL, "q8_attn_prep_qk_pair: null pointer");
     return attn_prep_qk_impl("q8_attn_prep_qk_pair", xq, xq_row_stride, xk, xk_row_stride, norm_wq, norm_wk, cos_t, sin_t, codes_q, scales_q,
-                             codes_k, scales_k, B, S, H, D, apply_fht, scale, mid_dtype, static_cast<hipStream_t>(stream_));
+                             codes_k, scales_k, nullptr, 0, nullptr, nullptr, B, S, H, D, apply_fht, scale, mid_dtype,
+                             static_cast<hipStream_t>(stream_));
+}
+
+extern "C" int q8_attn_prep_qkv(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride, const void* xv,
+                                int64_t xv_row_stride, const float* norm_wq, const float* norm_wk, const float* cos_t,
+                                const float* sin_t, void* codes_q, float* scales_q, void* codes_k, float* scales_k,
+                                void* codes_v, float* scales_v, int B, int S, int H, int D, int apply_fht, float scale,
+                                int mid_dtype, q8_stream_t stream_) {
+    if (!xk || !xv) return fail(Q8_ERR_NULL, "q8_attn_prep_qkv: null pointer");
+    return attn_prep_qk_impl("q8_attn_prep_qkv", xq, xq_row_stride, xk, xk_row_stride, norm_wq, norm_wk, cos_t, sin_t, codes_q, scales_q,
+                             codes_k, scales_k, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, apply_fht, scale, mid_dtype,
+                             static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,

@@ -72,7 +72,19 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
-    if q.shape == k.shape:  # self-attention: one pass over both, the tables are read once
+    if q.shape == k.shape == v.shape and d == 64 and (k.shape[1] > 128 or per_token_scales):
+        # self-attention: one pass over the three projections (the tables are read once, V is only cast and stays
+        # token-major; the attention kernel turns its tiles while reading them from LDS). Sequences of at most 128
+        # keys with unit scales keep the transposed V: the register-resident kernel that serves them reads V^T.
+        qc, kc, vc = _C.attn_prep_qkv(q, k, v, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                                      q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
+        if per_token_scales:
+            (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
+            return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
+                                      v_scales=vs, token_major_out=True, v_token_major=True)
+        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                  v_token_major=True)
+    if q.shape == k.shape:  # one pass over q and k
         qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
                                       q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
     else:

@@ -327,3 +327,54 @@ def test_register_resident_path_for_short_kv(dev, n, lens):
     assert o8.dtype == E4M3 and ((o8.cpu().float() - short.cpu().float()).abs() <= 0.07 * short.cpu().float().abs() + 0.02).all()
     unit = _C().flash_attention(*args, out_dtype=torch.bfloat16, p_unit_range=True)
     _check(unit, q, k, v, 0.125, l, what="register-resident, p <= 1", p_scale=1.0)
+
+
+@pytest.mark.parametrize("m,n,lens", [(256, 64, None), (33, 17, None), (300, 640, None), (512, 1000, [1000, 333]),
+                                      (130, 128, [128, 5]), (70, 200, [0, 200]), (1, 1, None), (257, 6144, None)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_token_major_v_gives_the_bits_of_the_transposed_layout(dev, m, n, lens, scaled):
+    """V passed as [B,H,N,64] (turned by the kernel while it reads its LDS tile) against the same V passed
+    pre-transposed: the two paths feed identical operands to identical arithmetic, so every output bit agrees;
+    the transposed layout is checked against the oracle once more here."""
+    from q8_kernels_amd import _lib
+    b, h = 2, 3
+    g = torch.Generator().manual_seed(m * 31 + n)
+    if scaled:
+        qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)
+        kf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 4 + 0.2)
+        vf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 2 + 0.5)
+        (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+        kw = dict(q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+        sc = (sq, sk, sv)
+    else:
+        q, k, v = _inputs(m * 1000 + n, b, h, m, n)
+        kw, sc = {}, (None, None, None)
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+    lens_d = None if lens is None else lens_t.to(dev)
+    for out_dtype in (torch.bfloat16, E4M3):
+        _lib.check(_lib.lib().q8_attn_set_config(3))  # the transposed layout through the general kernel as well
+        try:
+            want = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens_d, out_dtype=out_dtype, **kw)
+        finally:
+            _lib.check(_lib.lib().q8_attn_set_config(0))
+        got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=out_dtype,
+                                   v_token_major=True, **kw)
+        assert torch.equal(got.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu(),
+                           want.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu()), (m, n, lens, scaled, out_dtype)
+    if n <= 1000:
+        got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=torch.bfloat16,
+                                   v_token_major=True, **kw)
+        _check(got, q, k, v, 0.125, lens_t, sc, what="token-major V m=%d n=%d" % (m, n))
+
+
+def test_token_major_v_rejects_what_it_cannot_do(dev):
+    from q8_kernels_amd import Q8Error, _lib
+    q, k, v = _inputs(3, 1, 1, 64, 64)
+    with pytest.raises(RuntimeError):  # a token-major V has K's shape
+        _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev)[..., :48], 0.125, None, v_token_major=True)
+    _lib.check(_lib.lib().q8_attn_set_config(1))
+    try:
+        with pytest.raises(Q8Error):
+            _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, None, v_token_major=True)
+    finally:
+        _lib.check(_lib.lib().q8_attn_set_config(0))

@@ -191,6 +191,33 @@ def test_attn_prep_qk_pair_equals_two_single_calls(dev, shape, rope, scaled):
         assert_bit_equal(pk, sk, "k codes")
 
 
+@pytest.mark.parametrize("shape", [(2, 70, 8, 64), (1, 33, 32, 64), (3, 5, 1, 64), (1, 300, 24, 64), (2, 19, 8, 128)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_qkv_equals_pair_plus_cast_of_v(dev, shape, scaled):
+    """One pass over the three slices of a fused QKV projection: Q and K as attn_prep_qk_pair gives them, V as the
+    e4m3 cast (or per (token, head) quantisation) of its heads, token-major [B, H, S, D]."""
+    b, s, h, d = shape
+    g = torch.Generator().manual_seed(s * 11 + h)
+    qkv = (torch.randn(b, s, 3 * h * d, generator=g) * 1.5).to(BF16)
+    qkv[0, s // 3] = 0
+    qkv_d = qkv.to(dev)
+    q, k, v = (qkv_d[..., i * h * d:(i + 1) * h * d] for i in range(3))
+    ang = torch.rand(b, s, h * d // 2, generator=g) * 6.28
+    cos, sin = torch.cos(ang).repeat_interleave(2, -1).to(dev), torch.sin(ang).repeat_interleave(2, -1).to(dev)
+    gq, gk, gv = _C().attn_prep_qkv(q, k, v, h, cos, sin, True, 0.125, scaled)
+    wq, wk = _C().attn_prep_qk_pair(q, k, h, cos, sin, True, 0.125, scaled)
+    vh = qkv[..., 2 * h * d:].reshape(b, s, h, d).transpose(1, 2).contiguous()
+    if scaled:
+        wv = O.ref_quant(vh, E4M3)
+        for got, want, what in ((gq, wq, "q"), (gk, wk, "k"), (gv, wv, "v")):
+            assert_bit_equal(got[0], want[0], what + " codes")
+            assert_bit_equal(got[1], want[1], what + " scales")
+    else:
+        assert_bit_equal(gq, wq, "q codes")
+        assert_bit_equal(gk, wk, "k codes")
+        assert_bit_equal(gv, O.e4m3_c10(vh), "v codes")
+
+
 def test_attn_prep_qk_strided_slice_of_fused_projection(dev):
     g = torch.Generator().manual_seed(77)
     qkv = torch.randn(2, 50, 3 * 2048, generator=g).to(BF16)
