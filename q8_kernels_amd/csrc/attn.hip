@@ -247,45 +247,64 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
         __builtin_amdgcn_s_barrier();
         issue_loads(it + 3, it + 3 < n_tiles);
         const unsigned st = fbase + (it & (kStages - 1)) * kStage;
-        v4i kl[2], kh[2];
+        const unsigned so = (it & (kStages - 1)) * kStage;
+        const unsigned sc = lds_addr(lds_sc) + (it & (kStages - 1)) * 512 + 128 * h;
+        (void)so; (void)sc;
+        // The LDS reads of a tile. Unit scales: K and V operands together, one wait. Per-token scales: K and the 32 key
+        // scales of this lane first (the logits wait for the K operand only, the scales arrive under the two MFMAs); the
+        // value scales and the V operand are requested once the logits have been scaled and arrive under the exponentials.
+        v4i kl[2], kh[2], vl[2], vh[2], rk[SCALED ? 8 : 1], rv[SCALED ? 8 : 1];
+        v2i vr[2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             kl[t] = t ? lds_read_b128<2048>(st + fpc0) : lds_read_b128<0>(st + fpc0);
             kh[t] = t ? lds_read_b128<2048>(st + fpc1) : lds_read_b128<0>(st + fpc1);
         }
+        auto read_v = [&]() __attribute__((always_inline)) {
+            if constexpr (VTOK) {
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+                    vr[d][0] = lds_read_tr_b64<0>(so + vtb[d]);
+                    vr[d][1] = lds_read_tr_b64<512>(so + vtb[d]);
+                    vr[d][2] = lds_read_tr_b64<1024>(so + vtb[d]);
+                    vr[d][3] = lds_read_tr_b64<1536>(so + vtb[d]);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    vl[t] = t ? lds_read_b128<4096 + 2048>(st + fpc0) : lds_read_b128<4096>(st + fpc0);
+                    vh[t] = t ? lds_read_b128<4096 + 2048>(st + fpc1) : lds_read_b128<4096>(st + fpc1);
+                }
+            }
+        };
+        // s_waitcnt lgkmcnt(0) that names the V operand registers, then the operand in MFMA form
         v8i kf[2], vf[2];
-        if constexpr (VTOK) {
-            const unsigned so = (it & (kStages - 1)) * kStage;
-            v2i r[2][4];
+        auto wait_v = [&]() __attribute__((always_inline)) {
+            if constexpr (VTOK) {
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(vr[0][0]), "+v"(vr[0][1]), "+v"(vr[0][2]), "+v"(vr[0][3]), "+v"(vr[1][0]), "+v"(vr[1][1]),
+                               "+v"(vr[1][2]), "+v"(vr[1][3])
+                             :
+                             : "memory");
 #pragma unroll
-            for (int d = 0; d < 2; ++d) {
-                r[d][0] = lds_read_tr_b64<0>(so + vtb[d]);
-                r[d][1] = lds_read_tr_b64<512>(so + vtb[d]);
-                r[d][2] = lds_read_tr_b64<1024>(so + vtb[d]);
-                r[d][3] = lds_read_tr_b64<1536>(so + vtb[d]);
+                for (int d = 0; d < 2; ++d)
+                    vf[d] = v8i{vr[d][0][0], vr[d][0][1], vr[d][1][0], vr[d][1][1], vr[d][2][0], vr[d][2][1], vr[d][3][0], vr[d][3][1]};
+            } else {
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1]) : : "memory");
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
             }
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]),
-                           "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3])
-                         :
-                         : "memory");
-#pragma unroll
-            for (int d = 0; d < 2; ++d)
-                vf[d] = v8i{r[d][0][0], r[d][0][1], r[d][1][0], r[d][1][1], r[d][2][0], r[d][2][1], r[d][3][0], r[d][3][1]};
+        };
+        if constexpr (SCALED) {
+            rk[0] = lds_read_b128<0>(sc); rk[1] = lds_read_b128<16>(sc); rk[2] = lds_read_b128<32>(sc); rk[3] = lds_read_b128<48>(sc);
+            rk[4] = lds_read_b128<64>(sc); rk[5] = lds_read_b128<80>(sc); rk[6] = lds_read_b128<96>(sc); rk[7] = lds_read_b128<112>(sc);
+            // LDS reads return in order: at most the 8 scale reads outstanding = the K operand is there
+            asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]) : : "memory");
         } else {
-            v4i vl[2], vh[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                vl[t] = t ? lds_read_b128<4096 + 2048>(st + fpc0) : lds_read_b128<4096>(st + fpc0);
-                vh[t] = t ? lds_read_b128<4096 + 2048>(st + fpc1) : lds_read_b128<4096>(st + fpc1);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]), "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1])
-                         :
-                         : "memory");
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                vf[t] = v8i{vl[t][0], vl[t][1], vl[t][2], vl[t][3], vh[t][0], vh[t][1], vh[t][2], vh[t][3]};
+            read_v();
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kl[0]), "+v"(kh[0]), "+v"(kl[1]), "+v"(kh[1]) : : "memory");
+            wait_v();
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -293,24 +312,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
 
         // per-key scales of this lane's 32 keys (key = kv0 + 32h + e): broadcast reads from the stage's scale rows
         float skv[SCALED ? 32 : 1], svv[SCALED ? 32 : 1];
-        if constexpr (SCALED) {
-            const unsigned sc = lds_addr(lds_sc) + (it & (kStages - 1)) * 512 + 128 * h;
-            v4i r[16];
-            r[0] = lds_read_b128<0>(sc); r[1] = lds_read_b128<16>(sc); r[2] = lds_read_b128<32>(sc); r[3] = lds_read_b128<48>(sc);
-            r[4] = lds_read_b128<64>(sc); r[5] = lds_read_b128<80>(sc); r[6] = lds_read_b128<96>(sc); r[7] = lds_read_b128<112>(sc);
-            r[8] = lds_read_b128<256>(sc); r[9] = lds_read_b128<272>(sc); r[10] = lds_read_b128<288>(sc); r[11] = lds_read_b128<304>(sc);
-            r[12] = lds_read_b128<320>(sc); r[13] = lds_read_b128<336>(sc); r[14] = lds_read_b128<352>(sc); r[15] = lds_read_b128<368>(sc);
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]), "+v"(r[8]),
-                           "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]), "+v"(r[15])
-                         :
-                         : "memory");
-#pragma unroll
-            for (int e = 0; e < 32; ++e) {
-                skv[e] = __int_as_float(r[e >> 2][e & 3]);
-                svv[e] = __int_as_float(r[8 + (e >> 2)][e & 3]);
-            }
-        }
         const bool partial = kv0 + kKV > valid;
 
 #pragma unroll
@@ -323,12 +324,32 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
                 for (int e = 0; e < 16; ++e) z[e] = 0.f;
                 s[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[t], qf[qt], z, 0, 0, 0, 0, 0, 0);
             }
+            if constexpr (SCALED) {
+                if (qt == 0) {
+                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                 : "+v"(rk[0]), "+v"(rk[1]), "+v"(rk[2]), "+v"(rk[3]), "+v"(rk[4]), "+v"(rk[5]), "+v"(rk[6]), "+v"(rk[7])
+                                 :
+                                 : "memory");
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) skv[e] = __int_as_float(rk[e >> 2][e & 3]);
+                }
+            }
             // logits in units of log2: x = s * c (c > 0); the maximum is taken on the raw accumulators
             float x[32];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) x[16 * t + e] = SCALED ? s[t][e] * skv[16 * t + e] : s[t][e];
+            if constexpr (SCALED) {
+                if (qt == 0) {
+                    // the scaled logits exist (with one query tile per wave the key scales and the K operand are dead now):
+                    // the value scales and the V operand are requested and arrive under the exponentials
+                    asm volatile("" : "+v"(x[15]), "+v"(x[31]));
+                    rv[0] = lds_read_b128<256>(sc); rv[1] = lds_read_b128<272>(sc); rv[2] = lds_read_b128<288>(sc); rv[3] = lds_read_b128<304>(sc);
+                    rv[4] = lds_read_b128<320>(sc); rv[5] = lds_read_b128<336>(sc); rv[6] = lds_read_b128<352>(sc); rv[7] = lds_read_b128<368>(sc);
+                    read_v();
+                }
+            }
             if (partial) {
 #pragma unroll
                 for (int e = 0; e < 32; ++e)
@@ -355,9 +376,21 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams 
             float pr[32];
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                const float pe = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^p_shift: inside the e4m3 range
-                psum += pe;
-                pr[e] = SCALED ? pe * svv[e] : pe;
+                pr[e] = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^p_shift: inside the e4m3 range
+                psum += pr[e];
+            }
+            if constexpr (SCALED) {
+                if (qt == 0) {
+                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                 : "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]), "+v"(rv[4]), "+v"(rv[5]), "+v"(rv[6]), "+v"(rv[7])
+                                 :
+                                 : "memory");
+                    wait_v();
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) svv[e] = __int_as_float(rv[e >> 2][e & 3]);
+                }
+#pragma unroll
+                for (int e = 0; e < 32; ++e) pr[e] *= svv[e];
             }
             v8i pf;
 #pragma unroll
