@@ -146,7 +146,7 @@ def _extras_attn(dev, steps, warmup, g, out):
 
     t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk,
                                             v_scales=sv), steps, warmup)
-    out["attn_self_fp8_per_token_scales"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 8 waves x 32 queries>")
+    out["attn_self_fp8_per_token_scales"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>")
     t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16), steps, warmup)
     out["attn_self_fp8_reference_casts"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>")
     v_tok = vt.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)  # [B,H,S,64]: V as the fused prologue leaves it

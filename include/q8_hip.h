@@ -302,9 +302,10 @@ int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int3
                 float softmax_scale, int out_dtype, int flags, q8_stream_t stream);
 
 /*
- * Workgroup-shape override for q8_attn_fwd: 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries,
- * 2 = 4 waves x 32 queries, 3 = as 0 without the register-resident kernel that otherwise takes N <= 128 with unit
- * scales. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
+ * Workgroup-shape override for q8_attn_fwd: 0 = the default of the mode (unit scales: 8 waves x 32 queries, per-token
+ * scales: 4 waves x 32 queries), 1 = 4 waves x 64 queries (Q8_V_DS only), 2 = 4 waves x 32 queries, 3 = as 0 without the
+ * register-resident kernel that otherwise takes N <= 128 with unit scales, 4 = 8 waves x 32 queries. All shapes give the
+ * same bits. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
  * workgroup is fixed at 4 warps x 16 queries, csrc/flash_attention/flash_attention_cuda.cu:279-287).
  */
 int q8_attn_set_config(int cfg);

@@ -1,6 +1,7 @@
 // FP8 FlashAttention-2 forward for gfx950, head dim 64, non-causal, optional per-batch KV length.
 //
-// One workgroup = 8 waves x 32 query rows of one (batch, head) (4 x 64 and 4 x 32 are instantiated as well); KV is
+// One workgroup = 8 waves x 32 query rows of one (batch, head) with unit scales, 4 waves x 32 with per-token scales (whose
+// register need allows three such workgroups on a CU but only one of 8 waves); 4 x 64 is instantiated as well. KV is
 // walked forward in tiles of 64 keys that all waves share through a four-stage LDS ring filled by
 // global_load_lds_dwordx4. Key / value sequences of at most 128 tokens with unit scales take attn_short_kernel instead.
 // V arrives either channel-major per head (V^T [B,H,64,Nv], Q8_V_DS) or token-major like K ([B,H,N,64], Q8_V_SD); the
@@ -91,7 +92,7 @@ __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, con
 // kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
 // VTOK: V is token-major ([B,H,N,64])
 template <int OUT, bool SCALED, int kQT, int kWaves, bool VTOK = false>
-__global__ __launch_bounds__(kWaves * 64) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 3 : 1) void attn_fwd_kernel(const AttnParams p) {
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
     __shared__ __attribute__((aligned(256))) float lds_sc[SCALED ? kStages * 128 : 4];  // per stage: sk[64], sv[64]
@@ -569,11 +570,12 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
 
 using namespace q8;
 
-static thread_local int g_attn_cfg = 0;  // per thread: 0 = 8 waves x 32 queries (default), 1 = 4 waves x 64 queries, 2 = 4 waves x 32 queries,
-                            // 3 = as 0 and without the register-resident path for N <= 128
+// per thread: 0 = default (unit scales: 8 waves x 32 queries; per-token scales: 4 waves x 32 queries), 1 = 4 waves x 64
+// queries, 2 = 4 waves x 32 queries, 3 = as 0 and without the register-resident path for N <= 128, 4 = 8 waves x 32 queries
+static thread_local int g_attn_cfg = 0;
 
 extern "C" int q8_attn_set_config(int cfg) {
-    if (cfg < 0 || cfg > 3) return fail(Q8_ERR_FLAGS, "q8_attn_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 4) return fail(Q8_ERR_FLAGS, "q8_attn_set_config: %d", cfg);
     g_attn_cfg = cfg;
     return Q8_OK;
 }
@@ -602,8 +604,8 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
                  (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
     if (!(softmax_scale > 0.f)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: softmax_scale must be positive");
     const int cfg = g_attn_cfg;
-    if (vtok && (cfg == 1 || cfg == 2))
-        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4-wave tuning shapes read V^T only (Q8_V_DS)");
+    if (vtok && cfg == 1)
+        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape reads V^T only (Q8_V_DS)");
     if (N <= 128 && !scaled && cfg != 3 && !vtok) {
         // K and V^T stay in registers; enough waves to fill the device, each walking over several query tiles
         // (tiles per wave and batch: about 2048 waves in all, one 8-wave workgroup per CU)
@@ -617,20 +619,25 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
             hipLaunchKernelGGL((attn_short_kernel<Q8_E4M3>), dim3(gx, (unsigned)H), dim3(512), 0, stream, p, (int)tpw);
         return launch_status("q8_attn_fwd");
     }
-#define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV)                                                                         \
-    hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
-                                                                  (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
-#define Q8_ATTN_CFG(OUTT, SC)                                                                                     \
-    if (vtok)                                                                                                      \
-        hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, 1, 8, true>), dim3((unsigned)((M + 255) / 256), (unsigned)(B * H)), \
-                           dim3(512), 0, stream, p);                                                               \
-    else if (cfg == 1) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4);                                                             \
-    else if (cfg == 2) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4);                                                             \
-    else Q8_ATTN_LAUNCH(OUTT, SC, 1, 8)
+    // Shapes: with unit scales 8 waves x 32 queries fit 128 registers (two workgroups = 4 waves per SIMD) and share a K / V
+    // tile among 256 queries. With per-token scales a wave also holds the 64 scales of a tile and needs about 150 registers:
+    // 4 waves x 32 queries then place three workgroups on a CU (3 waves per SIMD) where the 8-wave shape places one.
+    const int waves = (cfg == 1 || cfg == 2) ? 4 : (cfg == 4 ? 8 : (scaled ? 4 : 8));
+    const int qtiles = cfg == 1 ? 2 : 1;
+#define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV, VT)                                                                           \
+    hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV, VT>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
+                                                                      (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
+#define Q8_ATTN_CFG(OUTT, SC)                                                        \
+    if (qtiles == 2) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4, false);                           \
+    else if (waves == 4) {                                                            \
+        if (vtok) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4, true); else Q8_ATTN_LAUNCH(OUTT, SC, 1, 4, false); \
+    } else {                                                                          \
+        if (vtok) Q8_ATTN_LAUNCH(OUTT, SC, 1, 8, true); else Q8_ATTN_LAUNCH(OUTT, SC, 1, 8, false); \
+    }
     if (out_dtype == Q8_BF16) {
-        if (scaled) { Q8_ATTN_CFG(Q8_BF16, true); } else { Q8_ATTN_CFG(Q8_BF16, false); }
+        if (scaled) { Q8_ATTN_CFG(Q8_BF16, true) } else { Q8_ATTN_CFG(Q8_BF16, false) }
     } else {
-        if (scaled) { Q8_ATTN_CFG(Q8_E4M3, true); } else { Q8_ATTN_CFG(Q8_E4M3, false); }
+        if (scaled) { Q8_ATTN_CFG(Q8_E4M3, true) } else { Q8_ATTN_CFG(Q8_E4M3, false) }
     }
 #undef Q8_ATTN_CFG
 #undef Q8_ATTN_LAUNCH

@@ -56,7 +56,7 @@ def _check(got, q, k, v, scale, lens=None, sc=(None, None, None), what="", p_sca
         assert cosine(g, exact) >= 0.999, "%s: cosine %g" % (what, cosine(g, exact))
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["8waves_x32q", "4waves_x64q", "4waves_x32q"])
+@pytest.fixture(params=[0, 1, 2, 4], ids=["default", "4waves_x64q", "4waves_x32q", "8waves_x32q"])
 def attn_cfg(request):
     """every workgroup shape q8_attn_set_config offers (the library's default is the first)"""
     from q8_kernels_amd import _lib
@@ -222,7 +222,7 @@ def test_attention_random_shapes(dev, sweep_seed):
     for case in range(14):
         b, h = rnd.choice([(1, 1), (1, 3), (2, 2), (3, 1)])
         m, n = rnd.randint(1, 420), rnd.randint(1, 900)
-        cfg = rnd.choice([0, 1, 2])
+        cfg = rnd.choice([0, 1, 2, 4])
         scaled, masked = rnd.random() < 0.4, rnd.random() < 0.6
         std = rnd.choice([0.5, 1.0, 2.0])
         seed = rnd.randint(0, 1 << 30)
@@ -253,7 +253,7 @@ def test_attention_random_shapes(dev, sweep_seed):
 
 
 def test_workgroup_shapes_give_identical_bits(dev):
-    """A query row meets the same 64-key tiles in the same order whatever the workgroup shape, so the three shapes
+    """A query row meets the same 64-key tiles in the same order whatever the workgroup shape, so the shapes
     of q8_attn_set_config have to agree bit for bit (direct casts with a mask, and per-token scales)."""
     from q8_kernels_amd import _lib
     g = torch.Generator().manual_seed(77)
@@ -266,7 +266,7 @@ def test_workgroup_shapes_give_identical_bits(dev):
     (q2, sq), (k2, sk), (v2, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
     outs = {}
     try:
-        for cfg in (0, 1, 2):
+        for cfg in (0, 1, 2, 4):
             _lib.check(_lib.lib().q8_attn_set_config(cfg))
             plain = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16)
             scaled = _C().flash_attention(q2.to(dev), k2.to(dev), _vt(v2).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
@@ -274,7 +274,7 @@ def test_workgroup_shapes_give_identical_bits(dev):
             outs[cfg] = (plain.cpu().view(torch.int16), scaled.cpu().view(torch.int16))
     finally:
         _lib.check(_lib.lib().q8_attn_set_config(0))
-    for cfg in (1, 2):
+    for cfg in (1, 2, 4):
         assert torch.equal(outs[cfg][0], outs[0][0]), "direct casts, shape %d" % cfg
         assert torch.equal(outs[cfg][1], outs[0][1]), "per-token scales, shape %d" % cfg
 
@@ -357,10 +357,15 @@ def test_token_major_v_gives_the_bits_of_the_transposed_layout(dev, m, n, lens, 
             want = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens_d, out_dtype=out_dtype, **kw)
         finally:
             _lib.check(_lib.lib().q8_attn_set_config(0))
-        got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=out_dtype,
-                                   v_token_major=True, **kw)
-        assert torch.equal(got.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu(),
-                           want.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu()), (m, n, lens, scaled, out_dtype)
+        for cfg in (0, 2, 4):  # the default shape of the mode and both shapes that read token-major V
+            _lib.check(_lib.lib().q8_attn_set_config(cfg))
+            try:
+                got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=out_dtype,
+                                           v_token_major=True, **kw)
+            finally:
+                _lib.check(_lib.lib().q8_attn_set_config(0))
+            assert torch.equal(got.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu(),
+                               want.view(torch.uint8 if out_dtype == E4M3 else torch.int16).cpu()), (m, n, lens, scaled, out_dtype, cfg)
     if n <= 1000:
         got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=torch.bfloat16,
                                    v_token_major=True, **kw)
