@@ -101,12 +101,34 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     assert L.q8_attn_prep_qk(16, 512, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1      # cos without sin
     assert L.q8_attn_prep_qk_pair(16, 512, None, 512, None, None, None, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
     assert L.q8_attn_prep_qk_pair(16, 512, 16, 512, None, None, None, None, 16, 16, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
+    # q8_attn_prep_qkv(xq, sq, xk, sk, xv, sv, nwq, nwk, cos, sin, cq, scq, ck, sck, cv, scv, B, S, H, D, fht, scale, mid, stream)
+    assert L.q8_attn_prep_qkv(None, 512, None, 512, None, 512, None, None, None, None, None, None, None, None, None, None,
+                              0, 5, 8, 64, 1, 1.0, B16, None) == -1                                  # no V at all
+    assert L.q8_attn_prep_qkv(16, 512, 16, 512, 16, 512, None, None, None, None, 16, None, 16, None, None, None,
+                              1, 5, 8, 64, 1, 1.0, B16, None) == -1                                  # V given, its codes not
+    assert L.q8_attn_prep_qkv(16, 512, 16, 512, 16, 500, None, None, None, None, 16, None, 16, None, 16, None,
+                              1, 5, 8, 64, 1, 1.0, B16, None) == -3                                  # V stride < H * D
+    assert L.q8_attn_prep_qkv(16, 512, 16, 512, 16, 512, None, None, None, None, 16, 16, 16, 16, 16, None,
+                              1, 5, 8, 64, 1, 1.0, B16, None) == -1                                  # scales for q, k but not v
+    assert L.q8_attn_prep_qkv(16, 512, 16, 512, 8, 512, None, None, None, None, 16, None, 16, None, 16, None,
+                              1, 5, 8, 64, 1, 1.0, B16, None) == -4                                  # V not 16-byte aligned
+    assert L.q8_attn_prep_qkv(16, 512, 16, 512, 16, 512, None, None, None, None, 16, None, 16, None, 16, None,
+                              0, 5, 8, 64, 1, 1.0, B16, None) == 0                                   # no tokens: nothing to do
     assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 64, 5, None) == -3                          # S_pad % 16
     assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 128, 16, None) == -3
     assert L.q8_gemm_residual(16, 16, None, 16, 16, None, 16, 1, 1, 8, 8, 384, I8, 0, None) == -1
     assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 8, 256, I8, 0, None) == -3     # K must exceed 256
     assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 12, 384, I8, 0, None) == -3    # N % 8
     assert L.q8_gemm_set_config(7) == -6
+    assert L.q8_attn_set_config(5) == -6 and L.q8_attn_set_config(-1) == -6
+    # q8_attn_fwd(q, k, v, o, kv_len, sq, sk, sv, B, H, M, N, D, v_layout, v_row_stride, scale, out_dtype, flags, stream)
+    assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 2, 16, 0.125, B16, 0, None) == -3   # V layout 2
+    assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, _lib.Q8_V_DS, 8, 0.125, B16, 0, None) == -3  # V^T stride
+    assert L.q8_attn_set_config(1) == 0
+    try:  # the 4 waves x 64 queries shape reads V^T only
+        assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, _lib.Q8_V_SD, 0, 0.125, B16, 0, None) == -6
+    finally:
+        assert L.q8_attn_set_config(0) == 0
 
 
 def test_python_wrappers_refuse_cpu_tensors():
