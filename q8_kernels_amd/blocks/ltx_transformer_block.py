@@ -50,6 +50,10 @@ class LTXTransformerBlock(nn.Module):
                 and non_mm_precision == torch.bfloat16 and hidden_states.dim() == 3 and hidden_states.shape[-1] % 8 == 0
                 and not (torch.is_grad_enabled() and (hidden_states.requires_grad or ada_values.requires_grad)))
         bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
+        if fuse:
+            # the six modulation rows as contiguous bfloat16 slices of ONE copy (instead of six strided-to-contiguous copies
+            # further down): the same values, bf16(table + timestep)
+            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = bf(ada_values.transpose(1, 2)).unbind(dim=1)
 
         if fuse:  # (int8 codes, row scales) of the rotated, modulated norm: what attn1's projections would compute
             norm_hidden_states = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm1.weight, bf(scale_msa),
