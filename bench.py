@@ -322,8 +322,11 @@ def main():
     }
     traffic_file = os.path.join(ROOT, "profiles", "gemm_fp8_traffic.json")
     if os.path.exists(traffic_file):
+        # not measured by this run (counters need rocprofv3): the figure of the two --pmc runs summarised under profiles/
         with open(traffic_file) as fh:
-            result["roofline"]["traffic"] = json.load(fh).get("hbm_bytes_per_launch")
+            tr = json.load(fh)
+        result["roofline"]["traffic"] = tr.get("hbm_bytes_per_launch")
+        result["roofline"]["traffic_source"] = tr.get("source")
     if not args.no_cpu:
         result["cpu_baseline"] = _cpu_baseline_gemm(x, w, bias)
     else:
