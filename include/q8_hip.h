@@ -250,6 +250,18 @@ int q8_gemm_residual(const void* A, const void* B, const float* bias, const floa
                      int fuse_gelu, q8_stream_t stream);
 
 /*
+ * q8_gemm_residual (one batch) with a gate: C = bf16(fma(bf16(epi(...)), gate[m / rows_per_gate, n], residual[m, n])),
+ * gate bf16 [ceil(M / rows_per_gate), N]: the gated residual of the AdaLN block,
+ * `attn_output * gate_msa + hidden_states` and `ff_output * gate_mlp + hidden_states`
+ * (q8_kernels/blocks/ltx_transformer_block.py:44,57), in the epilogue of the projection that produces the first factor.
+ * The bits are those of q8_gemm (bf16 output) followed by q8_fma with bf16 operands. rows_per_gate (tokens per batch
+ * element) must be a multiple of 768, so that a 192- or 256-row tile has one gate row; other conditions as q8_gemm_residual.
+ */
+int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, const float* sa, const float* sb,
+                           const void* residual, const void* gate, int64_t rows_per_gate, void* C, int M, int N, int K,
+                           int in_dtype, int fuse_gelu, q8_stream_t stream);
+
+/*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with
  * one tile per workgroup, 2 = 128x128 tiles, 4 = persistent pipelined 256x256 tiles (bf16 or e4m3 output, N % 8 == 0,
  * K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's tile to 192 / 256 rows /

@@ -165,10 +165,13 @@ def _check_input(t, name):
         raise RuntimeError("%s must be contiguous" % name)
 
 
-def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who, residual=None):
+def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who, residual=None, gate=None):
     """Shape rules of csrc/gemm/q8_gemm_api.cpp:45-91: a [.,M,K], b [.,N,K], result always [batch,M,N].
     residual (bfloat16, batch*M*N elements, bfloat16 output only): out = bf16(bf16(result) + residual), in the GEMM's
-    epilogue where the kernel supports the shape, otherwise by a separate addition with the same two roundings."""
+    epilogue where the kernel supports the shape, otherwise by a separate addition with the same two roundings.
+    gate (with residual; bfloat16 [G, N] or [G, 1, N], G dividing the batch*M rows: row r uses gate row r // (rows / G)):
+    out = bf16(fma(bf16(result), gate, residual)), in the epilogue where the kernel supports the shape, otherwise by the
+    fused multiply-add kernel on the projection's output: the same bits."""
     _check_input(a, "a")
     _check_input(b, "b")
     if a.dtype != in_dtype or b.dtype != in_dtype:
@@ -195,12 +198,33 @@ def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who, resi
         if bias.dtype != torch.float32 or bias.numel() != n:
             raise RuntimeError("%s: bias must be float32 with %d elements" % (who, n))
     out = torch.empty((batch, m, n), dtype=out_type, device=a.device)
+    if gate is not None and residual is None:
+        raise RuntimeError("%s: a gate comes with a residual" % who)
     if residual is not None:
         _require_gpu(residual, "residual")
         if out_type != torch.bfloat16 or residual.dtype != torch.bfloat16 or residual.numel() != out.numel():
             raise RuntimeError("%s: residual must be bfloat16 with the output's element count, output bfloat16" % who)
         residual = residual.contiguous()
         fusable = n % 8 == 0 and k % 128 == 0 and k > 256 and m * k < 2 ** 32 and n * k < 2 ** 32 and residual.data_ptr() % 16 == 0
+        if gate is not None:
+            _require_gpu(gate, "gate")
+            rows = batch * m
+            if gate.dtype != torch.bfloat16 or gate.shape[-1] != n or gate.numel() % n != 0 or rows % (gate.numel() // n) != 0:
+                raise RuntimeError("%s: gate must be bfloat16 [G, N] with G dividing the %d output rows" % (who, rows))
+            gate = gate.contiguous()
+            groups = gate.numel() // n
+            per = rows // groups
+            if (fusable and bs_b == 1 and per % 768 == 0 and rows * k < 2 ** 32 and gate.data_ptr() % 16 == 0):
+                with torch.cuda.device(a.device):  # one batch of batch * M rows: a and a_scales are contiguous over them
+                    _lib.check(_lib.lib().q8_gemm_gated_residual(
+                        a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(), residual.data_ptr(),
+                        gate.data_ptr(), per, out.data_ptr(), rows, n, k, _DT[in_dtype], 1 if fuse_gelu else 0, _stream(a)))
+                return out
+            with torch.cuda.device(a.device):
+                _lib.check(_lib.lib().q8_gemm(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
+                                              out.data_ptr(), bs_a, bs_b, m, n, k, _DT[in_dtype], _DT[out_type],
+                                              1 if fuse_gelu else 0, _stream(a)))
+            return fma_8bit(out.view(groups, per, n), gate.view(groups, 1, n), residual.view(groups, per, n)).view(batch, m, n)
         if fusable:
             with torch.cuda.device(a.device):
                 _lib.check(_lib.lib().q8_gemm_residual(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(),
@@ -217,27 +241,27 @@ def _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, in_dtype, who, resi
 
 
 def q8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
-          residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+          residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:40-97."""
-    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm", residual)
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm", residual, gate)
 
 
 def q8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
-               residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+               residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:100-164."""
-    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm_bias", residual)
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.int8, "q8_mm_bias", residual, gate)
 
 
 def fp8_mm(a, b, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
-           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+           residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:167-224."""
-    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm", residual)
+    return _mm(a, b, None, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm", residual, gate)
 
 
 def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optional[torch.dtype] = None, *,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/gemm/q8_gemm_api.cpp:227-291."""
-    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias", residual)
+    return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias", residual, gate)
 
 
 def q8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

@@ -60,9 +60,16 @@ class LTXTransformerBlock(nn.Module):
                                                                   bf(shift_msa), 1.0)
         else:
             norm_hidden_states = self._fma(self.norm1(hidden_states, non_mm_precision), scale_msa, shift_msa, 1.0)
-        attn_output = self.attn1(norm_hidden_states, freqs_cis, None, attention_mask, non_mm_precision, mm_out_dtype,
-                                 attn_type=attn_type)
-        hidden_states = self._fma(attn_output, gate_msa, hidden_states, 0.0)
+        # with the fused path the gated residuals `y * gate + x` are formed in the epilogue of the projection that produces y
+        # (attn1's output projection, the feed-forward's down projection): the bits of the fused multiply-add kernel
+        gated = fuse and mm_out_dtype == torch.bfloat16
+        if gated:
+            hidden_states = self.attn1(norm_hidden_states, freqs_cis, None, attention_mask, non_mm_precision, mm_out_dtype,
+                                       attn_type=attn_type, residual=hidden_states, gate=gate_msa)
+        else:
+            attn_output = self.attn1(norm_hidden_states, freqs_cis, None, attention_mask, non_mm_precision, mm_out_dtype,
+                                     attn_type=attn_type)
+            hidden_states = self._fma(attn_output, gate_msa, hidden_states, 0.0)
 
         # the residual around the cross-attention is added in the epilogue of its output projection where that applies
         hidden_states = self.attn2(hidden_states, freqs_cis=freqs_cis, encoder_hidden_states=encoder_hidden_states,
@@ -72,6 +79,8 @@ class LTXTransformerBlock(nn.Module):
         if fuse:
             codes, row_scales = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm2.weight, bf(scale_mlp),
                                                                  bf(shift_mlp), 1.0)
+            if gated:
+                return self.ff(codes, out_dtype=mm_out_dtype, x_scales=row_scales, residual=hidden_states, gate=gate_mlp)
             ff_output = self.ff(codes, out_dtype=mm_out_dtype, x_scales=row_scales).to(non_mm_precision)
         else:
             norm_hidden_states = self._fma(self.norm2(hidden_states, non_mm_precision), scale_mlp, shift_mlp, 1.0)

@@ -352,6 +352,30 @@ extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias,
     return fuse_gelu ? launch_persist<Q8_E4M3, true>(p, stream) : launch_persist<Q8_E4M3, false>(p, stream);
 }
 
+extern "C" int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, const float* sa, const float* sb,
+                                      const void* residual, const void* gate, int64_t rows_per_gate, void* C, int M, int N, int K,
+                                      int in_dtype, int fuse_gelu, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "q8_gemm_gated_residual";
+    if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;
+    if (int st = check_gemm(who, A, B, C, 1, 1, M, N, K)) return st;
+    if (!sa || !sb || !residual || !gate) return fail(Q8_ERR_NULL, "%s: scales, residual and gate are required", who);
+    if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "%s: input dtype %d", who, in_dtype);
+    if ((reinterpret_cast<uintptr_t>(C) % 16) || (reinterpret_cast<uintptr_t>(residual) % 16) || (reinterpret_cast<uintptr_t>(gate) % 16))
+        return fail(Q8_ERR_ALIGN, "%s: C, residual and gate must be 16-byte aligned", who);
+    // a tile (192 or 256 rows) must lie inside one group of rows that share a gate row
+    if (rows_per_gate <= 0 || rows_per_gate % 768 != 0 || rows_per_gate > 0x7fffffffLL)
+        return fail(Q8_ERR_SHAPE, "%s: rows_per_gate = %lld must be a positive multiple of 768", who, (long long)rows_per_gate);
+    GemmParams p{static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), bias, sa, sb, C, 1, 1, M, N, K};
+    p.residual = residual;
+    p.gate = static_cast<const uint16_t*>(gate);
+    p.rows_per_gate = (int)rows_per_gate;
+    if (!persist_eligible(p))
+        return fail(Q8_ERR_SHAPE, "%s: needs N %% 8 == 0 and K a multiple of 128 above 256 (N %d K %d)", who, N, K);
+    if (in_dtype == Q8_I8) return fuse_gelu ? launch_persist<Q8_I8, true>(p, stream) : launch_persist<Q8_I8, false>(p, stream);
+    return fuse_gelu ? launch_persist<Q8_E4M3, true>(p, stream) : launch_persist<Q8_E4M3, false>(p, stream);
+}
+
 extern "C" int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int K, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;

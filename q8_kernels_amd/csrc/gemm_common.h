@@ -15,6 +15,8 @@ struct GemmParams {
     int batch_a, batch_b;
     int M, N, K;
     const void* residual = nullptr;  // bf16 [batch, M, N] added to the rounded bf16 result (persistent kernel only)
+    const uint16_t* gate = nullptr;  // bf16 [ceil(M / rows_per_gate), N]: with it C = bf16(fma(bf16(result), gate, residual))
+    int rows_per_gate = 0;           // a multiple of the tile height, so that a tile has one gate row
 };
 
 __device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0};

@@ -22,8 +22,9 @@
 
 namespace q8 {
 
-constexpr int kPersistParOffset = kPipeStages * kPipeStageBytes;            // 2 x (sa[256], sb[256], bias[256])
-constexpr int kPersistStageOutOffset = kPersistParOffset + 2 * 3 * 256 * 4;   // 8 waves x 2 KiB
+constexpr int kPersistParBytes = 3 * 256 * 4 + 256 * 2;                      // sa[256], sb[256], bias[256] fp32, gate[256] bf16
+constexpr int kPersistParOffset = kPipeStages * kPipeStageBytes;            // 2 x parameters of a tile
+constexpr int kPersistStageOutOffset = kPersistParOffset + 2 * kPersistParBytes;   // 8 waves x 2 KiB
 constexpr int kPersistLds = kPersistStageOutOffset + 8 * 2048;
 
 __device__ __forceinline__ void lds_write_b128(unsigned addr, v4u v) {
@@ -53,7 +54,9 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 // MT = 32-row MFMA tiles per wave along M: the tile is 64 MT x 256, i.e. 256 x 256 (MT = 4) or 192 x 256 (MT = 3, for
 // problems whose 256-row tiles do not divide evenly over the CUs).
 // RES: C = bf16(bf16(result) + residual), the residual connection around a projection (two roundings, as the separate
-// element-wise addition of the two bf16 tensors gives).
+// element-wise addition of the two bf16 tensors gives); with p.gate (uniform) C = bf16(fma(bf16(result), gate, residual)),
+// the gated residual of an AdaLN block (blocks/ltx_transformer_block.py:44,57 in the reference), one gate row per
+// rows_per_gate rows: what the fused multiply-add kernel gives on the rounded projection.
 template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -115,9 +118,10 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
 #pragma unroll
         for (int i = 0; i < NCOPY; ++i) off[i] = 0;
     };
-    // two 4-byte-per-lane copies per wave: waves 0-3 bring sa and bias, waves 4-7 sb (twice, to keep the count equal)
+    // two 4-byte-per-lane copies per wave: waves 0-3 bring sa and bias, waves 4-7 sb and the tile's gate row (256 bf16 =
+    // 128 dwords: waves 4 / 6 the first 64, waves 5 / 7 the others; without a gate sb a second time, to keep the count equal)
     auto copy_params = [&](const Item& it, int buf, bool live) {
-        float* par = reinterpret_cast<float*>(lds + kPersistParOffset) + buf * 768;
+        float* par = reinterpret_cast<float*>(lds + kPersistParOffset + buf * kPersistParBytes);
         const int j = (wave & 3) * 64 + lane;
         const float* g0;
         const float* g1;
@@ -134,6 +138,14 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             const int n = (it.n0 + j < N) ? it.n0 + j : N - 1;
             g0 = g1 = p.sb + (size_t)it.zb * N + n;
             d0 = d1 = par + 256 + (wave & 3) * 64;
+            if constexpr (RES) {
+                if (p.gate != nullptr) {
+                    const int jj = (wave & 1) * 64 + lane;  // columns 2 jj, 2 jj + 1 of the tile (N is even)
+                    const int n2 = (it.n0 + 2 * jj + 1 < N) ? it.n0 + 2 * jj : N - 2;
+                    g1 = reinterpret_cast<const float*>(p.gate + (size_t)(it.m0 / p.rows_per_gate) * N + n2);
+                    d1 = par + 768 + (wave & 1) * 64;
+                }
+            }
         }
         if (!live) g0 = g1 = reinterpret_cast<const float*>(g_zero16);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g0,
@@ -249,7 +261,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         asm volatile("" : "+v"(lane_e));
         const int r32 = lane_e & 31, h = lane_e >> 5;
         const unsigned stage_out = lds0 + kPersistStageOutOffset + wave * 2048;
-        const unsigned par = lds0 + kPersistParOffset + (item & 1) * 3072;
+        const unsigned par = lds0 + kPersistParOffset + (item & 1) * kPersistParBytes;
         const size_t zc = (size_t)cur.z * M * N;
         const int mw0 = cur.m0 + wave_m * (32 * MT), nw0 = cur.n0 + wave_n * 64;
         v4i sbq[2][2][2], bq[2][2][2];  // [t][wp][low / high 4 columns]
@@ -275,6 +287,13 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                      : "memory");
         uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
         const uint16_t* const rbase = reinterpret_cast<const uint16_t*>(p.residual) + zc;
+        v4i gq = v4i{0, 0, 0, 0};  // the gate of the 8 columns this lane stores (RES with p.gate)
+        if constexpr (RES) {
+            if (p.gate != nullptr) {
+                gq = lds_read_b128<3072>(par + (wave_n * 64 + (lane_e & 7) * 8) * 2);
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(gq) : : "memory");
+            }
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             // the residual rows this lane will store in the four rounds of this MFMA tile: fetched now, used after the
@@ -352,14 +371,27 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0]), "+v"(w[1]) : : "memory");
                 if constexpr (RES) {
+                    if (p.gate != nullptr) {
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                        for (int j = 0; j < 2; ++j)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e];
-                            w[j][e] = (int)pack2_bf16(__uint_as_float(a << 16) + __uint_as_float(r << 16),
-                                                      __uint_as_float(a & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
-                        }
+                            for (int e = 0; e < 4; ++e) {
+                                const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e], gg = (uint32_t)gq[e];
+                                w[j][e] = (int)pack2_bf16(
+                                    __builtin_fmaf(__uint_as_float(a << 16), __uint_as_float(gg << 16), __uint_as_float(r << 16)),
+                                    __builtin_fmaf(__uint_as_float(a & 0xffff0000u), __uint_as_float(gg & 0xffff0000u),
+                                                   __uint_as_float(r & 0xffff0000u)));
+                            }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e];
+                                w[j][e] = (int)pack2_bf16(__uint_as_float(a << 16) + __uint_as_float(r << 16),
+                                                          __uint_as_float(a & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
+                            }
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {

@@ -51,7 +51,17 @@ class GeluFn(torch.autograd.Function):
 
 # ----------------------------------------------------------------------------- int8
 
-def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=None):
+def _gated_residual(out, residual, gate):
+    """the differentiable form of the fused epilogues: out (* gate) + residual with torch operators"""
+    if residual is None:
+        return out
+    if gate is None:
+        return out + residual.reshape(out.shape)
+    groups = gate.numel() // gate.shape[-1]
+    return (out.reshape(groups, -1, out.shape[-1]) * gate.reshape(groups, 1, -1)).reshape(out.shape) + residual.reshape(out.shape)
+
+
+def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=None, gate=None):
     a_needs_q = a.dtype == _FP8 or is_16bit(a)
     b_needs_q = b.dtype == _FP8 or is_16bit(b)
     assert (a_needs_q and scale_a is None) or (a.dtype == torch.int8 and scale_a is not None), \
@@ -65,9 +75,9 @@ def _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=Non
     if b_needs_q:
         b, scale_b = _rotate_quant(b)
     if bias is not None:
-        out = _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
+        out = _C.q8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual, gate=gate)
     else:
-        out = _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
+        out = _C.q8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual, gate=gate)
     return out, b, scale_b
 
 
@@ -100,10 +110,11 @@ class Q8LinearFunc(torch.autograd.Function):
 def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
               scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
               fuse_gelu: bool = False, out_dtype: Optional[torch.dtype] = None,
-              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+              residual: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [..., K] x b [N, K] -> [batch, M, N] through the int8 GEMM; out_dtype None -> e4m3 (as the reference).
     `residual` (bfloat16, the output's shape, out_dtype bfloat16) returns `residual + linear(a)` with the addition done
-    in the GEMM's epilogue: the bits of the separate bfloat16 addition."""
+    in the GEMM's epilogue: the bits of the separate bfloat16 addition. With `gate` (bfloat16 [B, 1, N]) it returns
+    `linear(a) * gate + residual`, one fused multiply-add on the bfloat16 projection (the gated residual of an AdaLN block)."""
     if _needs_grad(a):
         if fuse_gelu and out_dtype is not None and is_16bit(out_dtype):
             # the reference's backward ignores a fused GELU (functional/linear.py:44-52); here the activation follows as
@@ -111,13 +122,13 @@ def q8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = N
             out = GeluFn.apply(Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, False, out_dtype), out_dtype)
         else:
             out = Q8LinearFunc.apply(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype)
-        return out if residual is None else out + residual.reshape(out.shape)
-    return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual)[0]
+        return _gated_residual(out, residual, gate)
+    return _q8_forward(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual, gate)[0]
 
 
 # ----------------------------------------------------------------------------- fp8
 
-def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual=None):
+def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual=None, gate=None):
     assert (is_16bit(a) and scale_a is None) or (a.dtype == _FP8 and scale_a is not None), \
         "FP8LinearFunc: a dtype missmatch"
     assert (is_16bit(b) and scale_b is None) or (b.dtype == _FP8 and scale_b is not None), \
@@ -134,9 +145,9 @@ def _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gel
     if is_16bit(b):
         b, scale_b = quant(b)
     if bias is not None:
-        out = _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
+        out = _C.fp8_mm_bias(a, b, bias, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual, gate=gate)
     else:
-        out = _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual)
+        out = _C.fp8_mm(a, b, scale_a, scale_b, fuse_gelu, out_dtype, residual=residual, gate=gate)
     return out, b, scale_b
 
 
@@ -163,17 +174,19 @@ class FP8LinearFunc(torch.autograd.Function):
 def fp8_linear(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
                scale_a: Optional[torch.Tensor] = None, scale_b: Optional[torch.Tensor] = None,
                use_hadamard: bool = False, out_dtype: Optional[torch.dtype] = None, *,
-               fuse_gelu: bool = False, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+               fuse_gelu: bool = False, residual: Optional[torch.Tensor] = None,
+               gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [..., K] x b [N, K] -> [batch, M, N] through the fp8 GEMM; out_dtype must be 16-bit.
 
     Keyword-only extensions (defaults = the reference's behaviour): `fuse_gelu` applies tanh-GELU in the epilogue;
-    `residual` (bfloat16, the output's shape) returns `residual + linear(a)` with the addition done in the epilogue."""
+    `residual` (bfloat16, the output's shape) returns `residual + linear(a)` with the addition done in the epilogue;
+    with `gate` (bfloat16 [B, 1, N]) `linear(a) * gate + residual` as one fused multiply-add."""
     if _needs_grad(a):  # the fused epilogues carry no gradient: GELU and the residual addition follow as separate steps
         out = FP8LinearFunc.apply(a, b, bias, scale_a, scale_b, out_dtype, use_hadamard)
         if fuse_gelu:
             out = GeluFn.apply(out, out_dtype)
-        return out if residual is None else out + residual.reshape(out.shape)
-    return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual)[0]
+        return _gated_residual(out, residual, gate)
+    return _fp8_forward(a, b, bias, scale_a, scale_b, use_hadamard, out_dtype, fuse_gelu, residual, gate)[0]
 
 
 # ----------------------------------------------------------------------------- int8 base weight + 16-bit LoRA

@@ -47,22 +47,25 @@ class Attention(nn.Module):
     def _split_heads(self, t, batch):
         return t.view(batch, -1, self.num_heads, self.head_dim).transpose(1, 2)
 
-    def _project_out(self, hidden_states, mm_out_dtype, non_mm_precision, residual):
+    def _project_out(self, hidden_states, mm_out_dtype, non_mm_precision, residual, gate=None):
         if residual is None:
             return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
         if (self.fuse_prologue and mm_out_dtype == torch.bfloat16 and non_mm_precision == torch.bfloat16
-                and residual.dtype == torch.bfloat16 and hidden_states.is_cuda):
-            return self.to_out(hidden_states, out_dtype=mm_out_dtype, residual=residual.contiguous())
-        return self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision) + residual
+                and residual.dtype == torch.bfloat16 and hidden_states.is_cuda
+                and (gate is None or gate.dtype == torch.bfloat16)):
+            return self.to_out(hidden_states, out_dtype=mm_out_dtype, residual=residual.contiguous(), gate=gate)
+        out = self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
+        return out + residual if gate is None else out * gate + residual
 
     def forward(self, hidden_states, freqs_cis=None, encoder_hidden_states=None, attention_mask=None,
                 non_mm_precision=torch.bfloat16, mm_out_dtype=None, apply_qk_hadamard=True, attn_type="torch",
-                residual=None):
+                residual=None, gate=None):
         """hidden_states: the activations, or (for self-attention) a tuple (int8 codes, row scales) of their
         Hadamard-rotated quantization, which is what the q / k / v projections consume.
         residual (optional, the output's shape): the result is residual + attention(...), as the blocks compute it
         (q8_kernels/blocks/ltx_transformer_block.py:41-51); with bfloat16 everywhere the addition happens in the
-        epilogue of the output projection."""
+        epilogue of the output projection. gate (optional, with residual, [B, 1, dim]): attention(...) * gate + residual, the
+        gated residual of the AdaLN block (ltx_transformer_block.py:44), one fused multiply-add in that epilogue."""
         if attention_mask is not None and attention_mask.ndim > 1 and attn_type == "q8_kernels":
             # [B, Skv] 0/1 mask -> valid lengths, the reference's rule (first zero; an all-ones row gives 0)
             attention_mask = attention_mask.argmin(-1).squeeze().int()
@@ -98,7 +101,7 @@ class Attention(nn.Module):
                 freqs_cis=freqs_cis if rope else None,
                 q_norm_weight=self._norm_weight(self.q_norm) if self.qk_rms_norm else None,
                 k_norm_weight=self._norm_weight(self.k_norm) if self.qk_rms_norm else None)
-            return self._project_out(hidden_states, mm_out_dtype, non_mm_precision, residual)
+            return self._project_out(hidden_states, mm_out_dtype, non_mm_precision, residual, gate)
         if self.qk_rms_norm:
             query = self.q_norm(query, non_mm_precision)
             key = self.k_norm(key, non_mm_precision)
@@ -124,4 +127,4 @@ class Attention(nn.Module):
             raise ValueError(f"Invalid attention type: {attn_type}")
 
         hidden_states = hidden_states.transpose(1, 2).reshape(batch, -1, self.inner_dim).contiguous()
-        return self._project_out(hidden_states, mm_out_dtype, non_mm_precision, residual)
+        return self._project_out(hidden_states, mm_out_dtype, non_mm_precision, residual, gate)

@@ -13,5 +13,7 @@ class FeedForward(nn.Module):
         self.act = GELU(dim, self.inner_dim, bias=bias)
         self.proj_down = Q8Linear(self.inner_dim, dim, bias=bias)
 
-    def forward(self, x, out_dtype=None, x_scales=None):
-        return self.proj_down(self.act(x, out_dtype=out_dtype, x_scales=x_scales), out_dtype=out_dtype)
+    def forward(self, x, out_dtype=None, x_scales=None, residual=None, gate=None):
+        """residual / gate (extensions, see Q8Linear.forward): returns ff(x) (* gate) + residual from the down projection's epilogue"""
+        return self.proj_down(self.act(x, out_dtype=out_dtype, x_scales=x_scales), out_dtype=out_dtype, residual=residual,
+                              gate=gate)

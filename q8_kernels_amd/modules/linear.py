@@ -42,9 +42,9 @@ class Q8Linear(_QuantLinearBase):
     """int8 weights; activations are FHT-rotated and int8-quantized per token inside forward."""
     weight_dtype = torch.int8
 
-    def forward(self, x, x_scales=None, fuse_gelu=False, out_dtype=None, residual=None):
+    def forward(self, x, x_scales=None, fuse_gelu=False, out_dtype=None, residual=None, gate=None):
         return Q8F.linear.q8_linear(x, self.weight.data, self._bias(), x_scales, self.scales, fuse_gelu, out_dtype,
-                                    residual)
+                                    residual, gate)
 
     @classmethod
     def from_linear(cls, linear: nn.Linear, quant_with_hadamard=True):

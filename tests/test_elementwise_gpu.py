@@ -312,13 +312,15 @@ def test_ltx_transformer_block_matches_oracle(dev):
     # the comparison cannot pass by both runs taking the same path.
     from q8_kernels_amd.modules import Attention
     impl, calls = _C().norm_mod_fht_quant, []
-    mm_impl, with_residual = _C().q8_mm_bias, []
+    mm_impl, with_residual, with_gate = _C().q8_mm_bias, [], []
     def counted(*a, **k):
         calls.append(1)
         return impl(*a, **k)
     def counted_mm(*a, **k):
         if k.get("residual") is not None:
             with_residual.append(1)
+        if k.get("gate") is not None:
+            with_gate.append(1)
         return mm_impl(*a, **k)
     run = lambda: blk(hidden.to(dev), (cos.to(dev), sin.to(dev)), None, text.to(dev), lens.to(dev),  # noqa: E731
                       timestep.to(dev), attn_type="q8_kernels")
@@ -327,17 +329,63 @@ def test_ltx_transformer_block_matches_oracle(dev):
         with torch.no_grad():
             again = run()
         assert len(calls) == 2, f"fused prologue ran {len(calls)} times, expected 2 (attn1 and feed-forward)"
-        assert len(with_residual) == 1, f"{len(with_residual)} GEMMs carried a residual, expected 1 (attn2's output projection)"
+        assert len(with_residual) == 3, f"{len(with_residual)} GEMMs carried a residual, expected 3 (the output projections of attn1 and attn2, the feed-forward's down projection)"
+        assert len(with_gate) == 2, f"{len(with_gate)} GEMMs carried a gate, expected 2 (attn1 and the feed-forward)"
         LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = False
         with torch.no_grad():
             seq = run()
         assert len(calls) == 2, "the operator-by-operator path called the fused prologue"
-        assert len(with_residual) == 1, "the operator-by-operator path added a residual inside a GEMM"
+        assert len(with_residual) == 3 and len(with_gate) == 2, "the operator-by-operator path added a residual inside a GEMM"
     finally:
         _C().norm_mod_fht_quant, _C().q8_mm_bias = impl, mm_impl
         LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = True
     assert_bit_equal(got, again, "fused block, second run")
     assert_bit_equal(got, seq, "fused block vs operator sequence")
+
+
+def test_ltx_block_gated_residuals_in_the_gemm_epilogue(dev):
+    """768 tokens per batch element at dim 512: the two gated residuals of the block run inside the persistent GEMM's
+    epilogue (asserted through the record of the kernel that ran). The block gives the bits of the operator-by-operator
+    sequence, whose gated residuals are separate fused multiply-add kernels."""
+    import torch.nn as nn
+    from q8_kernels_amd import _lib
+    from q8_kernels_amd.blocks import LTXTransformerBlock
+    from q8_kernels_amd.modules import Attention, Q8Linear
+    torch.manual_seed(53)
+    dim, heads, hd, kv_dim, s_tok, s_txt = 512, 8, 64, 256, 768, 40
+    blk = LTXTransformerBlock(dim, heads, hd, kv_dim, bias=True, use_rope=True, norm_affine=False).to(dev)
+    for name, m in blk.named_modules():
+        if isinstance(m, Q8Linear):
+            q = Q8Linear.from_linear(nn.Linear(m.in_features, m.out_features).to(dev).to(BF16))
+            m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    g = torch.Generator().manual_seed(54)
+    hidden = torch.randn(2, s_tok, dim, generator=g).to(BF16).to(dev)
+    text = torch.randn(2, s_txt, kv_dim, generator=g).to(BF16).to(dev)
+    timestep = (torch.randn(2, 1, 6 * dim, generator=g) * 0.3).to(dev)
+    grid = torch.stack(torch.meshgrid(torch.arange(8), torch.arange(8), torch.arange(12), indexing="ij")).reshape(3, -1)
+    cos, sin = (t.to(dev) for t in O.ref_freqs_cis(grid[None].float().repeat(2, 1, 1), dim))
+    lens = torch.tensor([40, 17], dtype=torch.int32).to(dev)
+    mm_impl, kernels = _C().q8_mm_bias, []
+    def recording_mm(*a, **k):
+        out = mm_impl(*a, **k)
+        if k.get("gate") is not None:
+            kernels.append(_lib.lib().q8_gemm_last_kernel())
+        return out
+    run = lambda: blk(hidden, (cos, sin), None, text, lens, timestep, attn_type="q8_kernels")  # noqa: E731
+    try:
+        _C().q8_mm_bias = recording_mm
+        with torch.no_grad():
+            fused = run()
+        assert len(kernels) == 2 and all(kk & _lib.Q8_GEMM_KERNEL_RESIDUAL for kk in kernels), kernels
+        LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = False
+        with torch.no_grad():
+            seq = run()
+        assert len(kernels) == 2, "the operator-by-operator path passed a gate into a GEMM"
+    finally:
+        _C().q8_mm_bias = mm_impl
+        LTXTransformerBlock.fuse_prologue = Attention.fuse_prologue = True
+    assert torch.isfinite(fused.float()).all()
+    assert_bit_equal(fused, seq, "block with gated epilogues vs operator sequence")
 
 
 @pytest.mark.parametrize("dim", [256, 1000, 2048, 8192])

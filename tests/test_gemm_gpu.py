@@ -256,6 +256,44 @@ def test_residual_in_epilogue_equals_separate_addition(dev, case, fuse_gelu, til
     assert_bit_equal(fused, plain + res, "residual epilogue")
 
 
+@pytest.mark.parametrize("case", [(2, 1536, 768, 384), (3, 768, 2304, 640), (1, 2304, 520, 512), (2, 100, 264, 384)])
+@pytest.mark.parametrize("in_dtype", ["int8", "fp8"])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+@pytest.mark.parametrize("tile_rows", [43, 44], ids=["rows192", "rows256"])
+def test_gated_residual_in_epilogue_equals_the_fused_multiply_add(dev, case, in_dtype, fuse_gelu, tile_rows):
+    """out = linear(a) * gate + residual with one gate row per batch element (the AdaLN block's gated residual): the
+    epilogue form (tokens per batch element a multiple of 768: a tile never meets two gate rows) and the fallback (last
+    case) both give the bits of the bf16 GEMM followed by the fused multiply-add kernel. 3-D activations [B, T, K]."""
+    bsz, t, n, k = case
+    g = torch.Generator().manual_seed(bsz * 7 + t + n)
+    if in_dtype == "int8":
+        a, b = _rand_i8(g, bsz, t, k).to(dev), _rand_i8(g, n, k).to(dev)
+        sa = (torch.rand(bsz * t, generator=g) * 2e-3 + 1e-4).to(dev)
+        mm = _C().q8_mm_bias
+    else:
+        a, b = O.e4m3_c10(torch.randn(bsz, t, k, generator=g)).to(dev), O.e4m3_c10(torch.randn(n, k, generator=g)).to(dev)
+        sa = (torch.rand(bsz * t, generator=g) * 2e-1 + 1e-2).to(dev)
+        mm = _C().fp8_mm_bias
+    sb = (torch.rand(n, generator=g) * 2e-2 + 1e-3).to(dev)
+    bias = torch.randn(n, generator=g).to(dev)
+    res = torch.randn(bsz, t, n, generator=g).to(torch.bfloat16).to(dev)
+    gate = (torch.randn(bsz, 1, n, generator=g) * 0.7).to(torch.bfloat16).to(dev)
+    gate[0, 0, :8] = 0  # a closed gate passes the residual through
+    _set_cfg(4)
+    _set_cfg(tile_rows)
+    try:
+        plain = mm(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16)
+        fused = mm(a, b, bias, sa, sb, fuse_gelu, torch.bfloat16, residual=res, gate=gate)
+        if t % 768 == 0:
+            assert _last_kernel() == ({43: K_PERSIST192, 44: K_PERSIST256}[tile_rows] | K_RESIDUAL)
+    finally:
+        _set_cfg(40)
+        _set_cfg(0)
+    want = _C().fma_8bit(plain, gate, res)
+    assert_bit_equal(fused, want, "gated residual epilogue")
+    assert torch.equal(fused[0, :, :8], res[0, :, :8])
+
+
 # ------------------------------------------------------------------ fp8 at the benchmark shapes
 
 @pytest.mark.parametrize("m", [2048, 6144])
