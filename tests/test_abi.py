@@ -119,6 +119,13 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     assert L.q8_gemm_residual(16, 16, None, 16, 16, None, 16, 1, 1, 8, 8, 384, I8, 0, None) == -1
     assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 8, 256, I8, 0, None) == -3     # K must exceed 256
     assert L.q8_gemm_residual(16, 16, None, 16, 16, 16, 16, 1, 1, 8, 12, 384, I8, 0, None) == -3    # N % 8
+    # q8_gemm_gated_residual(A, B, bias, sa, sb, residual, gate, rows_per_gate, C, M, N, K, in_dtype, fuse_gelu, stream)
+    assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, None, 768, 16, 1536, 8, 384, I8, 0, None) == -1    # no gate
+    assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 16, 100, 16, 1536, 8, 384, I8, 0, None) == -3      # rows per gate % 768
+    assert b"768" in L.q8_last_error()
+    assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 8, 768, 16, 1536, 8, 384, I8, 0, None) == -4       # gate alignment
+    assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 16, 768, 16, 1536, 8, 256, I8, 0, None) == -3      # K must exceed 256
+    assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 16, 768, 16, 0, 8, 384, I8, 0, None) == 0          # no rows
     assert L.q8_gemm_set_config(7) == -6
     assert L.q8_attn_set_config(5) == -6 and L.q8_attn_set_config(-1) == -6
     # q8_attn_fwd(q, k, v, o, kv_len, sq, sk, sv, B, H, M, N, D, v_layout, v_row_stride, scale, out_dtype, flags, stream)
