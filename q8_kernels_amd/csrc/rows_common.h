@@ -3,10 +3,11 @@
 //
 // Row mapping: a row of `dim` elements is padded to N = 8 * LANES * CH (a power of two). LANES consecutive
 // threads own a row, thread t of the row holds the elements (c * LANES + t) * 8 + 0..7 for c = 0..CH-1, i.e.
-// one 128-bit bf16 load per chunk. A block is 256 threads = 256 / LANES rows. Element-index bits therefore
-// map, low to high, to (register index, lane, wave, chunk), which is also the order in which the Hadamard
-// butterflies run, so that every output is produced by the same sequence of fp32 additions as the
-// ascending-stride butterfly network of the reference
+// one 128-bit bf16 load per chunk; t is the thread's index in the row, or in the kernels that run a Hadamard
+// transform a permutation of it inside groups of 16 lanes (row_thread). A block is 256 threads = 256 / LANES rows.
+// Element-index bits therefore map, low to high, to (register index, thread, chunk), which is also the order in
+// which the Hadamard butterflies run, so that every output is produced by the same sequence of fp32 additions as
+// the ascending-stride butterfly network of the reference
 // (csrc/fast_hadamard/fast_hadamard_transform_cuda.cu:84-108).
 //
 // fp contraction is off in every file that includes this header: products and sums round separately, like
