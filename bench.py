@@ -190,6 +190,29 @@ def _extras_gemm(dev, steps, warmup, g, out):
         del gxq, gwq
 
 
+def _extras_library(dev, steps, warmup, g, out):
+    """Yardstick, not product: the vendor library's fp8 GEMM (hipBLASLt through torch._scaled_mm, row-wise scales, bf16
+    output, no bias, no activation) on the same operands, box and process as this repository's kernel with its fused
+    bias (+ GELU) epilogue."""
+    from q8_kernels_amd import _C
+    for (mm, nn, kk) in ((6144, 8192, 2048), (8192, 8192, 8192), (12288, 2048, 8192), (12288, 2048, 2048)):
+        _, _, gb, gxq, gsx, gwq, gsw = _gemm_inputs(dev, mm, nn, kk, seed=3)
+        gb = gb.to(dev)
+        flop = 2.0 * mm * nn * kk
+        entry = {}
+        try:
+            sa2, sb2, wt = gsx.view(-1, 1), gsw.view(1, -1), gwq.t()
+            t, _ = _time(lambda: torch._scaled_mm(gxq, wt, scale_a=sa2, scale_b=sb2, out_dtype=torch.bfloat16), steps, warmup)
+            entry["library_scaled_mm"] = {"ms": t * 1e3, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS}
+        except Exception as e:  # the yardstick is optional: an unsupported call must not take the bench line down
+            entry["library_scaled_mm"] = {"error": "%s: %s" % (type(e).__name__, str(e)[:200])}
+        for name, gelu in (("this_kernel_bias", False), ("this_kernel_bias_gelu", True)):
+            t, _ = _time(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, gelu, torch.bfloat16), steps, warmup)
+            entry[name] = {"ms": t * 1e3, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS}
+        out["library_yardstick_fp8_gemm_%dx%dx%d" % (mm, nn, kk)] = entry
+        del gxq, gwq
+
+
 def _extras_rows(dev, steps, warmup, g, out):
     from q8_kernels_amd import _C
     # row kernels on [12288, 2048] tokens
@@ -253,11 +276,12 @@ def _extras_blocks(dev, steps, warmup, g, out):
                                          "shape": "tokens [2,6144,2048], text [2,128,2048], int8 linears, fp8 attention"}
 
 
-EXTRA_GROUPS = {"attn": _extras_attn, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks}
+EXTRA_GROUPS = {"attn": _extras_attn, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks,
+                "library": _extras_library}
 
 
 def _extras(dev, steps, warmup, only=None):
-    """The other workloads of the metric. `only` (group names out of attn, gemm, rows, blocks) restricts the run to those
+    """The other workloads of the metric. `only` (group names out of attn, gemm, rows, blocks, library) restricts the run to those
     groups, e.g. for a counter-collection run of one kernel."""
     out = {}
     for name, fn in EXTRA_GROUPS.items():
@@ -272,7 +296,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
-    ap.add_argument("--only", default=None, help="comma-separated groups of the other workloads to run (attn, gemm, rows, blocks)")
+    ap.add_argument("--only", default=None, help="comma-separated groups of the other workloads to run (attn, gemm, rows, blocks, library)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 512 MiB (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
