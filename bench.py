@@ -211,6 +211,27 @@ def _extras_library(dev, steps, warmup, g, out):
             entry[name] = {"ms": t * 1e3, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS}
         out["library_yardstick_fp8_gemm_%dx%dx%d" % (mm, nn, kk)] = entry
         del gxq, gwq
+    # attention: the library's bf16 flash attention (torch scaled_dot_product_attention) at the shape of config 3, next to
+    # this repository's fp8 kernel on Hadamard-rotated e4m3 operands (direct casts and per-token scales)
+    B, H, S = 2, 32, 6144
+    flop = 4.0 * B * H * S * S * 64
+    a = _attn_inputs(dev, g, B, H, S)
+    q8, k8, vt, sq, sk, sv = a["scaled"]
+    qd, kd, _ = a["direct"]
+    entry = {}
+    try:
+        qb, kb, vb = (torch.randn(B, H, S, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+        t, _ = _time(lambda: torch.nn.functional.scaled_dot_product_attention(qb, kb, vb), steps, warmup)
+        entry["library_sdpa_bf16"] = {"ms": t * 1e3, "tflops": flop / t / 1e12}
+        del qb, kb, vb
+    except Exception as e:
+        entry["library_sdpa_bf16"] = {"error": "%s: %s" % (type(e).__name__, str(e)[:200])}
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16), steps, warmup)
+    entry["this_kernel_fp8_direct_casts"] = {"ms": t * 1e3, "tflops": flop / t / 1e12}
+    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk,
+                                            v_scales=sv), steps, warmup)
+    entry["this_kernel_fp8_per_token_scales"] = {"ms": t * 1e3, "tflops": flop / t / 1e12}
+    out["library_yardstick_attention_B2_H32_S6144_D64"] = entry
 
 
 def _extras_rows(dev, steps, warmup, g, out):
