@@ -32,6 +32,35 @@ def test_fht_quant_bit_exact(dev, dim, out_type):
         assert_bit_equal(scales, ws, "scales dim=%d rows=%d" % (dim, rows))
 
 
+@pytest.mark.parametrize("dim", [64, 2048, 8192, 1536])
+def test_fht_quant_rows_of_signed_zeros(dev, dim):
+    """Rows of zeros of both signs, bf16 and e4m3 inputs: codes (e4m3 keeps the sign of a zero), scales 0. The transform
+    carries signs differently from the sequential network and must still hand the quantizer the reference's zeros."""
+    g = torch.Generator().manual_seed(dim + 77)
+    rows = 21
+    xb = (torch.randn(rows, dim, generator=g) * 2).to(BF16)
+    neg = torch.tensor(-0.0, dtype=BF16)
+    xb[0] = neg
+    xb[3] = torch.where(torch.rand(dim, generator=g) < 0.5, neg, torch.tensor(0.0, dtype=BF16))
+    xb[7] = 0.0
+    xb[rows - 1] = neg
+    xb[rows - 1, dim // 3] = 0.0
+    x8 = O.e4m3_c10(xb.float())  # e4m3 input with the same zeros (code 0x80 for -0)
+    assert (x8.view(torch.uint8)[0] == 0x80).all()
+    for x, mids in ((xb, (BF16,)), (x8, (BF16, E4M3))):
+        for mid in mids:
+            for out_type in (E4M3, None):
+                kw = {} if mid == BF16 else {"mid_type": E4M3}
+                codes, scales = _C().fht_quant(x.to(dev), dim ** -0.5, out_type, **kw)
+                wc, ws = O.ref_quant(O.ref_fht(x, dim ** -0.5, mid), out_type)
+                what = "dim=%d in=%s mid=%s out=%s" % (dim, x.dtype, mid, out_type)
+                assert_bit_equal(codes, wc, "codes " + what)
+                assert_bit_equal(scales, ws, "scales " + what)
+    # the transform alone on the e4m3 input
+    got = _C().fast_hadamard_transform(x8.to(dev), dim ** -0.5, BF16)
+    assert_bit_equal(got, O.ref_fht(x8, dim ** -0.5, BF16), "fht of e4m3 zeros dim=%d" % dim)
+
+
 def test_fht_quant_fp8_input_and_unrounded_intermediate(dev):
     g = torch.Generator().manual_seed(5)
     x = O.e4m3_c10(torch.randn(3, 7, 256, generator=g) * 4)
