@@ -159,10 +159,19 @@ def _extras_attn(dev, steps, warmup, g, out):
     kx8 = _C.fast_hadamard_transform(kx, a["fold"], E4M3)
     vxt = vx.to(E4M3).view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
     t, _ = _time(lambda: _C.flash_attention(qd, kx8, vxt, 1.0, lens, out_dtype=torch.bfloat16), steps, warmup)
+    (kx8s, skx), (vx8s, svx) = _C.tokenwise_quant(_C.fast_hadamard_transform(kx, 0.125, torch.bfloat16), E4M3), _C.tokenwise_quant(vx, E4M3)
+    vxts = vx8s.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
+    t_scaled, _ = _time(lambda: _C.flash_attention(q8, kx8s, vxts, 0.125, lens, out_dtype=torch.bfloat16, q_scales=sq, k_scales=skx,
+                                                   v_scales=svx), steps, warmup)
     byts = B * H * (S * 64 + 2 * N * 64 + S * 64 * 2)
     out["attn_cross_fp8_masked"] = {"ms": t * 1e3, "gbs": byts / t / 1e9, "frac_of_hbm_peak": byts / t / 1e9 / HBM_PEAK_GBS,
                                     "tflops": 4.0 * B * H * S * N * 64 / t / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64",
                                     "valid_lengths": lens.tolist(), "kernel": "attn_short_kernel<bf16>"}
+    byts_s = byts + B * H * (S + 2 * N) * 4  # the per-token scales as well
+    out["attn_cross_fp8_masked_per_token_scales"] = {
+        "ms": t_scaled * 1e3, "gbs": byts_s / t_scaled / 1e9, "frac_of_hbm_peak": byts_s / t_scaled / 1e9 / HBM_PEAK_GBS,
+        "tflops": 4.0 * B * H * S * N * 64 / t_scaled / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64", "valid_lengths": lens.tolist(),
+        "kernel": "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>"}
 
 
 def _extras_gemm(dev, steps, warmup, g, out):

@@ -198,6 +198,39 @@ def test_attention_config4_cross_attention_mask(dev):
     assert cosine(out[:, hs].cpu(), plain) >= 0.998  # accuracy of the direct e4m3 casts, not of the kernel
 
 
+def test_attention_config4_cross_attention_mask_per_token_scales(dev):
+    """Config 4 with per-token e4m3 quantisation of Q, K (after the Hadamard rotation) and V: 6144 queries, 128 text keys,
+    valid lengths drawn from 16..128. The whole problem runs on the GPU; the oracle checks four (batch, head) pairs, and
+    masked keys and values have no influence at all."""
+    C = _C()
+    g = torch.Generator().manual_seed(44)
+    B, H, M, N = 2, 32, 6144, 128
+    q = torch.randn(B, H, M, 64, generator=g).to(torch.bfloat16)
+    k, v = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16) for _ in range(2))
+    lens = torch.randint(16, 129, (B,), generator=g, dtype=torch.int32)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    qr, kr = C.fast_hadamard_transform(qd, 0.125, torch.bfloat16), C.fast_hadamard_transform(kd, 0.125, torch.bfloat16)
+    (q8, sq), (k8, sk), (v8, sv) = C.tokenwise_quant(qr, E4M3), C.tokenwise_quant(kr, E4M3), C.tokenwise_quant(vd, E4M3)
+    vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
+    out = C.flash_attention(q8, k8, vt, 0.125, lens.to(dev), out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv)
+    assert out.shape == (B, H, M, 64)
+    for (b, h) in [(0, 0), (0, 21), (1, 7), (1, 31)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        oq, osq = O.ref_quant(O.ref_fht(q[sl], 0.125, torch.bfloat16), E4M3)
+        ok, osk = O.ref_quant(O.ref_fht(k[sl], 0.125, torch.bfloat16), E4M3)
+        ov, osv = O.ref_quant(v[sl], E4M3)
+        _check(out[sl], oq, ok, ov, 0.125, lens[b:b + 1], (osq, osk, osv), what="config 4 per token (b=%d,h=%d)" % (b, h))
+    k2, v2, sk2, sv2 = k8.clone().view(torch.uint8), v8.clone().view(torch.uint8), sk.clone(), sv.clone()
+    for b in range(B):
+        ln = int(lens[b])
+        k2[b, :, ln:], v2[b, :, ln:], sk2[b, :, ln:], sv2[b, :, ln:] = 0x55, 0x7E, 1e3, 1e3
+    vt2 = v2.transpose(2, 3).contiguous().view(E4M3)
+    out2 = C.flash_attention(q8, k2.view(E4M3), vt2, 0.125, lens.to(dev), out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk2,
+                             v_scales=sv2)
+    # (the common factor max_j sv_j runs over the valid keys only, so the masked scales must not show either)
+    assert torch.equal(out.cpu().view(torch.int16), out2.cpu().view(torch.int16))
+
+
 def test_attention_rejects_bad_arguments(dev):
     from q8_kernels_amd import Q8Error
     q, k, v = _inputs(1, 1, 1, 16, 16)
