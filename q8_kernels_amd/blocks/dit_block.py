@@ -30,7 +30,8 @@ class Fp8DiTBlock(nn.Module):
         mk = lambda i, o: FP8Linear(i, o, bias=True, device=device)  # noqa: E731
         self.to_qkv = mk(dim, 3 * dim)
         self.to_out = mk(dim, dim)
-        self.to_q2, self.to_k2, self.to_v2, self.to_out2 = mk(dim, dim), mk(text_dim, dim), mk(text_dim, dim), mk(dim, dim)
+        # the K and V projections of the text states share their input: one layer of 2 * dim outputs (K first), like to_qkv
+        self.to_q2, self.to_kv2, self.to_out2 = mk(dim, dim), mk(text_dim, 2 * dim), mk(dim, dim)
         self.ff_up, self.ff_down = mk(dim, ffn_dim), mk(ffn_dim, dim)
 
     @torch.no_grad()
@@ -69,8 +70,8 @@ class Fp8DiTBlock(nn.Module):
         a = Q8F.flash_attention.flash_attn_func(heads(q), heads(k), heads(v), None, None, True, out_dtype=bf16)
         hidden = hidden + lin(self.to_out, merge(a))
         n = self.norm2(hidden)
-        a = Q8F.flash_attention.flash_attn_func(heads(lin(self.to_q2, n)), heads(lin(self.to_k2, text)), heads(lin(self.to_v2, text)),
-                                                None, text_lens, True, out_dtype=bf16)
+        k2, v2 = lin(self.to_kv2, text).split(d, dim=-1)
+        a = Q8F.flash_attention.flash_attn_func(heads(lin(self.to_q2, n)), heads(k2), heads(v2), None, text_lens, True, out_dtype=bf16)
         hidden = hidden + lin(self.to_out2, merge(a))
         return hidden + lin(self.ff_down, lin(self.ff_up, self.norm3(hidden), True))
 
@@ -86,7 +87,8 @@ class Fp8DiTBlock(nn.Module):
         hidden = self._lin(self.to_out, a, residual=hidden)
         # cross-attention to the text states
         q2 = self._norm_lin(self.norm2, self.to_q2, hidden)
-        k2, v2 = self._lin(self.to_k2, text), self._lin(self.to_v2, text)
+        kv2 = self._lin(self.to_kv2, text)  # k and v are read in place, like q, k, v of the self-attention
+        k2, v2 = kv2[..., :d], kv2[..., d:]
         a = Q8F.fused.flash_attn_token_major(q2, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
                                              out_dtype=bf16)
         hidden = self._lin(self.to_out2, a, residual=hidden)

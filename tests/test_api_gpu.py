@@ -137,6 +137,7 @@ def test_dit_block_matches_oracle_block(dev):
     with torch.no_grad():
         got = blk(hidden.to(dev), text.to(dev), (cos.to(dev), sin.to(dev)), lens.to(dev))
     params = {n: (m.weight.data.cpu(), m.scales.data.cpu(), m.bias.data.cpu()) for n, m in blk.named_modules() if isinstance(m, FP8Linear)}
+    _split_kv(params)
     for n in ("norm1", "norm2", "norm3"):
         params[n] = getattr(blk, n).weight.data.cpu()
     want = O.ref_dit_block(hidden, text, (cos, sin), lens, params, heads, p_scale=256.0)  # the kernel's default P grid
@@ -344,6 +345,13 @@ def test_concurrent_threads_on_their_own_streams(dev):
 
 # ------------------------------------------------------------------ the DiT block at its real widths
 
+def _split_kv(params):
+    """the block keeps the text K and V projections as one layer (K rows first); the oracle names them separately"""
+    w, sc, b = params.pop("to_kv2")
+    d = w.shape[0] // 2
+    params["to_k2"], params["to_v2"] = (w[:d], sc[:d], b[:d]), (w[d:], sc[d:], b[d:])
+
+
 def _dit_case(dev, s_tok, s_txt, seed, grid_shape):
     from q8_kernels_amd.blocks import Fp8DiTBlock
     from q8_kernels_amd.functional.rope import precompute_freqs_cis, video_index_grid
@@ -367,6 +375,7 @@ def test_dit_block_real_widths_against_the_oracle(dev):
     with torch.no_grad():
         got = blk(hidden.to(dev), text.to(dev), (cos.to(dev), sin.to(dev)), lens.to(dev))
     params = {n: (m.weight.data.cpu(), m.scales.data.cpu(), m.bias.data.cpu()) for n, m in blk.named_modules() if isinstance(m, FP8Linear)}
+    _split_kv(params)
     for n in ("norm1", "norm2", "norm3"):
         params[n] = getattr(blk, n).weight.data.cpu()
     want = O.ref_dit_block(hidden, text, (cos, sin), lens, params, 32, p_scale=256.0)
