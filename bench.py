@@ -274,6 +274,23 @@ def _extras_rows(dev, steps, warmup, g, out):
     out["fht_quant_int8_fused_12288x8192"] = {"ms": t * 1e3, "gbs": xw.numel() * 3 / t / 1e9, "frac_of_hbm_peak": xw.numel() * 3 / t / 1e9 / HBM_PEAK_GBS}
 
 
+def _graph_replay_time(fn, steps, warmup):
+    """fn() captured once into a HIP graph (after two eager calls on the capture stream) and replayed: the block as a pure
+    sequence of kernel launches without the host-side work of the Python layer between them."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        keep = fn()
+    t, _ = _time(graph.replay, steps, warmup)
+    del keep, graph
+    return t
+
+
 def _extras_blocks(dev, steps, warmup, g, out):
     from q8_kernels_amd import _C
     from q8_kernels_amd.blocks import Fp8DiTBlock
@@ -287,6 +304,9 @@ def _extras_blocks(dev, steps, warmup, g, out):
     with torch.no_grad():
         t, _ = _time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
     out["dit_block"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12, "shape": "tokens [2,6144,2048], text [2,128,2048]"}
+    with torch.no_grad():
+        t = _graph_replay_time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
+    out["dit_block"]["ms_graph_replay"] = t * 1e3
     del blk
     # the reference's own block: AdaLN-modulated LTXTransformerBlock on int8 (Hadamard-rotated) Q8Linear layers
     from q8_kernels_amd.blocks import LTXTransformerBlock
@@ -304,6 +324,10 @@ def _extras_blocks(dev, steps, warmup, g, out):
                      max(3, steps // 4), max(1, warmup // 2))
     out["ltx_transformer_block_int8"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12,
                                          "shape": "tokens [2,6144,2048], text [2,128,2048], int8 linears, fp8 attention"}
+    with torch.no_grad():
+        t = _graph_replay_time(lambda: ltx(hidden, (cosf, sinf), None, text, lens, timestep, attn_type="q8_kernels"),
+                               max(3, steps // 4), max(1, warmup // 2))
+    out["ltx_transformer_block_int8"]["ms_graph_replay"] = t * 1e3
 
 
 EXTRA_GROUPS = {"attn": _extras_attn, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks,
