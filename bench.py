@@ -152,6 +152,12 @@ def _extras_attn(dev, steps, warmup, g, out):
     v_tok = vt.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)  # [B,H,S,64]: V as the fused prologue leaves it
     t, _ = _time(lambda: _C.flash_attention(qd, kd, v_tok, 1.0, None, out_dtype=torch.bfloat16, v_token_major=True), steps, warmup)
     out["attn_self_fp8_reference_casts_token_major_v"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, token-major V>")
+    # opt-in: the maximum trails the running maximum (fewer rescalings of O; the largest weight of a row is not exact)
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, lazy_max=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
+    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv,
+                                            lazy_max=True), steps, warmup)
+    out["attn_self_fp8_per_token_scales_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
     # cross-attention with a padding mask (config 4): HBM-bound
     N = 128
     kx, vx = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))

@@ -15,11 +15,17 @@
 //                 cast to e4m3, ARE the 32-byte B operand of that lane. For this the K rows are
 //                 placed in LDS in the order in which the S^T accumulator rows come out, such that
 //                 lane half h owns keys 32h .. 32h+31 of the tile in operand byte order.
-// Softmax runs in the log2 domain in fp32: p = exp2(s * c - m + 8), c = softmax_scale * log2(e); the row
-// sum accumulates the unrounded p while e4m3_sat(p) multiplies V (csrc/flash_attention/
+// Softmax runs in the log2 domain in fp32: p = exp2(s * c - m + 8), c = softmax_scale * log2(e), m the running row
+// maximum; the row sum accumulates the unrounded p while e4m3_sat(p) multiplies V (csrc/flash_attention/
 // flash_attention_cuda.cu:197-221,437). The factor 2^8 cancels in O / l; it places the row maximum at 256 so
 // that probabilities down to 2^-14 of the maximum stay in the normal range of e4m3 (with the reference's p <= 1
-// everything below 2^-10 is flushed to zero, which biases long, flat rows). Q8_ATTN_P_UNIT_RANGE restores p <= 1. Tiles that lie entirely beyond the valid KV length are
+// everything below 2^-10 is flushed to zero, which biases long, flat rows). Q8_ATTN_P_UNIT_RANGE restores p <= 1.
+// Q8_ATTN_LAZY_MAX lets m trail the running maximum: it is raised only when the running maximum exceeds it by more than
+// 3 (p = exp2(s * c - m + 5) <= 2^8 still), so the rescaling of O and l by 2^(m_old - m_new), which otherwise runs in every
+// tile that raises the maximum of one of the wave's 32 rows, is paid in the first tiles and hardly ever after. The same
+// error bound holds, but the largest weight of a row is no longer a power of two, i.e. no longer exact: on sharply
+// peaked rows the mean error grows by about two thirds, which is why it is not the default.
+// Tiles that lie entirely beyond the valid KV length are
 // skipped, the partial tile is masked with -inf (the reference walks backwards and needs -1e6 instead,
 // flash_attention_cuda_mask.cu:244).
 #include "q8_common.h"
@@ -39,7 +45,8 @@ struct AttnParams {
     int B, H, M, N;
     int64_t v_row_stride;  // V^T row stride in elements (>= N, multiple of 16); unused for token-major V
     float scale_log2;      // softmax_scale * log2(e)
-    float p_shift;         // probabilities are formed as 2^(x - max + p_shift)
+    float p_shift;         // probabilities are formed as 2^(x - m + p_shift), m = the row's reference maximum
+    float m_slack;         // m is raised to the running maximum once that exceeds it by more than m_slack (0: m is the running maximum)
     int flags;
 };
 
@@ -48,6 +55,7 @@ __device__ __attribute__((aligned(16))) const uint32_t g_attn_zero16[4] = {0, 0,
 constexpr int kKV = 64;         // keys per tile
 constexpr int kStage = 8192;    // K tile 4 KiB + V^T tile 4 KiB
 constexpr int kStages = 4;      // LDS ring: one tile being read, up to three in flight
+constexpr float kMaxSlack = 3.f;  // Q8_ATTN_LAZY_MAX: log2 units by which a row's running maximum may exceed its reference maximum
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -361,23 +369,27 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
             for (int e = 2; e < 32; e += 2) mx = fmaxf(fmaxf(mx, x[e]), x[e + 1]);
             mx = fmaxf(mx, lane_xor<32>(mx));
             const float c = sqc[qt];
-            const float m_new = fmaxf(m_run[qt], mx * c);
-            // rescale only when some row of the wave saw a new maximum (alpha is exactly 1 otherwise)
-            if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
-                const float alpha = fast_exp2(m_run[qt] - m_new);
+            // The reference maximum m of a row moves (and O, l are rescaled) only when the tile's maximum exceeds it by
+            // more than m_slack (0 unless Q8_ATTN_LAZY_MAX: the running maximum), so p <= 2^(p_shift + m_slack). Each
+            // row decides for itself (its result does not depend on the rows it shares a wave with); the wave skips
+            // the multiplications when no row moves.
+            const float mxc = mx * c;
+            const bool grow = mxc > m_run[qt] + p.m_slack;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+                const float alpha = grow ? fast_exp2(m_run[qt] - mxc) : 1.f;
+                m_run[qt] = grow ? mxc : m_run[qt];
                 l_run[qt] *= alpha;
 #pragma unroll
                 for (int d = 0; d < 2; ++d)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) o_acc[qt][d][e] *= alpha;
             }
-            m_run[qt] = m_new;
-            const float m_sub = m_new - exp_bias;
+            const float m_sub = m_run[qt] - exp_bias;
             float psum = 0.f;
             float pr[32];
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                pr[e] = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^p_shift: inside the e4m3 range
+                pr[e] = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^(p_shift + m_slack) = 2^8 or 1: inside the e4m3 range
                 psum += pr[e];
             }
             if constexpr (SCALED) {
@@ -521,7 +533,7 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
             }
             mx = fmaxf(mx, lane_xor<32>(mx));
             // (no valid key at all: everything below is skipped and the output is zero)
-            const float m_sub = mx * c - p.p_shift;
+            const float m_sub = mx * c - (p.p_shift + p.m_slack);  // the final maximum is known: no slack needed
             float psum = 0.f;
             v16f o_acc[2];
 #pragma unroll
@@ -590,7 +602,7 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (!q || !k || !v || !o) return fail(Q8_ERR_NULL, "q8_attn_fwd: null pointer");
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);
     if (out_dtype != Q8_BF16 && out_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "q8_attn_fwd: output dtype %d", out_dtype);
-    if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE | Q8_ATTN_O_TOKEN_MAJOR)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
+    if (flags & ~(Q8_ATTN_SUM_ROUNDED_P | Q8_ATTN_P_UNIT_RANGE | Q8_ATTN_O_TOKEN_MAJOR | Q8_ATTN_LAZY_MAX)) return fail(Q8_ERR_FLAGS, "q8_attn_fwd: flags 0x%x", flags);
     if (v_layout != Q8_V_DS && v_layout != Q8_V_SD) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V layout %d", v_layout);
     const bool vtok = v_layout == Q8_V_SD;
     if (!vtok && (v_row_stride < N || v_row_stride % 16 != 0))
@@ -599,9 +611,12 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     if (scaled && !(sq && sk && sv)) return fail(Q8_ERR_NULL, "q8_attn_fwd: sq, sk, sv must be given together");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(o) % 8))
         return fail(Q8_ERR_ALIGN, "q8_attn_fwd: q, k, v must be 16-byte and o 8-byte aligned");
+    if ((flags & Q8_ATTN_LAZY_MAX) && (flags & Q8_ATTN_P_UNIT_RANGE))
+        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: Q8_ATTN_LAZY_MAX needs the head room of the default probability range (not P_UNIT_RANGE)");
+    const float slack = (flags & Q8_ATTN_LAZY_MAX) ? kMaxSlack : 0.f;
     AttnParams p{static_cast<const uint8_t*>(q), static_cast<const uint8_t*>(k), static_cast<const uint8_t*>(v), o, kv_len, sq, sk, sv,
                  B, H, M, N, v_row_stride, softmax_scale * 1.44269504088896340736f,
-                 (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f, flags};
+                 (flags & Q8_ATTN_P_UNIT_RANGE) ? 0.f : 8.f - slack, slack, flags};
     if (!(softmax_scale > 0.f)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: softmax_scale must be positive");
     const int cfg = g_attn_cfg;
     if (vtok && cfg == 1)

@@ -33,7 +33,7 @@ def test_header_enums_match_python_constants():
     from q8_kernels_amd import _lib
     text = open(HEADER).read()
     for name in ("Q8_I8", "Q8_E4M3", "Q8_BF16", "Q8_F16", "Q8_F32", "Q8_QUANT_RNE", "Q8_QUANT_SCALE_DIV",
-                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR",
+                 "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR", "Q8_ATTN_LAZY_MAX",
                  "Q8_GEMM_KERNEL_PIPE256", "Q8_GEMM_KERNEL_TILE128", "Q8_GEMM_KERNEL_PERSIST256",
                  "Q8_GEMM_KERNEL_PERSIST192", "Q8_GEMM_KERNEL_RESIDUAL"):
         m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
@@ -131,6 +131,9 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     # q8_attn_fwd(q, k, v, o, kv_len, sq, sk, sv, B, H, M, N, D, v_layout, v_row_stride, scale, out_dtype, flags, stream)
     assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 2, 16, 0.125, B16, 0, None) == -3   # V layout 2
     assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, _lib.Q8_V_DS, 8, 0.125, B16, 0, None) == -3  # V^T stride
+    lazy_unit = _lib.Q8_ATTN_LAZY_MAX | _lib.Q8_ATTN_P_UNIT_RANGE   # the trailing maximum needs the head room above 2^5
+    assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 0, 16, 0.125, B16, lazy_unit, None) == -6
+    assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 0, 16, 0.125, B16, 16, None) == -6  # unknown flag
     assert L.q8_attn_set_config(1) == 0
     try:  # the 4 waves x 64 queries shape reads V^T only
         assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, _lib.Q8_V_SD, 0, 0.125, B16, 0, None) == -6

@@ -34,19 +34,20 @@ def _inputs(seed, b, h, m, n, std=1.0):
     return q, k, v
 
 
-def _check(got, q, k, v, scale, lens=None, sc=(None, None, None), what="", p_scale=256.0):
+def _check(got, q, k, v, scale, lens=None, sc=(None, None, None), what="", p_scale=256.0, p_floor=None):
     """Kernel output against float64 attention on the dequantised inputs.
     Rigorous part: P is rounded to e4m3 before it multiplies V: relative error <= 2^-4 per weight in the normal
     range, absolute error <= 2^-10 / p_scale below it, so |o - o_exact| <= 2^-4 W + (2^-10 / p_scale) U with
     W = sum_j p_ij |v_j| / l_i and U = sum_j |v_j| / l_i, plus the bf16 rounding of the output (2^-8 |o|).
     Statistical part: the rounding errors average out, cosine >= 0.999 and the mean error stays below half of
     the mean bound. Against the oracle that rounds P (relative to the final row maximum, the kernel rounds
-    relative to the running one) the distance is at most twice the bound."""
+    relative to the running one) the distance is at most twice the bound. p_floor: the smallest factor the kernel may
+    have scaled a probability by when that is not p_scale (lazy_max: 2^5 .. 2^8); it sets the subnormal term."""
     g = got.cpu().double()
     exact, wabs, uabs = O.ref_attention(q, k, v, scale, lens, *sc, round_p=False, return_weighted_abs=True)
     rounded = O.ref_attention(q, k, v, scale, lens, *sc, round_p=True, p_scale=p_scale)
     assert not torch.isnan(g).any(), what
-    bound = 2.0 ** -4 * 1.02 * wabs + 2.0 ** -10 / p_scale * uabs + 2.0 ** -8 * exact.abs() + 1e-6
+    bound = 2.0 ** -4 * 1.02 * wabs + 2.0 ** -10 / (p_floor or p_scale) * uabs + 2.0 ** -8 * exact.abs() + 1e-6
     e_exact, e_round = (g - exact).abs(), (g - rounded).abs()
     assert (e_exact <= bound).all(), "%s: max-abs vs exact %g exceeds the e4m3 rounding bound (worst ratio %g)" % (
         what, e_exact.max().item(), (e_exact / bound).max().item())
@@ -108,6 +109,36 @@ def test_attention_large_logits_and_scale(dev):
     for scale in (0.125, 0.02, 1.0):
         got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), scale, None, out_dtype=torch.bfloat16)
         _check(got, q, k, v, scale, what="scale=%g" % scale)
+
+
+@pytest.mark.parametrize("m,n,std", [(300, 640, 1.0), (96, 2000, 2.0), (257, 200, 1.0), (64, 4096, 0.5)])
+def test_attention_lazy_max(dev, attn_cfg, m, n, std):
+    """lazy_max=True: the maximum a row's probabilities are formed against trails the running maximum by at most 3 in log2
+    (p between 2^5 and 2^8 times the true softmax numerator): same rounding bound with the subnormal term of 2^5, masked
+    and per-token-scaled calls included; every workgroup shape gives the same bits (each row decides for itself)."""
+    from q8_kernels_amd import _lib
+    q, k, v = _inputs(m + n, 2, 2, m, n, std=std)
+    lens = torch.tensor([n, max(1, n // 3)], dtype=torch.int32)
+    run = lambda **kw: _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16, **kw)
+    got = run(lazy_max=True)
+    _check(got, q, k, v, 0.125, lens, what="lazy maximum m=%d n=%d" % (m, n), p_floor=32.0)
+    _lib.check(_lib.lib().q8_attn_set_config(0))
+    assert torch.equal(got.cpu().view(torch.int16), run(lazy_max=True).cpu().view(torch.int16))
+    with pytest.raises(RuntimeError, match="LAZY_MAX"):
+        run(lazy_max=True, p_unit_range=True)
+    g = torch.Generator().manual_seed(n)
+    sq, sk, sv = (torch.rand(2, 2, r, generator=g) + 0.5 for r in (m, n, n))
+    got_s = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16, lazy_max=True,
+                                 q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+    _check(got_s, q, k, v, 0.125, lens, (sq, sk, sv), what="lazy maximum, per-token scales", p_floor=32.0 * 0.5 / 1.5)
+
+
+def test_attention_lazy_max_short_sequences_unchanged(dev):
+    """N <= 128 with unit scales runs the register-resident kernel, which knows the final maximum: lazy_max changes nothing"""
+    q, k, v = _inputs(3, 2, 2, 200, 100)
+    a = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16)
+    b = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16, lazy_max=True)
+    assert torch.equal(a.cpu().view(torch.int16), b.cpu().view(torch.int16))
 
 
 def test_attention_reference_probability_range(dev):
