@@ -60,6 +60,23 @@ def _time(fn, steps, warmup, ramp=0.15):
     return start.elapsed_time(stop) * 1e-3 / steps, wall
 
 
+def _time_cold(make, copies, steps, warmup):
+    """Like _time, with every call on a buffer set of its own: make(i) returns the call on the i-th copy of the inputs, the
+    results of the last `copies` calls stay allocated (so the allocator hands out other memory for the next ones), and the
+    calls go round the copies. With the copies adding up to several times the L2s (8 x 4 MB) and the memory-side cache
+    (256 MB), no call finds any of its data left behind by an earlier one: the time of a pass through HBM proper."""
+    fns = [make(i) for i in range(copies)]
+    ring, pos = [None] * copies, [0]
+
+    def fn():
+        i = pos[0] % copies
+        ring[i] = fns[i]()
+        pos[0] += 1
+    t, _ = _time(fn, steps, warmup)
+    del ring, fns
+    return t
+
+
 def _gemm_inputs(dev, m, n, k, seed=0):
     from q8_kernels_amd import _C
     g = torch.Generator().manual_seed(seed)
@@ -273,6 +290,30 @@ def _extras_rows(dev, steps, warmup, g, out):
                           ("attn_prep_qkv_rope_fht_fp8", lambda: _C.attn_prep_qkv(xs, xs, xs, 32, cs3, sn3, True, 0.125), 17)):
         t, _ = _time(fn, steps, warmup)
         out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    # the same kernels with nothing left in any cache by the previous call (16 sets of inputs and outputs, 1.2-5 GB)
+    copies = 16
+    xc = [x.clone() for _ in range(copies)]
+    for name, make, bpe in (("quant_fp8", lambda i: (lambda: _C.tokenwise_quant(xc[i], E4M3)), 3),
+                            ("quant_int8", lambda i: (lambda: _C.tokenwise_quant(xc[i], None)), 3),
+                            ("fht_bf16", lambda i: (lambda: _C.fast_hadamard_transform(xc[i], 2048 ** -0.5, None)), 4),
+                            ("rmsnorm_bf16", lambda i: (lambda: _C.rms_norm(xc[i], w, None)), 4),
+                            ("fht_quant_int8_fused", lambda i: (lambda: _C.fht_quant(xc[i], 2048 ** -0.5, None)), 3),
+                            ("rmsnorm_quant_fp8_fused", lambda i: (lambda: _C.rms_norm_quant(xc[i], w, E4M3)), 3)):
+        t = _time_cold(make, copies, steps, warmup)
+        out.setdefault(name, {}).update({"ms_cold": t * 1e3, "gbs_cold": n * bpe / t / 1e9, "frac_of_hbm_peak_cold": n * bpe / t / 1e9 / HBM_PEAK_GBS})
+    # yardstick: the library's plain copy of the same tensor (2 B in, 2 B out), warm and cold
+    t, _ = _time(lambda: x.clone(), steps, warmup)
+    out["library_copy_bf16_yardstick"] = {"ms": t * 1e3, "gbs": n * 4 / t / 1e9, "frac_of_hbm_peak": n * 4 / t / 1e9 / HBM_PEAK_GBS}
+    t = _time_cold(lambda i: (lambda: xc[i].clone()), copies, steps, warmup)
+    out["library_copy_bf16_yardstick"].update({"ms_cold": t * 1e3, "gbs_cold": n * 4 / t / 1e9, "frac_of_hbm_peak_cold": n * 4 / t / 1e9 / HBM_PEAK_GBS})
+    cc, sc = [cos.clone() for _ in range(copies)], [sin.clone() for _ in range(copies)]
+    for name, make, bpe in (("rope_bf16", lambda i: (lambda: _C.rope(xc[i], cc[i], sc[i], None)), 12),
+                            ("attn_prep_qkv_rope_fht_fp8", lambda i: (lambda: _C.attn_prep_qkv(
+                                xc[i].view(2, 6144, 2048), xc[(i + 5) % copies].view(2, 6144, 2048), xc[(i + 10) % copies].view(2, 6144, 2048), 32,
+                                cc[i].view(2, 6144, 2048), sc[i].view(2, 6144, 2048), True, 0.125)), 17)):
+        t = _time_cold(make, copies, steps, warmup)
+        out.setdefault(name, {}).update({"ms_cold": t * 1e3, "gbs_cold": n * bpe / t / 1e9, "frac_of_hbm_peak_cold": n * bpe / t / 1e9 / HBM_PEAK_GBS})
+    del cc, sc, xc
     del x, cos, sin
     # the Hadamard rotation + int8 quantizer over the 8192-wide FFN hidden of the int8 block
     xw = torch.randn(12288, 8192, generator=g).to(torch.bfloat16).to(dev)
