@@ -172,6 +172,11 @@ def _extras_attn(dev, steps, warmup, g, out):
     # opt-in: the maximum trails the running maximum (fewer rescalings of O; the largest weight of a row is not exact)
     t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, lazy_max=True), steps, warmup)
     out["attn_self_fp8_reference_casts_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
+    # opt-in: the row sum over the rounded probabilities, taken by the matrix pipe; alone and with the trailing maximum
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_sum_rounded_p"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>")
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True, lazy_max=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_sum_rounded_p_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>, Q8_ATTN_LAZY_MAX")
     t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv,
                                             lazy_max=True), steps, warmup)
     out["attn_self_fp8_per_token_scales_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>, Q8_ATTN_LAZY_MAX")

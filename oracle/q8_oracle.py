@@ -240,7 +240,7 @@ def ref_fp8_linear(a, b, bias=None, scale_a=None, scale_b=None, use_hadamard=Fal
 def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                   kv_len: Optional[torch.Tensor] = None, sq=None, sk=None, sv=None,
                   round_p: bool = True, out_dtype: Optional[torch.dtype] = None, return_weighted_abs: bool = False,
-                  p_scale: float = 1.0):
+                  p_scale: float = 1.0, sum_rounded: bool = False):
     """Attention on e4m3 operands as the reference kernel defines it (csrc/flash_attention/
     flash_attention_cuda.cu:171-248,437,487-497; mask: flash_attention_cuda_mask.cu:244,319):
         s_ij = (q_i . k_j) * scale (* sq_i sk_j);  keys j >= kv_len[b] masked;
@@ -254,6 +254,8 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
     p_scale: the probabilities are rounded as e4m3_sat(p_scale * p). The default 1 is the reference (weights below
     2^-10 flush to zero); the HIP kernel's own default is 2^8, which cancels in o / l, and the tests of that default
     pass p_scale=256 explicitly.
+    sum_rounded (unit scales only): l_i sums the ROUNDED probabilities, the ones that multiply V, so that o_i is a true
+    convex combination of the v_j (the HIP kernel's Q8_ATTN_SUM_ROUNDED_P; the reference sums the unrounded ones).
     The online kernel rounds p against the running maximum, so its P-hat differs from this one in the
     last e4m3 bit here and there: comparisons carry a tolerance. With return_weighted_abs the function also
     returns W = sum_j p_ij |v_j| / l_i and U = sum_j |v_j| / l_i: rounding every weight with relative error eps
@@ -280,6 +282,10 @@ def ref_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sca
         pv = p * (svd / torch.where(sv_ref > 0, sv_ref, torch.ones_like(sv_ref))).unsqueeze(-2)
     if round_p:
         pv = e4m3_sat((pv * p_scale).to(torch.float32)).to(torch.float64) / p_scale
+    if sum_rounded:
+        if sv is not None or not round_p:
+            raise ValueError("sum_rounded is defined for rounded probabilities without per-token scales")
+        l = pv.sum(dim=-1, keepdim=True)
     o = pv @ vd
     if sv_ref is not None:
         o = o * sv_ref.unsqueeze(-1)

@@ -296,7 +296,9 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
     v_token_major=True takes v as [B,H,N,64] (k's layout): the kernel turns the tiles itself, no transposed copy;
     lazy_max=True lets the maximum the probabilities are formed against trail the running maximum by up to a factor 8
     (fewer rescalings of the accumulators: about 5 % faster on long sequences, the largest weight of a row no longer
-    exact; not with p_unit_range).
+    exact; not with p_unit_range); sum_rounded_p=True normalises by the sum of the rounded probabilities (the ones that
+    multiply v), taken on the matrix pipe: outputs are convex combinations of v's rows, about 6 % faster on long
+    sequences, unit scales only.
     """
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
         _check_input(t, name)

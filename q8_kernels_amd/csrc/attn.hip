@@ -98,9 +98,18 @@ __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, con
 }
 
 // kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
-// VTOK: V is token-major ([B,H,N,64])
-template <int OUT, bool SCALED, int kQT, int kWaves, bool VTOK = false>
+// VTOK: V is token-major ([B,H,N,64]).
+// MSUM (Q8_ATTN_SUM_ROUNDED_P; unit scales, kQT = 1): the row sum is taken over the e4m3-rounded probabilities, by the
+// matrix pipe: one v_mfma_f32_16x16x128_f8f6f4 per tile multiplies the P^T operand by a 16 x 128 matrix of ones and zeros.
+// In that instruction lane l of an operand holds 32 of the 128 reduction indices (block g = l / 16) of row or column
+// l % 16, and result register 0 of lane l is D[4 (l / 16)][l % 16]. P^T, laid out for the 32 x 32 product, puts query
+// (l % 32), key half (l / 32) into lane l: column n of the 16 x 128 view meets query n in blocks 0 and 2 and query n + 16
+// in blocks 1 and 3. With rows 0, 8 = ones on blocks {0, 2} and rows 4, 12 = ones on blocks {1, 3}, register 0 of EVERY
+// lane receives the complete row sum (both key halves) of that lane's own query: no cross-lane step, and the 32
+// additions per tile of the vector ALU are gone.
+template <int OUT, bool SCALED, int kQT, int kWaves, bool VTOK = false, bool MSUM = false>
 __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 3 : 1) void attn_fwd_kernel(const AttnParams p) {
+    static_assert(!MSUM || (!SCALED && kQT == 1), "the matrix-pipe row sum is built for unit scales and one query tile per wave");
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
     __shared__ __attribute__((aligned(256))) float lds_sc[SCALED ? kStages * 128 : 4];  // per stage: sk[64], sv[64]
@@ -214,6 +223,15 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
     float m_run[kQT], l_run[kQT];
 #pragma unroll
     for (int t = 0; t < kQT; ++t) { m_run[t] = -INFINITY; l_run[t] = 0.f; }
+    v4f l_acc = {0.f, 0.f, 0.f, 0.f};  // MSUM: [0] = row sum of this lane's query
+    v8i ones;                          // MSUM: this lane's 32 bytes of the ones-and-zeros matrix (e4m3 1.0 = 0x38)
+    {
+        const int mrow = lane & 15, blk = lane >> 4;
+        const int on = ((mrow & 3) == 0 && ((mrow >> 2) & 1) == (blk & 1)) ? 0x38383838 : 0;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) ones[w] = on;
+    }
+    (void)l_acc; (void)ones;
 
     const int n_tiles = (valid + kKV - 1) / kKV;
 
@@ -378,7 +396,7 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
             if (__builtin_amdgcn_ballot_w64(grow) != 0) {
                 const float alpha = grow ? fast_exp2(m_run[qt] - mxc) : 1.f;
                 m_run[qt] = grow ? mxc : m_run[qt];
-                l_run[qt] *= alpha;
+                if constexpr (MSUM) l_acc[0] *= alpha; else l_run[qt] *= alpha;
 #pragma unroll
                 for (int d = 0; d < 2; ++d)
 #pragma unroll
@@ -390,7 +408,7 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
                 pr[e] = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^(p_shift + m_slack) = 2^8 or 1: inside the e4m3 range
-                psum += pr[e];
+                if constexpr (!MSUM) psum += pr[e];
             }
             if constexpr (SCALED) {
                 if (qt == 0) {
@@ -412,14 +430,8 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
                 u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
                 pf[w] = (int)u;
             }
-            if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {
-                psum = 0.f;
-#pragma unroll
-                for (int w = 0; w < 8; ++w) {
-                    psum += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
-                }
-            }
-            l_run[qt] += psum;
+            if constexpr (MSUM) l_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pf, l_acc, 0, 0, 0, 0, 0, 0);
+            else l_run[qt] += psum;
 #pragma unroll
             for (int d = 0; d < 2; ++d)
                 o_acc[qt][d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[d], pf, o_acc[qt][d], 0, 0, 0, 0, 0, 0);
@@ -432,7 +444,7 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
 #pragma unroll
     for (int qt = 0; qt < kQT; ++qt) {
         const int row = q0 + 32 * qt + ql;
-        float l = l_run[qt] + lane_xor<32>(l_run[qt]);
+        const float l = MSUM ? l_acc[0] : l_run[qt] + lane_xor<32>(l_run[qt]);
         const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
         store_o_tile<OUT>(p.o, o_base + (size_t)row * o_rs, h, o_acc[qt], inv, row < M);
     }
@@ -534,7 +546,7 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
             mx = fmaxf(mx, lane_xor<32>(mx));
             // (no valid key at all: everything below is skipped and the output is zero)
             const float m_sub = mx * c - (p.p_shift + p.m_slack);  // the final maximum is known: no slack needed
-            float psum = 0.f;
+            float psum = 0.f, psum_rounded = 0.f;
             v16f o_acc[2];
 #pragma unroll
             for (int d = 0; d < 2; ++d)
@@ -556,12 +568,10 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
                         u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
                         pf[w] = (int)u;
                     }
-                    if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {
-#pragma unroll
-                        for (int e = 0; e < 32; ++e) psum -= pr[e];
+                    if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {  // this kernel waits for HBM: the vector ALU has the time
 #pragma unroll
                         for (int w = 0; w < 8; ++w)
-                            psum += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
+                            psum_rounded += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
                     }
 #pragma unroll
                     for (int d = 0; d < 2; ++d)
@@ -570,6 +580,7 @@ __global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int
             }
             // ---- O^T lane (q, h), tile d, register e holds dim 32 d + 8 (e/4) + 4 h + (e%4)
             const int row = 32 * tile + ql;
+            if (p.flags & Q8_ATTN_SUM_ROUNDED_P) psum = psum_rounded;
             const float l = psum + lane_xor<32>(psum);
             const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
             store_o_tile<OUT>(p.o, o_base + (size_t)row * o_rs, h, o_acc, inv, row < M);
@@ -613,6 +624,8 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
         return fail(Q8_ERR_ALIGN, "q8_attn_fwd: q, k, v must be 16-byte and o 8-byte aligned");
     if ((flags & Q8_ATTN_LAZY_MAX) && (flags & Q8_ATTN_P_UNIT_RANGE))
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: Q8_ATTN_LAZY_MAX needs the head room of the default probability range (not P_UNIT_RANGE)");
+    if ((flags & Q8_ATTN_SUM_ROUNDED_P) && scaled)
+        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: Q8_ATTN_SUM_ROUNDED_P is defined for unit scales only (with per-token scales P carries V's scales)");
     const float slack = (flags & Q8_ATTN_LAZY_MAX) ? kMaxSlack : 0.f;
     AttnParams p{static_cast<const uint8_t*>(q), static_cast<const uint8_t*>(k), static_cast<const uint8_t*>(v), o, kv_len, sq, sk, sv,
                  B, H, M, N, v_row_stride, softmax_scale * 1.44269504088896340736f,
@@ -621,6 +634,9 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     const int cfg = g_attn_cfg;
     if (vtok && cfg == 1)
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape reads V^T only (Q8_V_DS)");
+    const bool msum = (flags & Q8_ATTN_SUM_ROUNDED_P) != 0;
+    if (msum && cfg == 1)
+        return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape has no Q8_ATTN_SUM_ROUNDED_P form");
     if (N <= 128 && !scaled && cfg != 3 && !vtok) {
         // K and V^T stay in registers; enough waves to fill the device, each walking over several query tiles
         // (tiles per wave and batch: about 2048 waves in all, one 8-wave workgroup per CU)
@@ -639,22 +655,25 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     // 4 waves x 32 queries then place three workgroups on a CU (3 waves per SIMD) where the 8-wave shape places one.
     const int waves = (cfg == 1 || cfg == 2) ? 4 : (cfg == 4 ? 8 : (scaled ? 4 : 8));
     const int qtiles = cfg == 1 ? 2 : 1;
-#define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV, VT)                                                                           \
-    hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV, VT>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
-                                                                      (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
-#define Q8_ATTN_CFG(OUTT, SC)                                                        \
-    if (qtiles == 2) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4, false);                           \
-    else if (waves == 4) {                                                            \
-        if (vtok) Q8_ATTN_LAUNCH(OUTT, SC, 1, 4, true); else Q8_ATTN_LAUNCH(OUTT, SC, 1, 4, false); \
-    } else {                                                                          \
-        if (vtok) Q8_ATTN_LAUNCH(OUTT, SC, 1, 8, true); else Q8_ATTN_LAUNCH(OUTT, SC, 1, 8, false); \
-    }
+#define Q8_ATTN_LAUNCH(OUTT, SC, QT, WV, VT, MS)                                                                           \
+    hipLaunchKernelGGL((attn_fwd_kernel<OUTT, SC, QT, WV, VT, MS>), dim3((unsigned)((M + WV * QT * 32 - 1) / (WV * QT * 32)), \
+                                                                          (unsigned)(B * H)), dim3(WV * 64), 0, stream, p)
+#define Q8_ATTN_VT(OUTT, SC, WV, MS) \
+    if (vtok) Q8_ATTN_LAUNCH(OUTT, SC, 1, WV, true, MS); else Q8_ATTN_LAUNCH(OUTT, SC, 1, WV, false, MS)
+#define Q8_ATTN_CFG(OUTT, SC)                                     \
+    if (qtiles == 2) Q8_ATTN_LAUNCH(OUTT, SC, 2, 4, false, false); \
+    else if (waves == 4) { Q8_ATTN_VT(OUTT, SC, 4, false); }       \
+    else { Q8_ATTN_VT(OUTT, SC, 8, false); }
+#define Q8_ATTN_MSUM(OUTT) \
+    if (waves == 4) { Q8_ATTN_VT(OUTT, false, 4, true); } else { Q8_ATTN_VT(OUTT, false, 8, true); }
     if (out_dtype == Q8_BF16) {
-        if (scaled) { Q8_ATTN_CFG(Q8_BF16, true) } else { Q8_ATTN_CFG(Q8_BF16, false) }
+        if (msum) { Q8_ATTN_MSUM(Q8_BF16) } else if (scaled) { Q8_ATTN_CFG(Q8_BF16, true) } else { Q8_ATTN_CFG(Q8_BF16, false) }
     } else {
-        if (scaled) { Q8_ATTN_CFG(Q8_E4M3, true) } else { Q8_ATTN_CFG(Q8_E4M3, false) }
+        if (msum) { Q8_ATTN_MSUM(Q8_E4M3) } else if (scaled) { Q8_ATTN_CFG(Q8_E4M3, true) } else { Q8_ATTN_CFG(Q8_E4M3, false) }
     }
+#undef Q8_ATTN_MSUM
 #undef Q8_ATTN_CFG
+#undef Q8_ATTN_VT
 #undef Q8_ATTN_LAUNCH
     return launch_status("q8_attn_fwd");
 }

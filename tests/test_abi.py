@@ -134,6 +134,9 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     lazy_unit = _lib.Q8_ATTN_LAZY_MAX | _lib.Q8_ATTN_P_UNIT_RANGE   # the trailing maximum needs the head room above 2^5
     assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 0, 16, 0.125, B16, lazy_unit, None) == -6
     assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 0, 16, 0.125, B16, 16, None) == -6  # unknown flag
+    # the row sum over rounded probabilities is defined for unit scales
+    assert L.q8_attn_fwd(16, 16, 16, 16, None, 16, 16, 16, 1, 1, 8, 8, 64, 0, 16, 0.125, B16, _lib.Q8_ATTN_SUM_ROUNDED_P, None) == -6
+    assert b"unit scales" in L.q8_last_error()
     assert L.q8_attn_set_config(1) == 0
     try:  # the 4 waves x 64 queries shape reads V^T only
         assert L.q8_attn_fwd(16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, _lib.Q8_V_SD, 0, 0.125, B16, 0, None) == -6

@@ -141,6 +141,64 @@ def test_attention_lazy_max_short_sequences_unchanged(dev):
     assert torch.equal(a.cpu().view(torch.int16), b.cpu().view(torch.int16))
 
 
+@pytest.mark.parametrize("cfg", [0, 2, 4])
+@pytest.mark.parametrize("m,n,std", [(300, 640, 1.0), (96, 2000, 2.0), (257, 200, 1.0), (200, 100, 1.0), (33, 17, 1.0)])
+def test_attention_sum_rounded_p(dev, cfg, m, n, std):
+    """sum_rounded_p=True: the row sum runs over the e4m3-rounded probabilities (on the matrix pipe in the general kernel),
+    so every output is a convex combination of the valid v_j: a V with equal rows comes back bit for bit, outputs stay
+    inside the per-channel range of V, the distance to exact attention obeys the bound of a 2^-4 perturbation of the
+    weights in numerator and denominator, the distance to the oracle with the same definition twice that; all workgroup
+    shapes, both V layouts and the combination with lazy_max; refused with per-token scales and the 4 x 64 shape."""
+    from q8_kernels_amd import _lib
+    q, k, v = _inputs(7 * m + n, 2, 2, m, n, std=std)
+    lens = torch.tensor([n, max(1, n // 3)], dtype=torch.int32)
+    C = _C()
+    _lib.check(_lib.lib().q8_attn_set_config(cfg))
+    try:
+        run = lambda vv, **kw: C.flash_attention(q.to(dev), k.to(dev), _vt(vv).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
+                                                 sum_rounded_p=True, **kw)
+        row = O.e4m3_c10(torch.randn(64, generator=torch.Generator().manual_seed(n)))
+        v_const = row.expand(2, 2, n, 64).contiguous()
+        for kw in ({}, {"lazy_max": True}):
+            got = run(v_const, **kw)
+            assert torch.equal(got.cpu(), row.to(torch.bfloat16).expand(2, 2, m, 64)), "equal rows of V must come back exactly %s" % kw
+        got = run(v)
+        got_tok = C.flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16, sum_rounded_p=True,
+                                    v_token_major=True)
+        if n > 128:  # (shorter sequences: V^T takes the register-resident kernel, token-major V the general one)
+            assert torch.equal(got.cpu().view(torch.int16), got_tok.cpu().view(torch.int16))
+        lazy = run(v, lazy_max=True)
+    finally:
+        _lib.check(_lib.lib().q8_attn_set_config(0))
+    assert torch.equal(got.cpu().view(torch.int16), run(v).cpu().view(torch.int16)), "config %d against the default shape" % cfg
+    g = got.cpu().double()
+    exact, wabs, uabs = O.ref_attention(q, k, v, 0.125, lens, round_p=False, return_weighted_abs=True)
+    same_def = O.ref_attention(q, k, v, 0.125, lens, p_scale=256.0, sum_rounded=True)
+    eps = 2.0 ** -4 * 1.02
+    for out, floor in ((g, 256.0), (got_tok.cpu().double(), 256.0), (lazy.cpu().double(), 32.0)):
+        sub = 2.0 ** -10 / floor
+        bound = (eps * wabs + sub * uabs + (eps + sub * n) * exact.abs()) / (1 - eps) + 2.0 ** -8 * exact.abs() + 1e-6
+        assert ((out - exact).abs() <= bound).all(), (out - exact).abs().max().item()
+        assert ((out - same_def).abs() <= 2 * bound).all()
+        assert cosine(out, exact) >= 0.999
+        for b in range(2):
+            vb = v[b, :, :int(lens[b])].double()
+            lo, hi = vb.amin(dim=1, keepdim=True), vb.amax(dim=1, keepdim=True)
+            tol = 2.0 ** -8 * torch.maximum(lo.abs(), hi.abs())   # bf16 rounding of the output
+            assert (out[b] >= lo - tol).all() and (out[b] <= hi + tol).all(), "outside the range of V"
+    sc = torch.ones(2, 2, max(m, n), device=dev)
+    with pytest.raises(RuntimeError, match="unit scales"):
+        C.flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16, sum_rounded_p=True,
+                          q_scales=sc[..., :m].contiguous(), k_scales=sc[..., :n].contiguous(), v_scales=sc[..., :n].contiguous())
+    if n > 128:
+        _lib.check(_lib.lib().q8_attn_set_config(1))
+        try:
+            with pytest.raises(RuntimeError, match="4 waves x 64"):
+                run(v)
+        finally:
+            _lib.check(_lib.lib().q8_attn_set_config(0))
+
+
 def test_attention_reference_probability_range(dev):
     """p_unit_range=True rounds the probabilities on the reference's grid (p <= 1): same checks with the larger
     subnormal term, and on a long flat row the default (2^8 p) is the more accurate of the two."""

@@ -290,6 +290,32 @@ def test_attention_rounded_p_invariants():
     assert torch.allclose(os_, want, atol=1e-10)
 
 
+def test_attention_sum_of_rounded_probabilities_is_a_convex_combination():
+    """sum_rounded=True normalises by the weights that multiply V: a V whose rows are all equal comes back exactly,
+    whatever the rounding did to the weights (the default, which sums the unrounded ones, does not), every output lies
+    inside the per-channel range of the valid v_j, and the distance to exact attention obeys the bound of a 2^-4
+    perturbation of the weights in numerator and denominator."""
+    g = torch.Generator().manual_seed(24)
+    q = O.e4m3_c10(torch.randn(1, 2, 33, 64, generator=g) * 2)
+    k = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g) * 2)
+    row = O.e4m3_c10(torch.randn(64, generator=g))
+    v_const = row.expand(1, 2, 70, 64).contiguous()
+    lens = torch.tensor([41], dtype=torch.int32)
+    o = O.ref_attention(q, k, v_const, 0.125, lens, sum_rounded=True)
+    assert torch.allclose(o, row.double().expand_as(o), rtol=1e-14, atol=0)
+    plain = O.ref_attention(q, k, v_const, 0.125, lens)
+    assert (plain - row.double()).abs().max() > 1e-4
+    v = O.e4m3_c10(torch.randn(1, 2, 70, 64, generator=g))
+    o = O.ref_attention(q, k, v, 0.125, lens, sum_rounded=True, p_scale=256.0)
+    lo, hi = v[:, :, :41].double().amin(dim=2, keepdim=True), v[:, :, :41].double().amax(dim=2, keepdim=True)
+    assert (o >= lo - 1e-12).all() and (o <= hi + 1e-12).all()
+    exact, wabs, uabs = O.ref_attention(q, k, v, 0.125, lens, round_p=False, return_weighted_abs=True)
+    eps = 2.0 ** -4
+    assert ((o - exact).abs() <= (eps * wabs + 2.0 ** -18 * uabs + eps * exact.abs()) / (1 - eps) + 1e-12).all()
+    with pytest.raises(ValueError):
+        O.ref_attention(q, k, v, 0.125, lens, torch.ones(1, 2, 33), torch.ones(1, 2, 70), torch.ones(1, 2, 70), sum_rounded=True)
+
+
 def test_flash_attn_func_hadamard_identity():
     """(Hq).(Hk)/D = q.k: with the rotation the result approximates plain attention on the bf16 inputs."""
     g = torch.Generator().manual_seed(23)
