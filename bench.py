@@ -169,17 +169,6 @@ def _extras_attn(dev, steps, warmup, g, out):
     v_tok = vt.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)  # [B,H,S,64]: V as the fused prologue leaves it
     t, _ = _time(lambda: _C.flash_attention(qd, kd, v_tok, 1.0, None, out_dtype=torch.bfloat16, v_token_major=True), steps, warmup)
     out["attn_self_fp8_reference_casts_token_major_v"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, token-major V>")
-    # opt-in: the maximum trails the running maximum (fewer rescalings of O; the largest weight of a row is not exact)
-    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, lazy_max=True), steps, warmup)
-    out["attn_self_fp8_reference_casts_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
-    # opt-in: the row sum over the rounded probabilities, taken by the matrix pipe; alone and with the trailing maximum
-    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True), steps, warmup)
-    out["attn_self_fp8_reference_casts_sum_rounded_p"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>")
-    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True, lazy_max=True), steps, warmup)
-    out["attn_self_fp8_reference_casts_sum_rounded_p_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>, Q8_ATTN_LAZY_MAX")
-    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv,
-                                            lazy_max=True), steps, warmup)
-    out["attn_self_fp8_per_token_scales_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
     # cross-attention with a padding mask (config 4): HBM-bound
     N = 128
     kx, vx = (torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
@@ -382,16 +371,44 @@ def _extras_blocks(dev, steps, warmup, g, out):
     out["ltx_transformer_block_int8"]["ms_graph_replay"] = t * 1e3
 
 
-EXTRA_GROUPS = {"attn": _extras_attn, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks,
+def _extras_attn_options(dev, steps, warmup, g, out):
+    """The opt-in forms of the self-attention kernel (flags of q8_attn_fwd that change the arithmetic within the stated
+    tolerance; off by default and not used by the modules). A group of its own because two of them run the same kernel
+    symbols as the default calls: a per-kernel profile of the defaults leaves this group out (--skip attn_options)."""
+    from q8_kernels_amd import _C
+    B, H, S = 2, 32, 6144
+    a = _attn_inputs(dev, g, B, H, S)
+    q8, k8, vt, sq, sk, sv = a["scaled"]
+    qd, kd, _ = a["direct"]
+    flop = 4.0 * B * H * S * S * 64
+
+    def entry(t, kernel):
+        return {"ms": t * 1e3, "tflops": flop / t / 1e12, "frac_of_fp8_peak": flop / t / 1e12 / FP8_PEAK_TFLOPS, "shape": "B2 H32 S6144 D64",
+                "kernel": kernel}
+
+    # opt-in: the maximum trails the running maximum (fewer rescalings of O; the largest weight of a row is not exact)
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, lazy_max=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
+    # opt-in: the row sum over the rounded probabilities, taken by the matrix pipe; alone and with the trailing maximum
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_sum_rounded_p"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>")
+    t, _ = _time(lambda: _C.flash_attention(qd, kd, vt, 1.0, None, out_dtype=torch.bfloat16, sum_rounded_p=True, lazy_max=True), steps, warmup)
+    out["attn_self_fp8_reference_casts_sum_rounded_p_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, unit scales, 8 waves x 32 queries, row sum by MFMA>, Q8_ATTN_LAZY_MAX")
+    t, _ = _time(lambda: _C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv,
+                                            lazy_max=True), steps, warmup)
+    out["attn_self_fp8_per_token_scales_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
+
+
+EXTRA_GROUPS = {"attn": _extras_attn, "attn_options": _extras_attn_options, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks,
                 "library": _extras_library}
 
 
-def _extras(dev, steps, warmup, only=None):
-    """The other workloads of the metric. `only` (group names out of attn, gemm, rows, blocks, library) restricts the run to those
-    groups, e.g. for a counter-collection run of one kernel."""
+def _extras(dev, steps, warmup, only=None, skip=()):
+    """The other workloads of the metric. `only` (group names out of attn, attn_options, gemm, rows, blocks, library) restricts
+    the run to those groups, `skip` leaves groups out, e.g. for a counter-collection run of one kernel."""
     out = {}
     for name, fn in EXTRA_GROUPS.items():
-        if only is None or name in only:
+        if (only is None or name in only) and name not in skip:
             fn(dev, steps, warmup, torch.Generator().manual_seed(1 + sorted(EXTRA_GROUPS).index(name)), out)
     return out
 
@@ -402,7 +419,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
-    ap.add_argument("--only", default=None, help="comma-separated groups of the other workloads to run (attn, gemm, rows, blocks, library)")
+    ap.add_argument("--only", default=None,
+                    help="comma-separated groups of the other workloads to run (attn, attn_options, gemm, rows, blocks, library)")
+    ap.add_argument("--skip", default="", help="comma-separated groups of the other workloads to leave out")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 512 MiB (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -463,7 +482,7 @@ def main():
         result["cpu_baseline"] = None
     if not args.no_extras:
         only = None if args.only is None else set(args.only.split(","))
-        result["extras"] = _extras(dev, args.steps, args.warmup, only)
+        result["extras"] = _extras(dev, args.steps, args.warmup, only, set(filter(None, args.skip.split(","))))
         a = result["extras"].get("attn_self_fp8_per_token_scales")
         if a is not None:
             result["attn_tflops"] = a["tflops"]
