@@ -73,11 +73,13 @@ __device__ __forceinline__ v2i lds_read_tr_b64(unsigned addr) {
 // holds dim 32 d + 8 (e / 4) + 4 h + (e % 4) of query q, i.e. the two lanes of a query hold alternate groups of 4 dims.
 // One v_permlane32_swap per packed word hands every lane 8 consecutive dims (lane half 0 those of the even groups of 8,
 // lane half 1 the odd ones), so a lane stores 16 bytes of bf16 (8 bytes of e4m3) and the two lanes of a query 32 (16)
-// contiguous bytes per instruction: half as many, twice as large write requests as storing the groups of 4 directly.
+// contiguous bytes per instruction: half as many, twice as large write requests as storing the groups of 4 directly
+// (e4m3: a second exchange, 16 bytes per lane as well).
 template <int OUT>
 __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, const v16f (&o_acc)[2], float inv, bool live) {
 #pragma unroll
-    for (int d = 0; d < 2; ++d)
+    for (int d = 0; d < 2; ++d) {
+        uint32_t c8[2][2];  // e4m3: [wp] the 8 codes of dims 32 d + 16 wp + 8 h .. + 7
 #pragma unroll
         for (int wp = 0; wp < 2; ++wp) {  // the pair of 8-dim groups 2 wp, 2 wp + 1 of this 32-dim tile
             float a[8];
@@ -92,9 +94,18 @@ __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, con
             } else {
                 const auto s0 = __builtin_amdgcn_permlane32_swap(pack4_e4m3_sat(a[0], a[1], a[2], a[3]),
                                                                  pack4_e4m3_sat(a[4], a[5], a[6], a[7]), false, false);
-                if (live) *reinterpret_cast<v2i*>(reinterpret_cast<uint8_t*>(o) + row_off + dim) = v2i{(int)s0[0], (int)s0[1]};
+                c8[wp][0] = s0[0];
+                c8[wp][1] = s0[1];
             }
         }
+        if constexpr (OUT != Q8_BF16) {
+            // a second exchange of the same kind between the two 8-byte chunks: lane half 0 ends up with dims 32 d .. + 15,
+            // lane half 1 with dims 32 d + 16 .. + 31, so every lane stores 16 bytes and the two lanes of a query 32
+            const auto t0 = __builtin_amdgcn_permlane32_swap(c8[0][0], c8[1][0], false, false);
+            const auto t1 = __builtin_amdgcn_permlane32_swap(c8[0][1], c8[1][1], false, false);
+            if (live) *reinterpret_cast<v4u*>(reinterpret_cast<uint8_t*>(o) + row_off + 32 * d + 16 * h) = v4u{t0[0], t1[0], t0[1], t1[1]};
+        }
+    }
 }
 
 // kQT = 32-query tiles per wave, kWaves = waves per workgroup (4 or 8); a workgroup covers kWaves * kQT * 32 queries.
@@ -450,143 +461,259 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
     }
 }
 
+// One 32-query tile of attn_short_kernel against NB key blocks that lie in LDS at `st` (lane's row address; `so` the same
+// without the lane's row: base of the transposing V reads).
+template <int OUT, bool VTOK, int NB>
+__device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, unsigned st, unsigned so, unsigned fpc0, unsigned fpc1,
+                                           const unsigned (&vtb)[2], int valid, uint32_t keep, int h, size_t row_off, bool live) {
+    const float c = p.scale_log2;
+    v4i kl[NB][2], kh[NB][2];
+#pragma unroll
+    for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            kl[kb][t] = t ? lds_read_b128<2048>(st + kb * kStage + fpc0) : lds_read_b128<0>(st + kb * kStage + fpc0);
+            kh[kb][t] = t ? lds_read_b128<2048>(st + kb * kStage + fpc1) : lds_read_b128<0>(st + kb * kStage + fpc1);
+        }
+    if constexpr (NB == 2)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(kl[0][0]), "+v"(kh[0][0]), "+v"(kl[0][1]), "+v"(kh[0][1]), "+v"(kl[NB - 1][0]), "+v"(kh[NB - 1][0]),
+                       "+v"(kl[NB - 1][1]), "+v"(kh[NB - 1][1])
+                     :
+                     : "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kl[0][0]), "+v"(kh[0][0]), "+v"(kl[0][1]), "+v"(kh[0][1]) : : "memory");
+    float x[NB][32];
+#pragma unroll
+    for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const v8i kf = v8i{kl[kb][t][0], kl[kb][t][1], kl[kb][t][2], kl[kb][t][3], kh[kb][t][0], kh[kb][t][1], kh[kb][t][2], kh[kb][t][3]};
+            v16f z;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) z[e] = 0.f;
+            const v16f s = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf, z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) x[kb][16 * t + e] = s[e];
+        }
+    // Masking in the last block that holds valid keys (the only one that can be partial): bit e of `keep` says that this
+    // lane's key e of that block is valid; a sign-extending bit-field extract and a bit select per logit, no comparison
+    // (32 independent comparisons would each hold a pair of scalar registers).
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < NB; ++kb) {
+        if (kb == NB - 1 && 64 * NB > valid) {
+#pragma unroll
+            for (int e = 0; e < 32; ++e) {
+                const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)keep, e, 1);  // all ones: keep
+                x[kb][e] = __uint_as_float((__float_as_uint(x[kb][e]) & m) | (0xff800000u & ~m));
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 32; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[kb][e]), x[kb][e + 1]);
+    }
+    mx = fmaxf(mx, lane_xor<32>(mx));
+    const float m_sub = mx * c - (p.p_shift + p.m_slack);  // the final maximum is known: no slack needed
+    float psum = 0.f, psum_rounded = 0.f;
+    v16f o_acc[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[d][e] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < NB; ++kb) {
+        // the V operand of this block is requested now and arrives under the block's exponentials
+        v4i vl[2], vh[2];
+        v2i vr[2][4];
+        (void)vl; (void)vh; (void)vr;
+        if constexpr (VTOK) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+                vr[d][0] = lds_read_tr_b64<0>(so + kb * kStage + vtb[d]);
+                vr[d][1] = lds_read_tr_b64<512>(so + kb * kStage + vtb[d]);
+                vr[d][2] = lds_read_tr_b64<1024>(so + kb * kStage + vtb[d]);
+                vr[d][3] = lds_read_tr_b64<1536>(so + kb * kStage + vtb[d]);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                vl[t] = t ? lds_read_b128<4096 + 2048>(st + kb * kStage + fpc0) : lds_read_b128<4096>(st + kb * kStage + fpc0);
+                vh[t] = t ? lds_read_b128<4096 + 2048>(st + kb * kStage + fpc1) : lds_read_b128<4096>(st + kb * kStage + fpc1);
+            }
+        }
+        v8i pf;
+        float pr[32];
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            pr[e] = fast_exp2(fmaf(x[kb][e], c, -m_sub));
+            psum += pr[e];
+        }
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
+            u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
+            pf[w] = (int)u;
+        }
+        if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {
+#pragma unroll
+            for (int w = 0; w < 8; ++w)
+                psum_rounded += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
+        }
+        // (the probabilities pass through the wait as well: the exponentials stay above it, under the reads' latency)
+        if constexpr (VTOK) {
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(vr[0][0]), "+v"(vr[0][1]), "+v"(vr[0][2]), "+v"(vr[0][3]), "+v"(vr[1][0]), "+v"(vr[1][1]),
+                           "+v"(vr[1][2]), "+v"(vr[1][3]), "+v"(pf)
+                         :
+                         : "memory");
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vl[0]), "+v"(vh[0]), "+v"(vl[1]), "+v"(vh[1]), "+v"(pf) : : "memory");
+        }
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            v8i vf;
+            if constexpr (VTOK)
+                vf = v8i{vr[d][0][0], vr[d][0][1], vr[d][1][0], vr[d][1][1], vr[d][2][0], vr[d][2][1], vr[d][3][0], vr[d][3][1]};
+            else
+                vf = v8i{vl[d][0], vl[d][1], vl[d][2], vl[d][3], vh[d][0], vh[d][1], vh[d][2], vh[d][3]};
+            o_acc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, o_acc[d], 0, 0, 0, 0, 0, 0);
+        }
+    }
+    // ---- O^T lane (q, h), tile d, register e holds dim 32 d + 8 (e/4) + 4 h + (e%4)
+    if (p.flags & Q8_ATTN_SUM_ROUNDED_P) psum = psum_rounded;
+    const float l = psum + lane_xor<32>(psum);
+    const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
+    store_o_tile<OUT>(p.o, row_off, h, o_acc, inv, live);
+}
+
 // Short key / value sequences (N <= 128: cross-attention to a text prompt, csrc/flash_attention/
-// flash_attention_cuda_mask.cu:254-535 in the reference). The whole K and V^T of a (batch, head) are 16 KiB: every wave
-// keeps them in registers as ready-made MFMA operands (64 registers, loaded once) and walks over many 32-query tiles with
-// them, so a tile costs one 2 KiB read of Q (requested one tile ahead) and one store of O and nothing else: no LDS, no
-// barrier, no running maximum (all keys of a query are present at once, the probabilities are rounded against the
-// final maximum like the oracle's). Operand layouts, masking, P rounding and the output stage are those of
-// attn_fwd_kernel; a 64-key block beyond the valid length is skipped. A workgroup belongs to one head and takes its
-// share of the queries of EVERY batch in turn: the valid lengths differ per batch, and with a workgroup per
-// (batch, head) the launch would last as long as its longest batch.
-template <int OUT>
-__global__ __launch_bounds__(512) void attn_short_kernel(const AttnParams p, int tiles_per_wave) {
+// flash_attention_cuda_mask.cu:254-535 in the reference). The whole K and V of a (batch, head) are 16 KiB: they are copied
+// to LDS once, in the tile layouts of attn_fwd_kernel (two 64-key blocks), and every wave of the workgroup walks over
+// several 32-query tiles with them, so a tile costs one 2 KiB read of Q (requested one tile ahead), 16 operand reads from
+// LDS and one store of O. All keys of a query are present at once: no running maximum, the probabilities are rounded
+// against the final maximum like the oracle's. Operand layouts, masking, P rounding and the output stage are those of
+// attn_fwd_kernel; a 64-key block beyond the valid length is skipped. A workgroup (4 waves, three per CU) belongs to one
+// head and takes its share of the queries of EVERY batch in turn - the valid lengths differ per batch, and with a
+// workgroup per (batch, head) the launch would last as long as its longest batch - and while it works on one batch the
+// K / V of the next one are already on their way into the other half of the LDS buffer.
+template <int OUT, bool VTOK>
+__global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, int tiles_per_wave) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * 2 * kStage];  // [batch parity][key block]: K tile, V tile
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
-    const int M = p.M, N = p.N;
-    for (int b = 0; b < p.B; ++b) {
-        const int bh = b * p.H + blockIdx.y;
-        int valid = N;
-        if (p.kv_len) {
-            const int len = p.kv_len[b];
-            valid = len < N ? (len < 0 ? 0 : len) : N;
-        }
-        const uint8_t* Qg = p.q + (size_t)bh * M * 64;
+    const int M = p.M, N = p.N, head = blockIdx.y;
+    const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
+    const size_t o_rs = o_tok ? (size_t)p.H * 64 : 64;
+    const int q_tiles = (M + 31) >> 5;
+    const int tile0 = blockIdx.x * (4 * tiles_per_wave) + wave;  // this wave's tiles: tile0 + 4 it
+
+    auto valid_of = [&](int b) {
+        if (!p.kv_len) return N;
+        const int len = p.kv_len[b];
+        return len < N ? (len < 0 ? 0 : len) : N;
+    };
+    // copy plan of attn_fwd_kernel with 4 waves: wave w fills LDS rows 16 w .. 16 w + 15 of the K tile and of the V tile of
+    // both key blocks, 4 copies per wave and batch (blocks without valid keys are filled from a block of zeros, so that
+    // every wave always issues the same number of copies)
+    const int crow = 16 * wave + (lane >> 2);
+    const int cchunk = (lane & 3) ^ ((crow >> 2) & 3);
+    const int vchunk = (lane & 3) ^ (((crow >> 2) & 1) << 1);
+    int k_src_row;
+    {
+        const int t = crow >> 5, i = crow & 31;
+        k_src_row = 32 * ((i >> 2) & 1) + 16 * t + 4 * (i >> 3) + (i & 3);
+    }
+    auto issue_copies = [&](int b) {
+        const int bh = b * p.H + head;
         const uint8_t* Kg = p.k + (size_t)bh * N * 64;
-        const uint8_t* Vg = p.v + (size_t)bh * 64 * p.v_row_stride;
-        const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
-        const size_t o_base = o_tok ? ((size_t)b * M * p.H + (size_t)(bh - b * p.H)) * 64 : (size_t)bh * M * 64;
-        const size_t o_rs = o_tok ? (size_t)p.H * 64 : 64;
+        const uint8_t* Vg = p.v + (size_t)bh * 64 * (VTOK ? (size_t)N : (size_t)p.v_row_stride);
+        const int n_blocks = (valid_of(b) + 63) >> 6;
+        const uint8_t* zero = reinterpret_cast<const uint8_t*>(g_attn_zero16);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            uint8_t* base = lds + ((b & 1) * 2 + kb) * kStage;
+            const bool real = kb < n_blocks;
+            int kr = 64 * kb + k_src_row;
+            kr = kr < N ? kr : N - 1;
+            const uint8_t* ks = real ? Kg + (size_t)kr * 64 + cchunk * 16 : zero;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
+                                             (__attribute__((address_space(3))) void*)(base + wave * 1024), 16, 0, 0);
+            const uint8_t* vs;
+            if constexpr (VTOK) {
+                int vr = 64 * kb + crow;
+                vr = vr < N ? vr : N - 1;  // rows past the end repeat the last key; their probabilities are zero
+                vs = real ? Vg + (size_t)vr * 64 + vchunk * 16 : zero;
+            } else {
+                const int col = 64 * kb + cchunk * 16;
+                vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
+            }
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
+                                             (__attribute__((address_space(3))) void*)(base + 4096 + wave * 1024), 16, 0, 0);
+        }
+    };
+    // operand fetch addresses inside a key block (as in attn_fwd_kernel)
+    const unsigned fbase = lds_addr(lds) + ql * 64;
+    const unsigned fpc0 = ((2 * h) ^ ((ql >> 2) & 3)) * 16, fpc1 = fpc0 ^ 16;
+    unsigned vtb[2];
+    {
+        const int l16 = lane & 15, a = (lane >> 4) & 1, f = ((l16 >> 3) & 1) << 1;
+        const unsigned row_off = (unsigned)(32 * h + (l16 >> 1)) * 64 + (l16 & 1) * 8;
+        vtb[0] = lds_addr(lds) + 4096 + row_off + ((0 + a) ^ f) * 16;
+        vtb[1] = lds_addr(lds) + 4096 + row_off + ((2 + a) ^ f) * 16;
+    }
+    auto load_q = [&](int b, int tile) {  // Q^T operand: lane (q, h) holds bytes 32 h .. 32 h + 31 of query row q
+        int row = 32 * tile + ql;
+        row = row < M ? row : M - 1;
+        const v4i* src = reinterpret_cast<const v4i*>(p.q + ((size_t)(b * p.H + head) * M + row) * 64 + 32 * h);
+        const v4i a = src[0], c = src[1];
+        return v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
+    };
+    issue_copies(0);
+    v8i qf = load_q(0, tile0 < q_tiles ? tile0 : 0);
+    for (int b = 0; b < p.B; ++b) {
+        // the copies of batch b (issued one batch ago) have landed - for every wave after the barrier, which also says that
+        // all waves are done with batch b - 1, whose half of the buffer the next copies overwrite
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (b + 1 < p.B) issue_copies(b + 1);
+        const int bh = b * p.H + head;
+        const size_t o_base = o_tok ? ((size_t)b * M * p.H + (size_t)head) * 64 : (size_t)bh * M * 64;
+        const int valid = valid_of(b);
         const int n_blocks = (valid + 63) >> 6;  // 64-key blocks that hold valid keys: 0, 1 or 2
-
-        // K operand of block kb, tile t: lane (i, h) holds bytes 32 h .. 32 h + 31 of the key that comes out as row i of the
-        // S^T accumulator tile (lane half h then owns keys 32 h .. 32 h + 31 of the block in operand byte order);
-        // V^T operand of block kb, tile d: lane (i, h) holds keys 64 kb + 32 h .. + 31 of V^T row 32 d + i.
-        v8i kf[2][2], vf[2][2];
-        const v4i zero4 = v4i{0, 0, 0, 0};
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                int key = 64 * kb + 32 * ((ql >> 2) & 1) + 16 * t + 4 * (ql >> 3) + (ql & 3);
-                key = key < N ? key : N - 1;
-                const v4i* ks = reinterpret_cast<const v4i*>(Kg + (size_t)key * 64 + 32 * h);
-                v4i a = zero4, c = zero4, va = zero4, vc = zero4;
-                if (kb < n_blocks) {
-                    a = ks[0];
-                    c = ks[1];
-                    const int col = 64 * kb + 32 * h;
-                    const uint8_t* vs = Vg + (size_t)(32 * t + ql) * p.v_row_stride + col;
-                    if (col < p.v_row_stride) va = *reinterpret_cast<const v4i*>(vs);
-                    if (col + 16 < p.v_row_stride) vc = *reinterpret_cast<const v4i*>(vs + 16);
-                }
-                kf[kb][t] = v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
-                vf[kb][t] = v8i{va[0], va[1], va[2], va[3], vc[0], vc[1], vc[2], vc[3]};
-            }
-
-        const int q_tiles = (M + 31) >> 5;
-        const int wave_id = blockIdx.x * 8 + wave, waves = gridDim.x * 8;
-        auto load_q = [&](int tile) {  // Q^T operand: lane (q, h) holds bytes 32 h .. 32 h + 31 of query row q
-            int row = 32 * tile + ql;
-            row = row < M ? row : M - 1;
-            const v4i* src = reinterpret_cast<const v4i*>(Qg + (size_t)row * 64 + 32 * h);
-            const v4i a = src[0], c = src[1];
-            return v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
-        };
-        const float c = p.scale_log2;
-        int tile = wave_id;
-        v8i qf = load_q(tile < q_tiles ? tile : 0);
-        for (int it = 0; it < tiles_per_wave && tile < q_tiles; ++it, tile += waves) {
-            const int next = tile + waves;
-            const v8i qn = load_q(next < q_tiles ? next : tile);  // requested now, used in the next round
-            float x[2][32];
-            float mx = -INFINITY;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                if (kb < n_blocks) {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        v16f z;
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) z[e] = 0.f;
-                        const v16f s = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[kb][t], qf, z, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) x[kb][16 * t + e] = s[e];
-                    }
-                    if (64 * kb + 64 > valid) {
-#pragma unroll
-                        for (int e = 0; e < 32; ++e)
-                            if (64 * kb + 32 * h + e >= valid) x[kb][e] = -INFINITY;
-                    }
-#pragma unroll
-                    for (int e = 0; e < 32; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[kb][e]), x[kb][e + 1]);
-                }
-            }
-            mx = fmaxf(mx, lane_xor<32>(mx));
-            // (no valid key at all: everything below is skipped and the output is zero)
-            const float m_sub = mx * c - (p.p_shift + p.m_slack);  // the final maximum is known: no slack needed
-            float psum = 0.f, psum_rounded = 0.f;
-            v16f o_acc[2];
-#pragma unroll
-            for (int d = 0; d < 2; ++d)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o_acc[d][e] = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                if (kb < n_blocks) {
-                    v8i pf;
-                    float pr[32];
-#pragma unroll
-                    for (int e = 0; e < 32; ++e) {
-                        pr[e] = fast_exp2(fmaf(x[kb][e], c, -m_sub));
-                        psum += pr[e];
-                    }
-#pragma unroll
-                    for (int w = 0; w < 8; ++w) {
-                        uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
-                        u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
-                        pf[w] = (int)u;
-                    }
-                    if (p.flags & Q8_ATTN_SUM_ROUNDED_P) {  // this kernel waits for HBM: the vector ALU has the time
-#pragma unroll
-                        for (int w = 0; w < 8; ++w)
-                            psum_rounded += e4m3_to_f32<0>(pf[w]) + e4m3_to_f32<1>(pf[w]) + e4m3_to_f32<2>(pf[w]) + e4m3_to_f32<3>(pf[w]);
-                    }
+        const unsigned buf = (b & 1) * 2 * kStage;
+        // valid keys among this lane's 32 of the last block with valid keys (keys 64 (n_blocks - 1) + 32 h + e), as a bit mask
+        uint32_t keep = 0xffffffffu;
+        {
+            const int lim = valid - 64 * (n_blocks - 1) - 32 * h;
+            keep = lim >= 32 ? 0xffffffffu : (lim <= 0 ? 0u : ((1u << lim) - 1u));
+        }
+        for (int it = 0; it < tiles_per_wave; ++it) {
+            const int tile = tile0 + 4 * it;
+            // the Q operand of this wave's next tile (of the next batch after the last one of this batch)
+            const bool last_it = it + 1 == tiles_per_wave;
+            const int nb = last_it ? (b + 1 < p.B ? b + 1 : b) : b;
+            const int nt = last_it ? tile0 : tile + 4;
+            const v8i qn = load_q(nb, nt < q_tiles ? nt : 0);
+            if (tile < q_tiles) {
+                const size_t row_off = o_base + (size_t)(32 * tile + ql) * o_rs;
+                const bool live = 32 * tile + ql < M;
+                // straight-line code per number of key blocks (uniform per batch)
+                if (n_blocks == 2) short_tile<OUT, VTOK, 2>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live);
+                else if (n_blocks == 1) short_tile<OUT, VTOK, 1>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live);
+                else {  // no valid key at all: the output is zero
+                    v16f o_acc[2];
 #pragma unroll
                     for (int d = 0; d < 2; ++d)
-                        o_acc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[kb][d], pf, o_acc[d], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) o_acc[d][e] = 0.f;
+                    store_o_tile<OUT>(p.o, row_off, h, o_acc, 1.f, live);
                 }
             }
-            // ---- O^T lane (q, h), tile d, register e holds dim 32 d + 8 (e/4) + 4 h + (e%4)
-            const int row = 32 * tile + ql;
-            if (p.flags & Q8_ATTN_SUM_ROUNDED_P) psum = psum_rounded;
-            const float l = psum + lane_xor<32>(psum);
-            const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
-            store_o_tile<OUT>(p.o, o_base + (size_t)row * o_rs, h, o_acc, inv, row < M);
             qf = qn;
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace q8
@@ -620,8 +747,8 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
         return fail(Q8_ERR_SHAPE, "q8_attn_fwd: V row stride %lld must be >= N and a multiple of 16", (long long)v_row_stride);
     const bool scaled = sq || sk || sv;
     if (scaled && !(sq && sk && sv)) return fail(Q8_ERR_NULL, "q8_attn_fwd: sq, sk, sv must be given together");
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (reinterpret_cast<uintptr_t>(o) % 8))
-        return fail(Q8_ERR_ALIGN, "q8_attn_fwd: q, k, v must be 16-byte and o 8-byte aligned");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return fail(Q8_ERR_ALIGN, "q8_attn_fwd: q, k, v and o must be 16-byte aligned");
     if ((flags & Q8_ATTN_LAZY_MAX) && (flags & Q8_ATTN_P_UNIT_RANGE))
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: Q8_ATTN_LAZY_MAX needs the head room of the default probability range (not P_UNIT_RANGE)");
     if ((flags & Q8_ATTN_SUM_ROUNDED_P) && scaled)
@@ -637,17 +764,18 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     const bool msum = (flags & Q8_ATTN_SUM_ROUNDED_P) != 0;
     if (msum && cfg == 1)
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape has no Q8_ATTN_SUM_ROUNDED_P form");
-    if (N <= 128 && !scaled && cfg != 3 && !vtok) {
-        // K and V^T stay in registers; enough waves to fill the device, each walking over several query tiles
-        // (tiles per wave and batch: about 2048 waves in all, one 8-wave workgroup per CU)
+    if (N <= 128 && !scaled && cfg != 3) {
+        // K and V stay in LDS; enough workgroups of 4 waves to place two on every CU (about 2048 waves in all), each wave
+        // walking over several query tiles of every batch
         const long q_tiles = (M + 31) / 32;
         long tpw = (q_tiles * H + 2047) / 2048;
         tpw = tpw < 1 ? 1 : (tpw > 16 ? 16 : tpw);
-        const unsigned gx = (unsigned)((q_tiles + 8 * tpw - 1) / (8 * tpw));
-        if (out_dtype == Q8_BF16)
-            hipLaunchKernelGGL((attn_short_kernel<Q8_BF16>), dim3(gx, (unsigned)H), dim3(512), 0, stream, p, (int)tpw);
-        else
-            hipLaunchKernelGGL((attn_short_kernel<Q8_E4M3>), dim3(gx, (unsigned)H), dim3(512), 0, stream, p, (int)tpw);
+        const unsigned gx = (unsigned)((q_tiles + 4 * tpw - 1) / (4 * tpw));
+#define Q8_ATTN_SHORT(OUTT)                                                                                             \
+    if (vtok) hipLaunchKernelGGL((attn_short_kernel<OUTT, true>), dim3(gx, (unsigned)H), dim3(256), 0, stream, p, (int)tpw); \
+    else hipLaunchKernelGGL((attn_short_kernel<OUTT, false>), dim3(gx, (unsigned)H), dim3(256), 0, stream, p, (int)tpw)
+        if (out_dtype == Q8_BF16) { Q8_ATTN_SHORT(Q8_BF16); } else { Q8_ATTN_SHORT(Q8_E4M3); }
+#undef Q8_ATTN_SHORT
         return launch_status("q8_attn_fwd");
     }
     // Shapes: with unit scales 8 waves x 32 queries fit 128 registers (two workgroups = 4 waves per SIMD) and share a K / V

@@ -75,14 +75,22 @@ __device__ __forceinline__ float clamp448(float v) {
     return v;
 }
 __device__ __forceinline__ uint32_t pack4_e4m3_sat(float a, float b, float c, float d) {
-    uint32_t p = cvt_pk_e4m3(clamp448(a), clamp448(b), 0u, false);
-    p = cvt_pk_e4m3(clamp448(c), clamp448(d), p, true);
-    uint32_t m = 0u;
-    m |= (a != a) ? 0x0000007fu : 0u;
-    m |= (b != b) ? 0x00007f00u : 0u;
-    m |= (c != c) ? 0x007f0000u : 0u;
-    m |= (d != d) ? 0x7f000000u : 0u;
-    return p | m;
+    // One v_med3_f32 per value clamps everything that is not NaN (a NaN would come out as -448); two unordered
+    // comparisons say whether any of the four values of any lane is NaN, and only then the wave takes the form that
+    // keeps NaN (compare-and-select clamps, 0x7f patched over the code). Same codes as that form for every input.
+    const bool any_nan = __builtin_isunordered(a, b) || __builtin_isunordered(c, d);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(any_nan) != 0, 0)) {
+        uint32_t p = cvt_pk_e4m3(clamp448(a), clamp448(b), 0u, false);
+        p = cvt_pk_e4m3(clamp448(c), clamp448(d), p, true);
+        uint32_t m = 0u;
+        m |= (a != a) ? 0x0000007fu : 0u;
+        m |= (b != b) ? 0x00007f00u : 0u;
+        m |= (c != c) ? 0x007f0000u : 0u;
+        m |= (d != d) ? 0x7f000000u : 0u;
+        return p | m;
+    }
+    uint32_t p = cvt_pk_e4m3(__builtin_amdgcn_fmed3f(a, -448.f, 448.f), __builtin_amdgcn_fmed3f(b, -448.f, 448.f), 0u, false);
+    return cvt_pk_e4m3(__builtin_amdgcn_fmed3f(c, -448.f, 448.f), __builtin_amdgcn_fmed3f(d, -448.f, 448.f), p, true);
 }
 
 // ---------------------------------------------------------------- cross-lane exchange (wave64)

@@ -165,8 +165,7 @@ def test_attention_sum_rounded_p(dev, cfg, m, n, std):
         got = run(v)
         got_tok = C.flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16, sum_rounded_p=True,
                                     v_token_major=True)
-        if n > 128:  # (shorter sequences: V^T takes the register-resident kernel, token-major V the general one)
-            assert torch.equal(got.cpu().view(torch.int16), got_tok.cpu().view(torch.int16))
+        assert torch.equal(got.cpu().view(torch.int16), got_tok.cpu().view(torch.int16))  # both layouts take the same kernel
         lazy = run(v, lazy_max=True)
     finally:
         _lib.check(_lib.lib().q8_attn_set_config(0))
@@ -474,14 +473,12 @@ def test_token_major_v_gives_the_bits_of_the_transposed_layout(dev, m, n, lens, 
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32)
     lens_d = None if lens is None else lens_t.to(dev)
     for out_dtype in (torch.bfloat16, E4M3):
-        _lib.check(_lib.lib().q8_attn_set_config(3))  # the transposed layout through the general kernel as well
-        try:
-            want = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens_d, out_dtype=out_dtype, **kw)
-        finally:
-            _lib.check(_lib.lib().q8_attn_set_config(0))
-        for cfg in (0, 2, 4):  # the default shape of the mode and both shapes that read token-major V
+        # the default shape of the mode, both shapes that read token-major V and the general kernel where a short
+        # sequence would take the LDS-resident one: each against the transposed layout under the same configuration
+        for cfg in (0, 2, 3, 4):
             _lib.check(_lib.lib().q8_attn_set_config(cfg))
             try:
+                want = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens_d, out_dtype=out_dtype, **kw)
                 got = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, lens_d, out_dtype=out_dtype,
                                            v_token_major=True, **kw)
             finally:
