@@ -316,6 +316,8 @@ int q8_gemm_i32(const int8_t* A, const int8_t* B, int32_t* C, int M, int N, int 
  * kv_len: int32 [B] or NULL; sq: fp32 [B,H,M], sk, sv: fp32 [B,H,N] per-token dequantisation scales
  * or NULL (all three given or none). D must be 64. softmax_scale is the plain (natural-log) scale.
  * B == 0 or M == 0 (no queries) returns Q8_OK without touching any pointer; N has to be positive.
+ * q, k, v and o 16-byte aligned (Q8_ERR_ALIGN otherwise). N <= 128 runs a kernel that holds K and V of a (batch, head)
+ * in LDS and rounds P against the final row maximum; longer sequences round it against the running maximum.
  */
 int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int32_t* kv_len,
                 const float* sq, const float* sk, const float* sv,
@@ -325,8 +327,8 @@ int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int3
 /*
  * Workgroup-shape override for q8_attn_fwd: 0 = the default of the mode (unit scales: 8 waves x 32 queries, per-token
  * scales: 4 waves x 32 queries), 1 = 4 waves x 64 queries (Q8_V_DS only), 2 = 4 waves x 32 queries, 3 = as 0 without the
- * register-resident kernel that otherwise takes N <= 128 with unit scales, 4 = 8 waves x 32 queries. All shapes give the
- * same bits. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
+ * short-sequence kernel that otherwise takes N <= 128 (K and V of a (batch, head) resident in LDS, P rounded against the
+ * final row maximum), 4 = 8 waves x 32 queries. All shapes of one kernel give the same bits. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
  * workgroup is fixed at 4 warps x 16 queries, csrc/flash_attention/flash_attention_cuda.cu:279-287).
  */
 int q8_attn_set_config(int cfg);

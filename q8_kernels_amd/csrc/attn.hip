@@ -3,7 +3,7 @@
 // One workgroup = 8 waves x 32 query rows of one (batch, head) with unit scales, 4 waves x 32 with per-token scales (whose
 // register need allows three such workgroups on a CU but only one of 8 waves); 4 x 64 is instantiated as well. KV is
 // walked forward in tiles of 64 keys that all waves share through a four-stage LDS ring filled by
-// global_load_lds_dwordx4. Key / value sequences of at most 128 tokens with unit scales take attn_short_kernel instead.
+// global_load_lds_dwordx4. Key / value sequences of at most 128 tokens take attn_short_kernel instead.
 // V arrives either channel-major per head (V^T [B,H,64,Nv], Q8_V_DS) or token-major like K ([B,H,N,64], Q8_V_SD); the
 // token-major tile is turned while it is read from LDS (ds_read_b64_tr_b8), so no transposed copy of V exists in HBM.
 //
@@ -463,10 +463,13 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
 
 // One 32-query tile of attn_short_kernel against NB key blocks that lie in LDS at `st` (lane's row address; `so` the same
 // without the lane's row: base of the transposing V reads).
-template <int OUT, bool VTOK, int NB>
+// SCALED: `c` = sq[query] * scale_log2 of this lane's query, `bias` the exponent bias (p_shift + m_slack + log2(1 / max sv)),
+// `sc` the LDS address of this lane half's 32 key scales of block 0 (value scales 512 bytes further, block 1 256 bytes
+// further): the per-token scales enter as in attn_fwd_kernel.
+template <int OUT, bool VTOK, bool SCALED, int NB>
 __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, unsigned st, unsigned so, unsigned fpc0, unsigned fpc1,
-                                           const unsigned (&vtb)[2], int valid, uint32_t keep, int h, size_t row_off, bool live) {
-    const float c = p.scale_log2;
+                                           const unsigned (&vtb)[2], int valid, uint32_t keep, int h, size_t row_off, bool live,
+                                           float c, float bias, unsigned sc) {
     v4i kl[NB][2], kh[NB][2];
 #pragma unroll
     for (int kb = 0; kb < NB; ++kb)
@@ -496,6 +499,24 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
 #pragma unroll
             for (int e = 0; e < 16; ++e) x[kb][16 * t + e] = s[e];
         }
+    if constexpr (SCALED) {
+        // the key scales of this lane's 32 keys per block (broadcast reads) multiply the raw logits
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb) {
+            v4i rk[8];
+            rk[0] = lds_read_b128<0>(sc + kb * 256); rk[1] = lds_read_b128<16>(sc + kb * 256);
+            rk[2] = lds_read_b128<32>(sc + kb * 256); rk[3] = lds_read_b128<48>(sc + kb * 256);
+            rk[4] = lds_read_b128<64>(sc + kb * 256); rk[5] = lds_read_b128<80>(sc + kb * 256);
+            rk[6] = lds_read_b128<96>(sc + kb * 256); rk[7] = lds_read_b128<112>(sc + kb * 256);
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(rk[0]), "+v"(rk[1]), "+v"(rk[2]), "+v"(rk[3]), "+v"(rk[4]), "+v"(rk[5]), "+v"(rk[6]), "+v"(rk[7])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int e = 0; e < 32; ++e) x[kb][e] *= __int_as_float(rk[e >> 2][e & 3]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
     // Masking in the last block that holds valid keys (the only one that can be partial): bit e of `keep` says that this
     // lane's key e of that block is valid; a sign-extending bit-field extract and a bit select per logit, no comparison
     // (32 independent comparisons would each hold a pair of scalar registers).
@@ -503,6 +524,9 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
 #pragma unroll
     for (int kb = 0; kb < NB; ++kb) {
         if (kb == NB - 1 && 64 * NB > valid) {
+            // (the mask passes through an empty asm: the 64 words derived from it would otherwise be computed once,
+            //  outside the tile loop, and held in registers)
+            asm volatile("" : "+v"(keep));
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
                 const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)keep, e, 1);  // all ones: keep
@@ -513,7 +537,7 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
         for (int e = 0; e < 32; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[kb][e]), x[kb][e + 1]);
     }
     mx = fmaxf(mx, lane_xor<32>(mx));
-    const float m_sub = mx * c - (p.p_shift + p.m_slack);  // the final maximum is known: no slack needed
+    const float m_sub = mx * c - bias;  // the final maximum is known: the slack of Q8_ATTN_LAZY_MAX is head room not needed
     float psum = 0.f, psum_rounded = 0.f;
     v16f o_acc[2];
 #pragma unroll
@@ -522,6 +546,9 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
         for (int e = 0; e < 16; ++e) o_acc[d][e] = 0.f;
 #pragma unroll
     for (int kb = 0; kb < NB; ++kb) {
+        // (scheduling fence: the second block's exponentials and reads stay behind the first block's products, which keeps
+        //  the live registers at one block's worth)
+        __builtin_amdgcn_sched_barrier(0);
         // the V operand of this block is requested now and arrives under the block's exponentials
         v4i vl[2], vh[2];
         v2i vr[2][4];
@@ -541,12 +568,28 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
                 vh[t] = t ? lds_read_b128<4096 + 2048>(st + kb * kStage + fpc1) : lds_read_b128<4096>(st + kb * kStage + fpc1);
             }
         }
+        v4i rv[SCALED ? 8 : 1];
+        if constexpr (SCALED) {
+            rv[0] = lds_read_b128<512>(sc + kb * 256); rv[1] = lds_read_b128<528>(sc + kb * 256);
+            rv[2] = lds_read_b128<544>(sc + kb * 256); rv[3] = lds_read_b128<560>(sc + kb * 256);
+            rv[4] = lds_read_b128<576>(sc + kb * 256); rv[5] = lds_read_b128<592>(sc + kb * 256);
+            rv[6] = lds_read_b128<608>(sc + kb * 256); rv[7] = lds_read_b128<624>(sc + kb * 256);
+        }
         v8i pf;
         float pr[32];
 #pragma unroll
         for (int e = 0; e < 32; ++e) {
             pr[e] = fast_exp2(fmaf(x[kb][e], c, -m_sub));
             psum += pr[e];
+        }
+        if constexpr (SCALED) {
+            // (the V operand reads were issued before these: in-order return, so this wait covers them as well)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]), "+v"(rv[4]), "+v"(rv[5]), "+v"(rv[6]), "+v"(rv[7])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int e = 0; e < 32; ++e) pr[e] *= __int_as_float(rv[e >> 2][e & 3]);
         }
 #pragma unroll
         for (int w = 0; w < 8; ++w) {
@@ -596,9 +639,10 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
 // head and takes its share of the queries of EVERY batch in turn - the valid lengths differ per batch, and with a
 // workgroup per (batch, head) the launch would last as long as its longest batch - and while it works on one batch the
 // K / V of the next one are already on their way into the other half of the LDS buffer.
-template <int OUT, bool VTOK>
-__global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, int tiles_per_wave) {
+template <int OUT, bool VTOK, bool SCALED>
+__global__ __launch_bounds__(256, (SCALED || VTOK) ? 2 : 3) void attn_short_kernel(const AttnParams p, int tiles_per_wave) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * 2 * kStage];  // [batch parity][key block]: K tile, V tile
+    __shared__ __attribute__((aligned(256))) float lds_sc[SCALED ? 2 * 256 : 4];  // [batch parity]: sk[128], sv[128]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
@@ -651,6 +695,19 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
                                              (__attribute__((address_space(3))) void*)(base + 4096 + wave * 1024), 16, 0, 0);
         }
+        if constexpr (SCALED) {
+            if (wave < 2) {  // wave kb copies the 64 key scales and the 64 value scales of block kb, one dword per lane
+                int key = 64 * wave + lane;
+                key = key < N ? key : N - 1;
+                const bool real = wave < n_blocks;
+                const float* zf = reinterpret_cast<const float*>(g_attn_zero16);
+                float* dst = lds_sc + (b & 1) * 256 + 64 * wave;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sk + (size_t)bh * N + key : zf),
+                                                 (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sv + (size_t)bh * N + key : zf),
+                                                 (__attribute__((address_space(3))) void*)(dst + 128), 4, 0, 0);
+            }
+        }
     };
     // operand fetch addresses inside a key block (as in attn_fwd_kernel)
     const unsigned fbase = lds_addr(lds) + ql * 64;
@@ -669,8 +726,16 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
         const v4i a = src[0], c = src[1];
         return v8i{a[0], a[1], a[2], a[3], c[0], c[1], c[2], c[3]};
     };
+    // per-token scales: c of a tile's query, kept strictly positive like in attn_fwd_kernel (a masked key's -inf stays -inf)
+    auto load_c = [&](int b, int tile) {
+        if constexpr (!SCALED) return p.scale_log2;
+        int row = 32 * tile + ql;
+        row = row < M ? row : M - 1;
+        return fmaxf(p.sq[(size_t)(b * p.H + head) * M + row] * p.scale_log2, 1.17549435e-38f);
+    };
     issue_copies(0);
     v8i qf = load_q(0, tile0 < q_tiles ? tile0 : 0);
+    float cq = load_c(0, tile0 < q_tiles ? tile0 : 0);
     for (int b = 0; b < p.B; ++b) {
         // the copies of batch b (issued one batch ago) have landed - for every wave after the barrier, which also says that
         // all waves are done with batch b - 1, whose half of the buffer the next copies overwrite
@@ -682,6 +747,15 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
         const int valid = valid_of(b);
         const int n_blocks = (valid + 63) >> 6;  // 64-key blocks that hold valid keys: 0, 1 or 2
         const unsigned buf = (b & 1) * 2 * kStage;
+        // per-token V scales enter P as sv[j] / max_j sv[j] (maximum over the valid keys), the factor 1 / max as an exponent bias
+        float bias = p.p_shift + p.m_slack;
+        if constexpr (SCALED) {
+            const float* sv = lds_sc + (b & 1) * 256 + 128;
+            float mxv = fmaxf(lane < valid ? sv[lane] : 0.f, lane + 64 < valid ? sv[lane + 64] : 0.f);
+            mxv = group_max<64>(mxv);
+            bias += __builtin_log2f(mxv > 0.f ? 1.0f / mxv : 1.f);
+        }
+        const unsigned sc = lds_addr(lds_sc) + (b & 1) * 1024 + 128 * h;
         // valid keys among this lane's 32 of the last block with valid keys (keys 64 (n_blocks - 1) + 32 h + e), as a bit mask
         uint32_t keep = 0xffffffffu;
         {
@@ -695,12 +769,13 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
             const int nb = last_it ? (b + 1 < p.B ? b + 1 : b) : b;
             const int nt = last_it ? tile0 : tile + 4;
             const v8i qn = load_q(nb, nt < q_tiles ? nt : 0);
+            const float cn = load_c(nb, nt < q_tiles ? nt : 0);
             if (tile < q_tiles) {
                 const size_t row_off = o_base + (size_t)(32 * tile + ql) * o_rs;
                 const bool live = 32 * tile + ql < M;
                 // straight-line code per number of key blocks (uniform per batch)
-                if (n_blocks == 2) short_tile<OUT, VTOK, 2>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live);
-                else if (n_blocks == 1) short_tile<OUT, VTOK, 1>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live);
+                if (n_blocks == 2) short_tile<OUT, VTOK, SCALED, 2>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live, cq, bias, sc);
+                else if (n_blocks == 1) short_tile<OUT, VTOK, SCALED, 1>(p, qf, fbase + buf, buf, fpc0, fpc1, vtb, valid, keep, h, row_off, live, cq, bias, sc);
                 else {  // no valid key at all: the output is zero
                     v16f o_acc[2];
 #pragma unroll
@@ -711,6 +786,7 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
                 }
             }
             qf = qn;
+            cq = cn;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -721,7 +797,7 @@ __global__ __launch_bounds__(256, 2) void attn_short_kernel(const AttnParams p, 
 using namespace q8;
 
 // per thread: 0 = default (unit scales: 8 waves x 32 queries; per-token scales: 4 waves x 32 queries), 1 = 4 waves x 64
-// queries, 2 = 4 waves x 32 queries, 3 = as 0 and without the register-resident path for N <= 128, 4 = 8 waves x 32 queries
+// queries, 2 = 4 waves x 32 queries, 3 = as 0 and without the short-sequence kernel for N <= 128, 4 = 8 waves x 32 queries
 static thread_local int g_attn_cfg = 0;
 
 extern "C" int q8_attn_set_config(int cfg) {
@@ -764,17 +840,21 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     const bool msum = (flags & Q8_ATTN_SUM_ROUNDED_P) != 0;
     if (msum && cfg == 1)
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape has no Q8_ATTN_SUM_ROUNDED_P form");
-    if (N <= 128 && !scaled && cfg != 3) {
-        // K and V stay in LDS; enough workgroups of 4 waves to place two on every CU (about 2048 waves in all), each wave
-        // walking over several query tiles of every batch
+    if (N <= 128 && cfg != 3) {
+        // K and V stay in LDS; enough workgroups of 4 waves to fill every CU once (three per CU with unit scales and V^T,
+        // whose code fits 168 registers, two otherwise), each wave walking over several query tiles of every batch
         const long q_tiles = (M + 31) / 32;
-        long tpw = (q_tiles * H + 2047) / 2048;
+        const long wave_slots = (scaled || vtok) ? 2048 : 3072;
+        long tpw = (q_tiles * H + wave_slots - 1) / wave_slots;
         tpw = tpw < 1 ? 1 : (tpw > 16 ? 16 : tpw);
         const unsigned gx = (unsigned)((q_tiles + 4 * tpw - 1) / (4 * tpw));
-#define Q8_ATTN_SHORT(OUTT)                                                                                             \
-    if (vtok) hipLaunchKernelGGL((attn_short_kernel<OUTT, true>), dim3(gx, (unsigned)H), dim3(256), 0, stream, p, (int)tpw); \
-    else hipLaunchKernelGGL((attn_short_kernel<OUTT, false>), dim3(gx, (unsigned)H), dim3(256), 0, stream, p, (int)tpw)
-        if (out_dtype == Q8_BF16) { Q8_ATTN_SHORT(Q8_BF16); } else { Q8_ATTN_SHORT(Q8_E4M3); }
+#define Q8_ATTN_SHORT_L(OUTT, VT, SC) \
+    hipLaunchKernelGGL((attn_short_kernel<OUTT, VT, SC>), dim3(gx, (unsigned)H), dim3(256), 0, stream, p, (int)tpw)
+#define Q8_ATTN_SHORT(OUTT)                                                                              \
+    if (vtok) { if (scaled) Q8_ATTN_SHORT_L(OUTT, true, true); else Q8_ATTN_SHORT_L(OUTT, true, false); }  \
+    else { if (scaled) Q8_ATTN_SHORT_L(OUTT, false, true); else Q8_ATTN_SHORT_L(OUTT, false, false); }
+        if (out_dtype == Q8_BF16) { Q8_ATTN_SHORT(Q8_BF16) } else { Q8_ATTN_SHORT(Q8_E4M3) }
+#undef Q8_ATTN_SHORT_L
 #undef Q8_ATTN_SHORT
         return launch_status("q8_attn_fwd");
     }

@@ -72,10 +72,9 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
-    if q.shape == k.shape == v.shape and d == 64 and (k.shape[1] > 128 or per_token_scales):
+    if q.shape == k.shape == v.shape and d == 64:
         # self-attention: one pass over the three projections (the tables are read once, V is only cast and stays
-        # token-major; the attention kernel turns its tiles while reading them from LDS). Sequences of at most 128
-        # keys with unit scales keep the transposed V: the register-resident kernel that serves them reads V^T.
+        # token-major; the attention kernels turn its tiles while reading them from LDS).
         qc, kc, vc = _C.attn_prep_qkv(q, k, v, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
                                       q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
         if per_token_scales:

@@ -134,7 +134,7 @@ def test_attention_lazy_max(dev, attn_cfg, m, n, std):
 
 
 def test_attention_lazy_max_short_sequences_unchanged(dev):
-    """N <= 128 with unit scales runs the register-resident kernel, which knows the final maximum: lazy_max changes nothing"""
+    """N <= 128 runs the short-sequence kernel, which knows the final maximum: lazy_max changes nothing"""
     q, k, v = _inputs(3, 2, 2, 200, 100)
     a = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16)
     b = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16, lazy_max=True)
@@ -422,32 +422,45 @@ def test_zero_query_row_with_scales_and_masked_keys(dev, attn_cfg):
 
 
 @pytest.mark.parametrize("n,lens", [(128, [128, 16]), (100, [37, 100]), (64, [64, 1]), (17, [0, 17]), (1, [1, 1])])
-def test_register_resident_path_for_short_kv(dev, n, lens):
-    """N <= 128 with unit scales takes the kernel that keeps K and V^T in registers (single-pass softmax, no LDS). Same
-    bars as the general kernel, which is forced for comparison (config 3): both against the oracle, and against each
-    other within twice the rounding bound (they round P against different maxima)."""
+@pytest.mark.parametrize("scaled", [False, True])
+def test_short_kv_path(dev, n, lens, scaled):
+    """N <= 128 takes the kernel that keeps K and V of a (batch, head) in LDS and rounds P against the final maximum
+    (single-pass softmax), with unit scales and with per-token scales. Same bars as the general kernel, which is forced
+    for comparison (config 3): both against the oracle, and the two must differ somewhere when there are two key blocks
+    (they round P against different maxima), which shows that the two calls took different kernels."""
     from q8_kernels_amd import _lib
     b, h, m = 2, 3, 1000
-    q, k, v = _inputs(7000 + n, b, h, m, n)
+    if scaled:
+        g = torch.Generator().manual_seed(9000 + n)
+        qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)
+        kf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 4 + 0.2)
+        vf = torch.randn(b, h, n, 64, generator=g) * (torch.rand(b, h, n, 1, generator=g) * 2 + 0.5)
+        (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
+        kw = dict(q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
+        sc = (sq, sk, sv)
+    else:
+        q, k, v = _inputs(7000 + n, b, h, m, n)
+        kw, sc = {}, (None, None, None)
     l = torch.tensor(lens, dtype=torch.int32)
     args = (q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, l.to(dev))
-    short = _C().flash_attention(*args, out_dtype=torch.bfloat16)
+    short = _C().flash_attention(*args, out_dtype=torch.bfloat16, **kw)
     try:
         _lib.check(_lib.lib().q8_attn_set_config(3))
-        general = _C().flash_attention(*args, out_dtype=torch.bfloat16)
+        general = _C().flash_attention(*args, out_dtype=torch.bfloat16, **kw)
     finally:
         _lib.check(_lib.lib().q8_attn_set_config(0))
-    _check(short, q, k, v, 0.125, l, what="register-resident N=%d" % n)
-    _check(general, q, k, v, 0.125, l, what="general N=%d" % n)
+    _check(short, q, k, v, 0.125, l, sc, what="short KV N=%d" % n)
+    _check(general, q, k, v, 0.125, l, sc, what="general N=%d" % n)
     assert not torch.equal(short, general) or n <= 64, "both calls took the same kernel"
-    # token-major output, e4m3 output and the reference's P grid through the same path
-    tok = _C().flash_attention(*args, out_dtype=torch.bfloat16, token_major_out=True)
-    assert_equal = torch.equal(tok.view(b, m, h, 64).transpose(1, 2), short)
-    assert assert_equal, "token-major output differs"
-    o8 = _C().flash_attention(*args)
+    # token-major output, token-major V, e4m3 output and the reference's P grid through the same path
+    tok = _C().flash_attention(*args, out_dtype=torch.bfloat16, token_major_out=True, **kw)
+    assert torch.equal(tok.view(b, m, h, 64).transpose(1, 2), short), "token-major output differs"
+    vtok = _C().flash_attention(q.to(dev), k.to(dev), v.to(dev), 0.125, l.to(dev), out_dtype=torch.bfloat16, v_token_major=True, **kw)
+    assert torch.equal(vtok, short), "token-major V differs"
+    o8 = _C().flash_attention(*args, **kw)
     assert o8.dtype == E4M3 and ((o8.cpu().float() - short.cpu().float()).abs() <= 0.07 * short.cpu().float().abs() + 0.02).all()
-    unit = _C().flash_attention(*args, out_dtype=torch.bfloat16, p_unit_range=True)
-    _check(unit, q, k, v, 0.125, l, what="register-resident, p <= 1", p_scale=1.0)
+    unit = _C().flash_attention(*args, out_dtype=torch.bfloat16, p_unit_range=True, **kw)
+    _check(unit, q, k, v, 0.125, l, sc, what="short KV, p <= 1", p_scale=1.0)
 
 
 @pytest.mark.parametrize("m,n,lens", [(256, 64, None), (33, 17, None), (300, 640, None), (512, 1000, [1000, 333]),
