@@ -272,7 +272,7 @@ int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, cons
 
 /*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with
- * one tile per workgroup, 2 = 128x128 tiles, 4 = persistent pipelined 256x256 tiles (bf16 or e4m3 output, N % 8 == 0,
+ * one tile per workgroup, 2 = 128x128 tiles, 3 = 64x64 tiles, 4 = persistent pipelined 256x256 tiles (bf16 or e4m3 output, N % 8 == 0,
  * K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's tile to 192 / 256 rows /
  * back to automatic. It holds for the calling thread only; meant for tests and tuning, it has no counterpart in the
  * reference (whose tile is fixed at 128x128x64, csrc/gemm/fp8_matmul_bias.cu:426-429).
@@ -288,6 +288,7 @@ int q8_gemm_set_config(int cfg);
 enum {
     Q8_GEMM_KERNEL_PIPE256 = 1,    /* pipelined 256x256 tiles, one tile per workgroup */
     Q8_GEMM_KERNEL_TILE128 = 2,    /* 128x128 tiles                                    */
+    Q8_GEMM_KERNEL_TILE64 = 3,     /* 64x64 tiles (small problems)                     */
     Q8_GEMM_KERNEL_PERSIST256 = 4, /* persistent, 256-row tiles                        */
     Q8_GEMM_KERNEL_PERSIST192 = 5, /* persistent, 192-row tiles                        */
     Q8_GEMM_KERNEL_RESIDUAL = 16

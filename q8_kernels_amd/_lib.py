@@ -15,7 +15,7 @@ Q8_QUANT_RNE, Q8_QUANT_SCALE_DIV = 1, 2
 Q8_V_DS, Q8_V_SD = 0, 1
 Q8_ATTN_SUM_ROUNDED_P, Q8_ATTN_P_UNIT_RANGE, Q8_ATTN_O_TOKEN_MAJOR, Q8_ATTN_LAZY_MAX = 1, 2, 4, 8
 # values of q8_gemm_last_kernel (tests)
-Q8_GEMM_KERNEL_PIPE256, Q8_GEMM_KERNEL_TILE128 = 1, 2
+Q8_GEMM_KERNEL_PIPE256, Q8_GEMM_KERNEL_TILE128, Q8_GEMM_KERNEL_TILE64 = 1, 2, 3
 Q8_GEMM_KERNEL_PERSIST256, Q8_GEMM_KERNEL_PERSIST192, Q8_GEMM_KERNEL_RESIDUAL = 4, 5, 16
 
 _c = ctypes

@@ -4,7 +4,7 @@
 //
 // Structure of one workgroup (WAVES_M x WAVES_N waves, one BM x BN tile of C):
 //   * K is walked in steps of 128 bytes. A step's A rows (BM x 128 B) and B rows (BN x 128 B) are
-//     copied HBM -> LDS by `global_load_lds_dwordx4` (no VGPR staging), two LDS stages.
+//     copied HBM -> LDS by `global_load_lds_dwordx4` (no VGPR staging), four LDS stages, copies three steps ahead.
 //   * LDS holds plain 128-byte rows whose 16-byte chunks are XOR-swizzled by lds_swizzle(row). A
 //     ds_read_b128 is served in four passes of 16 lanes, and the lanes of one pass are NOT consecutive:
 //     measured on gfx950 they are {0-3, 12-15, 20-23, 24-27}, {4-7, 8-11, 16-19, 28-31} and the same
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
             src[i] = Bg + (size_t)n * K + c * 16;
         }
     }
-    auto issue_loads = [&](int stage, int k0) {
+    auto issue_loads = [&](int stage, int k0) {  // (k0 may lie past K: the whole step then comes from the block of zeros)
         uint8_t* base = lds + stage * C::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < C::PER_A + C::PER_B; ++i) {
@@ -92,41 +92,82 @@ __global__ __launch_bounds__(C::NT) void gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
+    // C::STAGES LDS stages and two sets of operand registers. In step kt the wave multiplies the operands of step kt, which
+    // it requested from LDS during step kt - 1, while the operands of step kt + 1 travel from LDS to the other register set
+    // and the copies of steps kt + 2 .. kt + STAGES - 1 travel from HBM to LDS. Every wave issues the same number of copies
+    // per step - past the end of K from a block of zeros - so "all but the (STAGES - 3) PER youngest copies" is exactly
+    // "step kt + 1 has landed". One barrier per step: it publishes step kt + 1 and says that everyone holds the operands
+    // of step kt - 1 (waited for before that step's multiplications), whose buffer the copies of step kt + STAGES - 1
+    // overwrite.
+    constexpr int PER = C::PER_A + C::PER_B, STAGES = C::STAGES;
+    static_assert(STAGES >= 4 && (STAGES - 3) * PER <= 63, "vmcnt holds 6 bits");
     const int KT = (K + 127) / 128;
-    issue_loads(0, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-        wait_vmcnt0();
-        __syncthreads();
-        const uint8_t* st = lds + (kt & 1) * C::STAGE_BYTES;
-        v4i a_lo[TM], a_hi[TM], b_lo[TN], b_hi[TN];
+    const unsigned lds0 = lds_addr(lds);
+    struct Frags { v4i a_lo[TM], a_hi[TM], b_lo[TN], b_hi[TN]; };
+    auto read_frags = [&](Frags& f, int stage) {
+        const unsigned st = lds0 + stage * C::STAGE_BYTES;
+        const unsigned br = st + b_row0 * 128, ar = st + a_row0 * 128;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const uint8_t* r = st + (b_row0 + 16 * j) * 128;
-            b_lo[j] = *reinterpret_cast<const v4i*>(r + pc0);
-            b_hi[j] = *reinterpret_cast<const v4i*>(r + pc1);
+            f.b_lo[j] = lds_read_b128<0>(br + 2048 * j + pc0);
+            f.b_hi[j] = lds_read_b128<0>(br + 2048 * j + pc1);
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const uint8_t* r = st + (a_row0 + 16 * i) * 128;
-            a_lo[i] = *reinterpret_cast<const v4i*>(r + pc0);
-            a_hi[i] = *reinterpret_cast<const v4i*>(r + pc1);
+            f.a_lo[i] = lds_read_b128<0>(ar + 2048 * i + pc0);
+            f.a_hi[i] = lds_read_b128<0>(ar + 2048 * i + pc1);
         }
-        if (kt + 1 < KT) issue_loads((kt + 1) & 1, (kt + 1) * 128);
+    };
+    auto wait_frags = [&](Frags& f) {  // every LDS read issued so far has landed; the registers of `f` pass through the wait
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(f.a_lo[i]), "+v"(f.a_hi[i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(f.b_lo[j]), "+v"(f.b_hi[j]));
+    };
+    auto multiply = [&](const Frags& f) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (C::IN == Q8_I8) {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b_lo[j], a_lo[i], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b_hi[j], a_hi[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f.b_lo[j], f.a_lo[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f.b_hi[j], f.a_hi[i], acc[i][j], 0, 0, 0);
                 } else {
-                    const v8i bf = {b_lo[j][0], b_lo[j][1], b_lo[j][2], b_lo[j][3], b_hi[j][0], b_hi[j][1], b_hi[j][2], b_hi[j][3]};
-                    const v8i af = {a_lo[i][0], a_lo[i][1], a_lo[i][2], a_lo[i][3], a_hi[i][0], a_hi[i][1], a_hi[i][2], a_hi[i][3]};
+                    const v8i bf = {f.b_lo[j][0], f.b_lo[j][1], f.b_lo[j][2], f.b_lo[j][3], f.b_hi[j][0], f.b_hi[j][1], f.b_hi[j][2], f.b_hi[j][3]};
+                    const v8i af = {f.a_lo[i][0], f.a_lo[i][1], f.a_lo[i][2], f.a_lo[i][3], f.a_hi[i][0], f.a_hi[i][1], f.a_hi[i][2], f.a_hi[i][3]};
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[i][j], 0, 0, 0, 0, 0, 0);
                 }
             }
         }
+    };
+    // one step: `cur` holds (in flight) the operands of step kt, `nxt` receives those of step kt + 1
+    auto step = [&](int kt, Frags& cur, Frags& nxt) {
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((STAGES - 3) * PER) : "memory");
+        __builtin_amdgcn_s_barrier();
+        issue_loads((kt + STAGES - 1) % STAGES, (kt + STAGES - 1) * 128);
+        wait_frags(cur);
+        read_frags(nxt, (kt + 1) % STAGES);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(cur);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int s = 0; s < STAGES - 2; ++s) issue_loads(s, s * 128);
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((STAGES - 3) * PER) : "memory");
+    __builtin_amdgcn_s_barrier();
+    issue_loads(STAGES - 2, (STAGES - 2) * 128);
+    Frags f0, f1;
+    read_frags(f0, 0);
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        step(kt, f0, f1);
+        step(kt + 1, f1, f0);
     }
+    if (kt < KT) step(kt, f0, f1);
+    // (the operand reads of the step past the last one target registers that nobody uses)
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f0.a_lo[0]), "+v"(f1.a_lo[0]) : : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the look-ahead copies past the last step
 
     // ---- epilogue: lane (mcol = lane%16, g = lane/16) holds, for tile (i, 2jj..2jj+1), row
     //      m = 16 i + mcol and the 8 columns 32 jj + 8 g + 0..7 of the wave's slab.
@@ -174,9 +215,10 @@ static int reserve_lds(const void* kern, int bytes, int& done_dev) {
 
 template <class C, int OUT, bool GELU>
 static int launch_gemm(const GemmParams& p, hipStream_t stream) {
-    g_last_kernel = Q8_GEMM_KERNEL_TILE128;
+    g_last_kernel = C::BM == 64 ? Q8_GEMM_KERNEL_TILE64 : Q8_GEMM_KERNEL_TILE128;
     const int tiles_m = (p.M + C::BM - 1) / C::BM, tiles_n = (p.N + C::BN - 1) / C::BN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
+    if ((long)tiles_m * tiles_n > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: grid too large");
     auto kern = gemm_kernel<C, OUT, GELU>;
     static thread_local int lds_dev = -1;
     if (int st = reserve_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES, lds_dev)) return st;
@@ -184,13 +226,19 @@ static int launch_gemm(const GemmParams& p, hipStream_t stream) {
     return launch_status("q8_gemm");
 }
 
-// Tile selection: pipelined 256x256 tiles (gemm_pipe.h / gemm_persist.h) for large problems, this file's 128x128 tiles
-// (4 waves of 64x64) when the large tile would leave most of the 256 CUs idle.
+// Tile selection: pipelined 256x256 tiles (gemm_pipe.h / gemm_persist.h) for large problems, this file's 128x128 or 64x64
+// tiles when the large tile would leave most of the 256 CUs idle.
+// Two shapes (measured on 2048-deep problems; a K step costs about in proportion to the tile's bytes, so what counts is
+// how many CUs the tiles reach): 8 waves (2 x 4, wave tiles of 64 x 32) on 128x128 tiles, and 4 waves (2 x 2, wave tiles
+// of 32 x 32) on 64x64 tiles, two workgroups per CU, for problems with at most 512 such tiles - 256 x 4096 x 2048: 8.5 us
+// against 12.5 us, 2048 x 2048 x 2048: 19.2 us against 14.6 us.
 template <int IN>
-using CfgSmall = GemmCfg<IN, 2, 2, 4, 4>;
+using CfgSmall = GemmCfg<IN, 2, 4, 4, 2>;
+template <int IN>
+using CfgSmall64 = GemmCfg<IN, 2, 2, 2, 2>;
 
 // per-thread override (q8_gemm_set_config): 0 = auto, 1 = pipelined 256x256 (one tile per workgroup), 2 = 128x128,
-// 4 = persistent pipelined 256x256 where eligible
+// 3 = 64x64, 4 = persistent pipelined 256x256 where eligible
 static thread_local int g_force_cfg = 0;
 
 template <int IN, int OUT, bool GELU>
@@ -276,6 +324,8 @@ static int dispatch_tile(const GemmParams& p, hipStream_t stream) {
         if (big && g_force_cfg != 1 && persist_eligible(p)) return launch_persist<IN, GELU, OUT == Q8_E4M3>(p, stream);
     }
     if (big) return launch_pipe<IN, OUT, GELU>(p, stream);
+    const long tiles64 = (long)((p.M + 63) / 64) * ((p.N + 63) / 64) * (p.batch_a > p.batch_b ? p.batch_a : p.batch_b);
+    if (g_force_cfg == 3 || (g_force_cfg == 0 && tiles64 <= 512)) return launch_gemm<CfgSmall64<IN>, OUT, GELU>(p, stream);
     return launch_gemm<CfgSmall<IN>, OUT, GELU>(p, stream);
 }
 
@@ -307,7 +357,7 @@ extern "C" int q8_gemm_last_kernel(void) { return g_last_kernel; }
 
 extern "C" int q8_gemm_set_config(int cfg) {
     if (cfg == 43 || cfg == 44 || cfg == 40) { g_persist_mt = cfg - 40; return Q8_OK; }  // tuning: persistent tile height
-    if (cfg < 0 || cfg > 4 || cfg == 3) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
+    if (cfg < 0 || cfg > 4) return fail(Q8_ERR_FLAGS, "q8_gemm_set_config: %d", cfg);
     g_force_cfg = cfg;
     return Q8_OK;
 }

@@ -24,7 +24,7 @@ __device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0
 constexpr int Q8_OUT_I32 = 100;  // raw accumulators (int8 only)
 constexpr int kGroupM = 4;
 
-template <int IN_, int WAVES_M_, int WAVES_N_, int TM_, int TN_>
+template <int IN_, int WAVES_M_, int WAVES_N_, int TM_, int TN_, int STAGES_ = 4>
 struct GemmCfg {
     static constexpr int IN = IN_;
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, TM = TM_, TN = TN_;
@@ -34,7 +34,8 @@ struct GemmCfg {
     static constexpr int BN = WAVES_N * TN * 16;
     static constexpr int BK = 128;
     static constexpr int STAGE_BYTES = (BM + BN) * BK;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int STAGES = STAGES_;  // LDS ring of the HBM -> LDS copies
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     static constexpr int RG_A = BM / 8, RG_B = BN / 8;  // 1 KiB row groups per stage
     static constexpr int PER_A = RG_A / NW, PER_B = RG_B / NW;
     static_assert(RG_A % NW == 0 && RG_B % NW == 0, "row groups must divide over the waves");

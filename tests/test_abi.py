@@ -34,7 +34,7 @@ def test_header_enums_match_python_constants():
     text = open(HEADER).read()
     for name in ("Q8_I8", "Q8_E4M3", "Q8_BF16", "Q8_F16", "Q8_F32", "Q8_QUANT_RNE", "Q8_QUANT_SCALE_DIV",
                  "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR", "Q8_ATTN_LAZY_MAX",
-                 "Q8_GEMM_KERNEL_PIPE256", "Q8_GEMM_KERNEL_TILE128", "Q8_GEMM_KERNEL_PERSIST256",
+                 "Q8_GEMM_KERNEL_PIPE256", "Q8_GEMM_KERNEL_TILE128", "Q8_GEMM_KERNEL_TILE64", "Q8_GEMM_KERNEL_PERSIST256",
                  "Q8_GEMM_KERNEL_PERSIST192", "Q8_GEMM_KERNEL_RESIDUAL"):
         m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
         assert m, name

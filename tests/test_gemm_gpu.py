@@ -21,7 +21,7 @@ def _set_cfg(c):
 
 from q8_kernels_amd._lib import (Q8_GEMM_KERNEL_PERSIST192 as K_PERSIST192, Q8_GEMM_KERNEL_PERSIST256 as K_PERSIST256,  # noqa: E402
                                  Q8_GEMM_KERNEL_PIPE256 as K_PIPE256, Q8_GEMM_KERNEL_RESIDUAL as K_RESIDUAL,
-                                 Q8_GEMM_KERNEL_TILE128 as K_TILE128)
+                                 Q8_GEMM_KERNEL_TILE128 as K_TILE128, Q8_GEMM_KERNEL_TILE64 as K_TILE64)
 
 
 PERSISTENT_KERNELS = {K_PERSIST256, K_PERSIST192}  # the workgroup-per-CU kernels that walk over several tiles
@@ -33,7 +33,7 @@ def _last_kernel():
 
 
 def _kernels_for(cfg, n, k, bf16_out=True):
-    """The kernels a call may launch under q8_gemm_set_config(cfg): the pins 1 and 2 always hold; 4 means the
+    """The kernels a call may launch under q8_gemm_set_config(cfg): the pins 1, 2 and 3 always hold; 4 means the
     persistent kernel for the shapes it takes (bf16 or e4m3 output, N % 8 == 0, K a multiple of 128 above 256) and the
     per-tile pipelined kernel otherwise. Asserted after the calls below so that a test of a pinned kernel cannot
     pass on a silent fall-back to another one."""
@@ -41,11 +41,13 @@ def _kernels_for(cfg, n, k, bf16_out=True):
         return {K_PIPE256}
     if cfg == 2:
         return {K_TILE128}
+    if cfg == 3:
+        return {K_TILE64}
     eligible = bf16_out and n % 8 == 0 and k > 256 and k % 128 == 0
     return {K_PERSIST256, K_PERSIST192} if eligible else {K_PIPE256}
 
 
-@pytest.fixture(params=[1, 2, 4], ids=["tile256", "tile128", "persistent256"])
+@pytest.fixture(params=[1, 2, 3, 4], ids=["tile256", "tile128", "tile64", "persistent256"])
 def tile_cfg(request):
     _set_cfg(request.param)
     yield request.param
