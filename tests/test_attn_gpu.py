@@ -463,6 +463,26 @@ def test_short_kv_path(dev, n, lens, scaled):
     _check(unit, q, k, v, 0.125, l, sc, what="short KV, p <= 1", p_scale=1.0)
 
 
+@pytest.mark.parametrize("b,h,m,n,lens", [(5, 2, 200, 100, [100, 0, 64, 7, 65]), (3, 40, 2500, 128, [128, 1, 90]),
+                                          (1, 1, 31, 128, [128]), (4, 1, 70, 65, None)])
+def test_short_kv_batches_and_tile_walk(dev, b, h, m, n, lens):
+    """The short-sequence kernel over more than two batches (the LDS halves alternate, a batch without valid keys lies
+    between batches with one and two key blocks), several tiles per wave with a ragged last tile, and more workgroups
+    than fit the device at once: against the oracle for every batch, and a batch's output must not depend on what the
+    other batches hold (each batch alone gives the same bits)."""
+    q, k, v = _inputs(8100 + b * 7 + m, b, h, m, n)
+    l = None if lens is None else torch.tensor(lens, dtype=torch.int32)
+    ld = None if l is None else l.to(dev)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, ld, out_dtype=torch.bfloat16)
+    _check(got[:, :2], q[:, :2], k[:, :2], v[:, :2], 0.125, l, what="short KV b=%d h=%d m=%d n=%d" % (b, h, m, n))
+    if lens is not None and 0 in lens:
+        assert (got[lens.index(0)] == 0).all(), "a batch without valid keys gives zeros"
+    for i in range(b):
+        alone = _C().flash_attention(q[i:i + 1].to(dev), k[i:i + 1].to(dev), _vt(v[i:i + 1]).to(dev), 0.125,
+                                     None if ld is None else ld[i:i + 1].contiguous(), out_dtype=torch.bfloat16)
+        assert torch.equal(alone[0], got[i]), "batch %d depends on its neighbours" % i
+
+
 @pytest.mark.parametrize("m,n,lens", [(256, 64, None), (33, 17, None), (300, 640, None), (512, 1000, [1000, 333]),
                                       (130, 128, [128, 5]), (70, 200, [0, 200]), (1, 1, None), (257, 6144, None)])
 @pytest.mark.parametrize("scaled", [False, True])
