@@ -211,6 +211,9 @@ int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, int apply_nor
  * q8_attn_prep_qkv: q8_attn_prep_qk_pair, and the V projection xv of the same tokens is cast in the same pass to
  *   e4m3 codes [B, H, S, D] (token-major per head: the Q8_V_SD operand of q8_attn_fwd, no transposed copy);
  *   scales_v [B, H, S] together with scales_q / scales_k, or all three NULL for the direct c10 cast.
+ * q8_attn_prep_kv: q8_attn_prep_qk on the K projection xk, and the V projection xv of the same tokens is cast in the
+ *   same pass to token-major e4m3 codes like in q8_attn_prep_qkv: the keys and values of a cross-attention (whose
+ *   queries are other tokens) in one launch.
  * q8_attn_prep_v: e4m3 codes [B, H, D, S_pad] (Q8_V_DS), columns S..S_pad-1 zero, S_pad % 16 == 0;
  *   scales as above. D == 64.
  */
@@ -226,6 +229,9 @@ int q8_attn_prep_qkv(const void* xq, int64_t xq_row_stride, const void* xk, int6
                      const float* sin_t, void* codes_q, float* scales_q, void* codes_k, float* scales_k, void* codes_v,
                      float* scales_v, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
                      q8_stream_t stream);
+int q8_attn_prep_kv(const void* xk, int64_t xk_row_stride, const void* xv, int64_t xv_row_stride, const float* norm_wk,
+                    const float* cos_t, const float* sin_t, void* codes_k, float* scales_k, void* codes_v, float* scales_v,
+                    int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype, q8_stream_t stream);
 int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
                    int S_pad, q8_stream_t stream);
 

@@ -547,6 +547,35 @@ def attn_prep_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: 
     return ((cq, sq), (ck, sk_), (cv, sv_)) if per_token_scales else (cq, ck, cv)
 
 
+def attn_prep_kv(k: torch.Tensor, v: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
+                 sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
+                 per_token_scales: bool = False, *, round_intermediate: bool = True,
+                 norm_weight: Optional[torch.Tensor] = None):
+    """attn_prep_qk on k, and the V projection of the same tokens is cast to e4m3 in the same pass, token-major per head
+    ([B, H, S, D], what flash_attention takes with v_token_major=True): keys and values of a cross-attention in one
+    launch. Returns (k_out, v_out), each codes or (codes, scales [B, H, S]) with per_token_scales."""
+    k, b, s, d = _token_major(k, num_heads, "attn_prep_kv")
+    v, bv, sv, dv = _token_major(v, num_heads, "attn_prep_kv")
+    if (bv, sv, dv) != (b, s, d):
+        raise RuntimeError("attn_prep_kv: k and v must have the same shape")
+    if (cos is None) != (sin is None):
+        raise RuntimeError("attn_prep_kv: cos and sin come together")
+    if cos is not None:
+        for t in (cos, sin):
+            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != k.numel():
+                raise RuntimeError("attn_prep_kv: tables must be float32 CUDA tensors of k's shape")
+        cos, sin = cos.contiguous(), sin.contiguous()
+    mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=k.device)  # noqa: E731
+    mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=k.device) if per_token_scales else None  # noqa: E731
+    ck, cv, sk_, sv_ = mk(), mk(), mks(), mks()
+    nw = _norm_w(norm_weight, k)  # bound to a name: alive across the launch
+    with torch.cuda.device(k.device):
+        _lib.check(_lib.lib().q8_attn_prep_kv(k.data_ptr(), k.stride(1), v.data_ptr(), v.stride(1), _ptr(nw), _ptr(cos), _ptr(sin),
+                                              ck.data_ptr(), _ptr(sk_), cv.data_ptr(), _ptr(sv_), b, s, num_heads, d,
+                                              int(apply_fht), float(scale), Q8_BF16 if round_intermediate else Q8_F32, _stream(k)))
+    return ((ck, sk_), (cv, sv_)) if per_token_scales else (ck, cv)
+
+
 def attn_prep_v(x: torch.Tensor, num_heads: int, per_token_scales: bool = False):
     """x [B, S, H*64] bfloat16 -> e4m3 [B, H, 64, S_pad] (S_pad = S rounded up to 16, zero filled), the V operand
     of flash_attention; with per_token_scales also scales [B, H, S]."""

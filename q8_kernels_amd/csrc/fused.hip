@@ -574,6 +574,16 @@ extern "C" int q8_attn_prep_qkv(const void* xq, int64_t xq_row_stride, const voi
                              static_cast<hipStream_t>(stream_));
 }
 
+extern "C" int q8_attn_prep_kv(const void* xk, int64_t xk_row_stride, const void* xv, int64_t xv_row_stride, const float* norm_wk,
+                               const float* cos_t, const float* sin_t, void* codes_k, float* scales_k, void* codes_v,
+                               float* scales_v, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                               q8_stream_t stream_) {
+    if (!xv) return fail(Q8_ERR_NULL, "q8_attn_prep_kv: null pointer");
+    return attn_prep_qk_impl("q8_attn_prep_kv", xk, xk_row_stride, nullptr, 0, norm_wk, nullptr, cos_t, sin_t, codes_k, scales_k, nullptr,
+                             nullptr, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, apply_fht, scale, mid_dtype,
+                             static_cast<hipStream_t>(stream_));
+}
+
 extern "C" int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
                               int S_pad, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);

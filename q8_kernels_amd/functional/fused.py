@@ -83,6 +83,19 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
                                       v_scales=vs, token_major_out=True, v_token_major=True)
         return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
                                   v_token_major=True)
+    if k.shape == v.shape and d == 64:
+        # other queries than keys (cross-attention): the queries alone, keys and values together in a second launch, V
+        # token-major again
+        qc = _C.attn_prep_qk(q, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                             norm_weight=q_norm_weight)
+        kc, vc = _C.attn_prep_kv(k, v, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
+                                 norm_weight=k_norm_weight)
+        if per_token_scales:
+            (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
+            return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
+                                      v_scales=vs, token_major_out=True, v_token_major=True)
+        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                  v_token_major=True)
     if q.shape == k.shape:  # one pass over q and k
         qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
                                       q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)

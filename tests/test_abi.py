@@ -114,6 +114,12 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
                               1, 5, 8, 64, 1, 1.0, B16, None) == -4                                  # V not 16-byte aligned
     assert L.q8_attn_prep_qkv(16, 512, 16, 512, 16, 512, None, None, None, None, 16, None, 16, None, 16, None,
                               0, 5, 8, 64, 1, 1.0, B16, None) == 0                                   # no tokens: nothing to do
+    # q8_attn_prep_kv(xk, sk, xv, sv, nwk, cos, sin, ck, sck, cv, scv, B, S, H, D, fht, scale, mid, stream)
+    assert L.q8_attn_prep_kv(None, 512, None, 512, None, None, None, None, None, None, None, 0, 5, 8, 64, 1, 1.0, B16, None) == -1  # no V
+    assert L.q8_attn_prep_kv(None, 512, 16, 512, None, None, None, None, None, None, None, 0, 5, 8, 64, 1, 1.0, B16, None) == 0    # no tokens
+    assert L.q8_attn_prep_kv(16, 512, 16, 512, None, None, None, 16, None, None, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1       # no V codes
+    assert L.q8_attn_prep_kv(16, 512, 16, 500, None, None, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -3        # V stride
+    assert L.q8_attn_prep_kv(16, 512, 16, 512, None, None, None, 16, 16, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1          # scales of K only
     assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 64, 5, None) == -3                          # S_pad % 16
     assert L.q8_attn_prep_v(16, 512, 16, None, 1, 5, 8, 128, 16, None) == -3
     assert L.q8_gemm_residual(16, 16, None, 16, 16, None, 16, 1, 1, 8, 8, 384, I8, 0, None) == -1

@@ -247,6 +247,31 @@ def test_attn_prep_qkv_equals_pair_plus_cast_of_v(dev, shape, scaled):
         assert_bit_equal(gv, O.e4m3_c10(vh), "v codes")
 
 
+@pytest.mark.parametrize("shape", [(2, 128, 32, 64), (1, 33, 8, 64), (3, 5, 1, 64), (2, 19, 8, 128)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_kv_equals_single_call_plus_cast_of_v(dev, shape, scaled):
+    """Keys and values of a cross-attention in one launch (strided slices of a fused K/V projection): K as attn_prep_qk
+    gives it, V as the e4m3 cast (or per (token, head) quantisation) of its heads, token-major [B, H, S, D]."""
+    b, s, h, d = shape
+    g = torch.Generator().manual_seed(s * 13 + h)
+    kv = (torch.randn(b, s, 2 * h * d, generator=g) * 1.5).to(BF16)
+    kv[0, s // 3] = 0
+    kv_d = kv.to(dev)
+    k, v = kv_d[..., :h * d], kv_d[..., h * d:]
+    w = (torch.rand(h * d, generator=g) + 0.5).to(dev)
+    gk, gv = _C().attn_prep_kv(k, v, h, None, None, True, 0.125, scaled, norm_weight=w)
+    wk = _C().attn_prep_qk(k, h, None, None, True, 0.125, scaled, norm_weight=w)
+    vh = kv[..., h * d:].reshape(b, s, h, d).transpose(1, 2).contiguous()
+    if scaled:
+        wv = O.ref_quant(vh, E4M3)
+        for got, want, what in ((gk, wk, "k"), (gv, wv, "v")):
+            assert_bit_equal(got[0], want[0], what + " codes")
+            assert_bit_equal(got[1], want[1], what + " scales")
+    else:
+        assert_bit_equal(gk, wk, "k codes")
+        assert_bit_equal(gv, O.e4m3_c10(vh), "v codes")
+
+
 def test_attn_prep_qk_strided_slice_of_fused_projection(dev):
     g = torch.Generator().manual_seed(77)
     qkv = torch.randn(2, 50, 3 * 2048, generator=g).to(BF16)
