@@ -50,7 +50,8 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 // Requirements checked by the host: K % 128 == 0 and K > 256 (at least 3 whole stages per tile), N % 8 == 0,
 // M * K and N * K below 2^32 (32-bit source offsets).
 // E4M3OUT: the output is e4m3 (saturating cast, the reference's default output type, csrc/gemm/q8_gemm_api.cpp:82-87) instead
-// of bf16: every lane stores its 8-byte chunks straight from the MFMA layout (no residual form).
+// of bf16: the lanes store their codes straight from the MFMA layout, 16 bytes each after a swap between the two lanes of
+// a row (no residual form).
 // MT = 32-row MFMA tiles per wave along M: the tile is 64 MT x 256, i.e. 256 x 256 (MT = 4) or 192 x 256 (MT = 3, for
 // problems whose 256-row tiles do not divide evenly over the CUs).
 // RES: C = bf16(bf16(result) + residual), the residual connection around a projection (two roundings, as the separate
@@ -285,6 +286,8 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                        "+v"(bq[1][0][0]), "+v"(bq[1][0][1]), "+v"(bq[1][1][0]), "+v"(bq[1][1][1])
                      :
                      : "memory");
+        const bool rows16 = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;  // e4m3 output: rows start 16-byte aligned
+        (void)rows16;
         uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
         const uint16_t* const rbase = reinterpret_cast<const uint16_t*>(p.residual) + zc;
         v4i gq = v4i{0, 0, 0, 0};  // the gate of the 8 columns this lane stores (RES with p.gate)
@@ -312,7 +315,9 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             // the lane's 4 chunks of row 32 i + r32: chunk c = 4 t + 2 wp + h
             v4u outc[2][2];
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t) {
+                uint32_t e8[2][2];  // e4m3 output: [wp][low / high 4 codes]
+                (void)e8;
 #pragma unroll
                 for (int wp = 0; wp < 2; ++wp) {
                     float v[8];
@@ -325,14 +330,35 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         v[e] = x;
                     }
                     if constexpr (E4M3OUT) {
-                        // 8 codes of row 32 i + r32; the two lane halves write 16 contiguous bytes of the row
-                        const int m = mw0 + 32 * i + r32, n = nw0 + 32 * t + 16 * wp + 8 * h;
-                        const v2i w = v2i{(int)pack4_e4m3_sat(v[0], v[1], v[2], v[3]), (int)pack4_e4m3_sat(v[4], v[5], v[6], v[7])};
-                        if (m < M && n < N) *reinterpret_cast<v2i*>(reinterpret_cast<uint8_t*>(p.C) + zc + (size_t)m * N + n) = w;
+                        // 8 codes of row 32 i + r32, columns 32 t + 16 wp + 8 h .. + 7 of the slab
+                        e8[wp][0] = pack4_e4m3_sat(v[0], v[1], v[2], v[3]);
+                        e8[wp][1] = pack4_e4m3_sat(v[4], v[5], v[6], v[7]);
                     } else {
                         outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
                     }
                 }
+                if constexpr (E4M3OUT) {
+                    // the two lanes of a row exchange one 8-byte chunk each (v_permlane32_swap: the upper half of the first
+                    // operand against the lower half of the second): lane half 0 then holds columns 32 t .. + 15, lane
+                    // half 1 columns 32 t + 16 .. + 31, 16 bytes per lane and 32 contiguous bytes per row and instruction
+                    // (only when every row starts on a 16-byte boundary, N % 16 == 0 and C aligned - uniform; otherwise each
+                    //  lane stores its two 8-byte chunks where they are)
+                    const int m = mw0 + 32 * i + r32;
+                    uint8_t* const row = reinterpret_cast<uint8_t*>(p.C) + zc + (size_t)m * N;
+                    if (rows16) {
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(e8[0][0], e8[1][0], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(e8[0][1], e8[1][1], false, false);
+                        const int n = nw0 + 32 * t + 16 * h;
+                        if (m < M && n < N) *reinterpret_cast<v4u*>(row + n) = v4u{s0[0], s1[0], s0[1], s1[1]};
+                    } else {
+#pragma unroll
+                        for (int wp = 0; wp < 2; ++wp) {
+                            const int n = nw0 + 32 * t + 16 * wp + 8 * h;
+                            if (m < M && n < N) *reinterpret_cast<v2i*>(row + n) = v2i{(int)e8[wp][0], (int)e8[wp][1]};
+                        }
+                    }
+                }
+            }
             if constexpr (E4M3OUT) {
                 continue;
             } else if constexpr (GELU && !RES) {
