@@ -60,6 +60,12 @@ __device__ __forceinline__ uint32_t e4m3_overflow_fix(uint32_t code, float v) {
 __device__ __forceinline__ uint32_t pack4_e4m3_c10(float a, float b, float c, float d) {
     uint32_t p = cvt_pk_e4m3(a, b, 0u, false);
     p = cvt_pk_e4m3(c, d, p, true);
+    // Up to |v| = 464 the hardware conversion IS the c10 cast; only larger magnitudes and NaN need the code patched in.
+    // One maximum of the four magnitudes and two unordered comparisons say whether any value of any lane is such a one,
+    // and only then the wave runs the per-byte repair below (same codes either way).
+    const float m = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b)), __builtin_fmaxf(__builtin_fabsf(c), __builtin_fabsf(d)));
+    const bool rare = !(m <= 464.f) || __builtin_isunordered(a, b) || __builtin_isunordered(c, d);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(rare) == 0, 1)) return p;
     uint32_t b0 = e4m3_overflow_fix(p & 0xffu, a);
     uint32_t b1 = e4m3_overflow_fix((p >> 8) & 0xffu, b);
     uint32_t b2 = e4m3_overflow_fix((p >> 16) & 0xffu, c);
