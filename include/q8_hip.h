@@ -277,6 +277,18 @@ int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, cons
                            int in_dtype, int fuse_gelu, q8_stream_t stream);
 
 /*
+ * q8_gemm for a fused QKV projection whose V part feeds the attention kernel directly: columns n < v_col0 (Q and K) are
+ * written as bf16 to C [M, v_col0]; columns n >= v_col0 (V, heads of 64) are rounded to bf16 like the others, cast to e4m3
+ * (the c10 cast of q8_kernels/functional/flash_attention.py:38-45) and written token-major per head to v_codes
+ * [M / tokens, (N - v_col0) / 64, tokens, 64], the Q8_V_SD operand of q8_attn_fwd: the V output of q8_attn_prep_qkv without
+ * the bf16 round trip through memory (the fourth fusion the reference's launch boundaries allow around the attention,
+ * q8_kernels/modules/attention.py:67-105). M rows = batch elements of `tokens` tokens each. Runs on the persistent kernel
+ * only: N % 8 == 0, K % 128 == 0, K > 256; v_col0 a multiple of 256, N - v_col0 a multiple of 64 (Q8_ERR_SHAPE otherwise).
+ */
+int q8_gemm_qkv(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C, void* v_codes,
+                int M, int N, int K, int v_col0, int tokens, int in_dtype, q8_stream_t stream);
+
+/*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with
  * one tile per workgroup, 2 = 128x128 tiles, 3 = 64x64 tiles, 4 = persistent pipelined 256x256 tiles (bf16 or e4m3 output, N % 8 == 0,
  * K % 128 == 0, K > 256; other calls fall back to 1); 43 / 44 / 40 pin the persistent kernel's tile to 192 / 256 rows /

@@ -264,6 +264,41 @@ def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optio
     return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias", residual, gate)
 
 
+def mm_bias_qkv(a, b, bias, a_scales, b_scales, tokens: int, v_col0: int):
+    """The GEMM of a fused QKV projection with the cast of V in its epilogue: a [B*S, K] codes (int8 or e4m3, rows of B
+    batch elements of `tokens` tokens), b [N, K], fp32 bias [N] or None, fp32 row / column scales. Returns (qk, v_codes):
+    qk bfloat16 [B, S, v_col0] (the Q and K columns as q8_mm_bias / fp8_mm_bias give them) and v_codes e4m3
+    [B, (N - v_col0) / 64, S, 64], the bf16-rounded V columns cast to e4m3 token-major per head, what attn_prep_qkv
+    produces from the bfloat16 projection and flash_attention takes with v_token_major=True."""
+    _check_input(a, "a")
+    _check_input(b, "b")
+    if a.dtype != b.dtype or a.dtype not in (torch.int8, torch.float8_e4m3fn) or a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise RuntimeError("mm_bias_qkv: a [M,K] and b [N,K] must both be int8 or e4m3 with equal K")
+    m, k, n = a.shape[0], a.shape[1], b.shape[0]
+    if tokens <= 0 or m % tokens != 0:
+        raise RuntimeError("mm_bias_qkv: %d rows are not batch elements of %d tokens" % (m, tokens))
+    for t, name, cnt in ((a_scales, "a_scales", m), (b_scales, "b_scales", n)):
+        _check_input(t, name)
+        if t.dtype != torch.float32 or t.numel() != cnt:
+            raise RuntimeError("mm_bias_qkv: %s must be float32 with %d elements" % (name, cnt))
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.dtype != torch.float32 or bias.numel() != n:
+            raise RuntimeError("mm_bias_qkv: bias must be float32 with %d elements" % n)
+    if not (0 < v_col0 < n) or (n - v_col0) % 64 != 0:
+        raise RuntimeError("mm_bias_qkv: v_col0 = %d does not split N = %d into Q/K columns and heads of 64" % (v_col0, n))
+    bsz = m // tokens
+    qk = torch.empty((bsz, tokens, v_col0), dtype=torch.bfloat16, device=a.device)
+    vc = torch.empty((bsz, (n - v_col0) // 64, tokens, 64), dtype=torch.float8_e4m3fn, device=a.device)
+    if m == 0:
+        return qk, vc
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().q8_gemm_qkv(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
+                                          qk.data_ptr(), vc.data_ptr(), m, n, k, v_col0, tokens,
+                                          Q8_I8 if a.dtype == torch.int8 else Q8_E4M3, _stream(a)))
+    return qk, vc
+
+
 def q8_mm_i32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """Raw int32 accumulators a @ b.T of the int8 GEMM mainloop (2-D operands), for bit-exact checks."""
     _check_input(a, "a")

@@ -11,6 +11,7 @@ reaches through its modules; AdaLN modulation and the qk-RMSNorm of that block a
 import torch
 import torch.nn as nn
 
+from .. import _C
 from .. import functional as Q8F
 from ..modules.linear import FP8Linear
 from ..modules.rms_norm import RMSNorm
@@ -81,9 +82,18 @@ class Fp8DiTBlock(nn.Module):
         bf16 = torch.bfloat16
         d, h = self.dim, self.num_heads
         # self-attention: q, k, v are read in place from the fused projection by the attention prologue kernels
-        qkv = self._norm_lin(self.norm1, self.to_qkv, hidden)
-        a = Q8F.fused.flash_attn_token_major(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], h,
-                                             apply_qk_hadamard=True, freqs_cis=freqs_cis, out_dtype=bf16)
+        if self.head_dim == 64 and d > 256 and d % 128 == 0:
+            # the V columns leave the projection's GEMM as the attention kernel's e4m3 operand, token-major per head
+            # (shapes of the persistent GEMM kernel: K = d a multiple of 128 above 256, the split 2 d on a tile boundary)
+            codes, scales = Q8F.fused.rms_norm_quantize(hidden, self.norm1.weight, torch.float8_e4m3fn)
+            qk, v_codes = _C.mm_bias_qkv(codes.reshape(-1, d), self.to_qkv.weight.data, self.to_qkv.bias.data, scales.reshape(-1),
+                                         self.to_qkv.scales, hidden.shape[1], 2 * d)
+            a = Q8F.fused.flash_attn_token_major(qk[..., :d], qk[..., d:], None, h, apply_qk_hadamard=True,
+                                                 freqs_cis=freqs_cis, out_dtype=bf16, v_codes=v_codes)
+        else:
+            qkv = self._norm_lin(self.norm1, self.to_qkv, hidden)
+            a = Q8F.fused.flash_attn_token_major(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], h,
+                                                 apply_qk_hadamard=True, freqs_cis=freqs_cis, out_dtype=bf16)
         hidden = self._lin(self.to_out, a, residual=hidden)
         # cross-attention to the text states
         q2 = self._norm_lin(self.norm2, self.to_q2, hidden)

@@ -276,14 +276,14 @@ static int persist_cus() {
     return cus;
 }
 
-template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT>
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT, bool VSPLIT = false>
 static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     constexpr int BM = 64 * MT;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
     const int batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     const long total = (long)tiles_m * tiles_n * batch;
     if (total > 0x7fffffffL) return fail(Q8_ERR_SHAPE, "q8_gemm: too many tiles");
-    auto kern = gemm_persist_kernel<IN, GELU, MT, RES, E4M3OUT>;
+    auto kern = gemm_persist_kernel<IN, GELU, MT, RES, E4M3OUT, VSPLIT>;
     g_last_kernel = (MT == 4 ? Q8_GEMM_KERNEL_PERSIST256 : Q8_GEMM_KERNEL_PERSIST192) | (RES ? Q8_GEMM_KERNEL_RESIDUAL : 0);
     static thread_local int lds_dev = -1;
     if (int st = reserve_lds(reinterpret_cast<const void*>(kern), kPersistLds, lds_dev)) return st;
@@ -304,6 +304,10 @@ static int launch_persist(const GemmParams& p, hipStream_t stream) {
         return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? 1.0 : 1.2);
     };
     const bool small = g_persist_mt == 3 || (g_persist_mt == 0 && cost(192) < cost(256));
+    if constexpr (!E4M3OUT && !GELU) {
+        if (p.v_codes != nullptr)
+            return small ? launch_persist_mt<IN, false, 3, false, false, true>(p, stream) : launch_persist_mt<IN, false, 4, false, false, true>(p, stream);
+    }
     if constexpr (!E4M3OUT) {
         if (p.residual != nullptr)
             return small ? launch_persist_mt<IN, GELU, 3, true, false>(p, stream) : launch_persist_mt<IN, GELU, 4, true, false>(p, stream);
@@ -400,6 +404,30 @@ extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias,
         return fail(Q8_ERR_SHAPE, "q8_gemm_residual: needs N %% 8 == 0 and K a multiple of 128 above 256 (N %d K %d)", N, K);
     if (in_dtype == Q8_I8) return fuse_gelu ? launch_persist<Q8_I8, true>(p, stream) : launch_persist<Q8_I8, false>(p, stream);
     return fuse_gelu ? launch_persist<Q8_E4M3, true>(p, stream) : launch_persist<Q8_E4M3, false>(p, stream);
+}
+
+extern "C" int q8_gemm_qkv(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C, void* v_codes,
+                           int M, int N, int K, int v_col0, int tokens, int in_dtype, q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "q8_gemm_qkv";
+    if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;
+    if (int st = check_gemm(who, A, B, C, 1, 1, M, N, K)) return st;
+    if (!sa || !sb || !v_codes) return fail(Q8_ERR_NULL, "%s: scales and v_codes are required", who);
+    if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "%s: input dtype %d", who, in_dtype);
+    if ((reinterpret_cast<uintptr_t>(C) % 16) || (reinterpret_cast<uintptr_t>(v_codes) % 16))
+        return fail(Q8_ERR_ALIGN, "%s: C and v_codes must be 16-byte aligned", who);
+    // whole 256-column tiles on either side of the split, whole heads of 64 in the V part, whole batch elements in M
+    if (v_col0 <= 0 || v_col0 >= N || v_col0 % 256 != 0 || (N - v_col0) % 64 != 0)
+        return fail(Q8_ERR_SHAPE, "%s: v_col0 = %d must be a multiple of 256 inside N = %d with N - v_col0 a multiple of 64", who, v_col0, N);
+    if (tokens <= 0 || M % tokens != 0) return fail(Q8_ERR_SHAPE, "%s: M = %d must be a multiple of tokens = %d", who, M, tokens);
+    GemmParams p{static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), bias, sa, sb, C, 1, 1, M, N, K};
+    p.v_codes = static_cast<uint8_t*>(v_codes);
+    p.v_col0 = v_col0;
+    p.v_tokens = tokens;
+    p.v_heads = (N - v_col0) / 64;
+    if (!persist_eligible(p))
+        return fail(Q8_ERR_SHAPE, "%s: needs N %% 8 == 0 and K a multiple of 128 above 256 (N %d K %d)", who, N, K);
+    return in_dtype == Q8_I8 ? launch_persist<Q8_I8, false>(p, stream) : launch_persist<Q8_E4M3, false>(p, stream);
 }
 
 extern "C" int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, const float* sa, const float* sb,

@@ -17,6 +17,11 @@ struct GemmParams {
     const void* residual = nullptr;  // bf16 [batch, M, N] added to the rounded bf16 result (persistent kernel only)
     const uint16_t* gate = nullptr;  // bf16 [ceil(M / rows_per_gate), N]: with it C = bf16(fma(bf16(result), gate, residual))
     int rows_per_gate = 0;           // a multiple of the tile height, so that a tile has one gate row
+    // q8_gemm_qkv (persistent kernel only): columns n >= v_col0 (a multiple of 256, head dim 64) are not written to C but
+    // cast to e4m3 (c10 cast of the bf16-rounded result) and written head-major to v_codes [rows / v_tokens, v_heads, v_tokens, 64];
+    // C then has ldc = v_col0 columns per row
+    uint8_t* v_codes = nullptr;
+    int v_col0 = 0, v_tokens = 0, v_heads = 0;
 };
 
 __device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0};

@@ -58,10 +58,15 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 // element-wise addition of the two bf16 tensors gives); with p.gate (uniform) C = bf16(fma(bf16(result), gate, residual)),
 // the gated residual of an AdaLN block (blocks/ltx_transformer_block.py:44,57 in the reference), one gate row per
 // rows_per_gate rows: what the fused multiply-add kernel gives on the rounded projection.
-template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false>
+// VSPLIT (bf16 output, no residual): the tiles from column p.v_col0 on hold the V projection of a fused QKV layer; their
+// results are rounded to bf16 like the others, then cast to e4m3 (the c10 cast of q8_kernels/functional/flash_attention.py:
+// 38-45) and written token-major per head, [B, H, S, 64], the Q8_V_SD operand of the attention kernel: what the attention
+// prologue otherwise produces from the bf16 projection. C holds the other columns only (p.v_col0 per row).
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false, bool VSPLIT = false>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     static_assert(!(RES && E4M3OUT), "the residual epilogue writes bf16");
+    static_assert(!VSPLIT || (!RES && !E4M3OUT), "the V split belongs to the plain bf16 epilogue");
     constexpr int BM = 64 * MT, BN = kPipeBN;
     constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
     const int tid = threadIdx.x, lane = tid & 63;
@@ -288,7 +293,10 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                      : "memory");
         const bool rows16 = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;  // e4m3 output: rows start 16-byte aligned
         (void)rows16;
-        uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + zc;
+        const int ldc = VSPLIT ? p.v_col0 : N;  // columns per row of C
+        const bool vtile = VSPLIT && cur.n0 >= p.v_col0;  // uniform: this tile holds V columns
+        (void)vtile;
+        uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + (VSPLIT ? (size_t)cur.z * M * ldc : zc);
         const uint16_t* const rbase = reinterpret_cast<const uint16_t*>(p.residual) + zc;
         v4i gq = v4i{0, 0, 0, 0};  // the gate of the 8 columns this lane stores (RES with p.gate)
         if constexpr (RES) {
@@ -337,6 +345,32 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
                     }
                 }
+                if constexpr (VSPLIT) {
+                    if (vtile) {
+                        // the wave's 64-column slab is one head: codes of the bf16-rounded results, the two lanes of a row
+                        // swap a chunk as below and store 16 bytes each of the (token, head) row
+#pragma unroll
+                        for (int wp = 0; wp < 2; ++wp) {
+                            float f[8];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                f[2 * e] = __uint_as_float(outc[t][wp][e] << 16);
+                                f[2 * e + 1] = __uint_as_float(outc[t][wp][e] & 0xffff0000u);
+                            }
+                            e8[wp][0] = pack4_e4m3_c10(f[0], f[1], f[2], f[3]);
+                            e8[wp][1] = pack4_e4m3_c10(f[4], f[5], f[6], f[7]);
+                        }
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(e8[0][0], e8[1][0], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(e8[0][1], e8[1][1], false, false);
+                        const int m = mw0 + 32 * i + r32, n = nw0 + 32 * t + 16 * h;
+                        if (m < M && n < N) {
+                            const int bb = m / p.v_tokens, ss = m - bb * p.v_tokens, head = (nw0 - p.v_col0) >> 6;
+                            uint8_t* dst = p.v_codes + (((size_t)cur.z * (M / p.v_tokens) + bb) * p.v_heads + head) * (size_t)p.v_tokens * 64 +
+                                           (size_t)ss * 64 + 32 * t + 16 * h;
+                            *reinterpret_cast<v4u*>(dst) = v4u{s0[0], s1[0], s0[1], s1[1]};
+                        }
+                    }
+                }
                 if constexpr (E4M3OUT) {
                     // the two lanes of a row exchange one 8-byte chunk each (v_permlane32_swap: the upper half of the first
                     // operand against the lower half of the second): lane half 0 then holds columns 32 t .. + 15, lane
@@ -359,6 +393,9 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     }
                 }
             }
+            if constexpr (VSPLIT) {
+                if (vtile) continue;
+            }
             if constexpr (E4M3OUT) {
                 continue;
             } else if constexpr (GELU && !RES) {
@@ -374,7 +411,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
 #pragma unroll
                     for (int wp = 0; wp < 2; ++wp) {
                         const int n = nw0 + 32 * t + 16 * wp + 8 * h;
-                        if (m < M && n < N) *reinterpret_cast<v4u*>(cbase + (size_t)m * N + n) = outc[t][wp];
+                        if (m < M && n < N) *reinterpret_cast<v4u*>(cbase + (size_t)m * ldc + n) = outc[t][wp];
                     }
             } else {
 #pragma unroll
@@ -423,7 +460,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                 for (int j = 0; j < 2; ++j) {
                     const int m = mw0 + 32 * i + 16 * half + 8 * j + (lane_e >> 3);
                     const int n = nw0 + (lane_e & 7) * 8;
-                    if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * N + n) = w[j];
+                    if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * ldc + n) = w[j];
                 }
             }
             }

@@ -56,9 +56,12 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
                            softmax_scale: Optional[float] = None, batch_mask: Optional[torch.Tensor] = None,
                            apply_qk_hadamard: bool = False, freqs_cis=None, out_dtype: Optional[torch.dtype] = None,
                            per_token_scales: bool = False, q_norm_weight: Optional[torch.Tensor] = None,
-                           k_norm_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           k_norm_weight: Optional[torch.Tensor] = None, v_codes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [B, M, H*64], k, v [B, N, H*64] bfloat16 projections (strided slices of a fused projection are read in
     place) -> attention output [B, M, H*64].
+
+    v_codes (instead of v, which is then None; direct casts only): the e4m3 V operand [B, H, N, 64] that the QKV
+    projection's GEMM wrote itself (_C.mm_bias_qkv); the prologue then handles q and k only.
 
     q_norm_weight / k_norm_weight (fp32 [H*64]) apply the qk-RMSNorm (over all heads of a token, no epsilon) first;
     freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape).
@@ -72,6 +75,13 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
+    if v_codes is not None:
+        if per_token_scales or v is not None or d != 64 or q.shape != k.shape:
+            raise RuntimeError("flash_attn_token_major: v_codes replaces v for direct casts of a self-attention with head dim 64")
+        qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, False,
+                                      q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
+        return _C.flash_attention(qc, kc, v_codes, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                  v_token_major=True)
     if q.shape == k.shape == v.shape and d == 64:
         # self-attention: one pass over the three projections (the tables are read once, V is only cast and stays
         # token-major; the attention kernels turn its tiles while reading them from LDS).

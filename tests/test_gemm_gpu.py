@@ -423,3 +423,44 @@ def test_fp8_linear_block_shapes_m12288(dev, nk):
         steps = lambda c: (c & 0x7F) * (1 - 2 * (c >> 7))  # noqa: E731
         diff = (steps(g8.view(torch.uint8).int()) - steps(want8.view(torch.uint8).int())).abs()
         assert int(diff.max()) <= 1 and (diff > 0).float().mean() < 0.01, (int(diff.max()), (diff > 0).float().mean().item())
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "i8"])
+@pytest.mark.parametrize("shape", [(2, 96, 768, 384, 512), (1, 200, 768, 640, 256), (3, 192, 1024, 512, 768)])
+@pytest.mark.parametrize("rows", [43, 44], ids=["tile192", "tile256"])
+def test_qkv_gemm_casts_v_in_its_epilogue(dev, in_dtype, shape, rows):
+    """q8_gemm_qkv: the Q / K columns are those of the plain GEMM, the V columns the c10 e4m3 cast of the plain GEMM's
+    bf16 result, token-major per head ([B, H, S, 64]): bit-equal to the GEMM followed by the cast that the attention
+    prologue applies, under both tile heights of the persistent kernel."""
+    from q8_kernels_amd import _lib
+    b, s, n, k, v0 = shape
+    g = torch.Generator().manual_seed(n + k + s)
+    if in_dtype == "i8":
+        a, w = _rand_i8(g, b * s, k), _rand_i8(g, n, k)
+        sa, sw = torch.rand(b * s, generator=g) * 2e-3 + 1e-4, torch.rand(n, generator=g) * 2e-2 + 1e-3
+        mmb = _C().q8_mm_bias
+    else:
+        a, w = O.e4m3_c10(torch.randn(b * s, k, generator=g) * 50), O.e4m3_c10(torch.randn(n, k, generator=g) * 50)
+        sa, sw = torch.rand(b * s, generator=g) * 1e-2 + 1e-4, torch.rand(n, generator=g) * 1e-2 + 1e-4
+        mmb = _C().fp8_mm_bias
+    sw[v0 + 5] = 30.0   # a column of V beyond the e4m3 range: its codes are the NaN code of the c10 cast
+    bias = torch.randn(n, generator=g)
+    args = (a.to(dev), w.to(dev), bias.to(dev), sa.to(dev), sw.to(dev))
+    _set_cfg(rows)
+    try:
+        qk, vc = _C().mm_bias_qkv(*args, s, v0)
+        assert _last_kernel() in PERSISTENT_KERNELS
+    finally:
+        _set_cfg(40)
+    want = mmb(*args, False, torch.bfloat16).reshape(b, s, n)
+    assert torch.equal(qk.view(torch.int16), want[..., :v0].contiguous().view(torch.int16)), "Q / K columns"
+    h = (n - v0) // 64
+    want_v = O.e4m3_c10(want[..., v0:].cpu().reshape(b, s, h, 64).transpose(1, 2).contiguous())
+    got_v, want_v8 = vc.cpu().view(torch.uint8), want_v.view(torch.uint8)
+    nan = (want_v8 & 0x7f) == 0x7f
+    assert nan.any() and torch.equal(got_v & 0x7f == 0x7f, nan), "NaN codes of the overflowing column"
+    assert torch.equal(got_v[~nan], want_v8[~nan]), "V codes"
+    with pytest.raises(RuntimeError):
+        _C().mm_bias_qkv(*args, s, v0 + 64)       # the split is not on a tile boundary
+    with pytest.raises(RuntimeError):
+        _C().mm_bias_qkv(*args, s + 1, v0)        # rows are not whole batch elements
