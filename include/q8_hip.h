@@ -284,6 +284,7 @@ int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, cons
  * the bf16 round trip through memory (the fourth fusion the reference's launch boundaries allow around the attention,
  * q8_kernels/modules/attention.py:67-105). M rows = batch elements of `tokens` tokens each. Runs on the persistent kernel
  * only: N % 8 == 0, K % 128 == 0, K > 256; v_col0 a multiple of 256, N - v_col0 a multiple of 64 (Q8_ERR_SHAPE otherwise).
+ * v_col0 == 0 is a V projection of its own (a separate to_v layer): every column goes to v_codes, C may be NULL.
  */
 int q8_gemm_qkv(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C, void* v_codes,
                 int M, int N, int K, int v_col0, int tokens, int in_dtype, q8_stream_t stream);

@@ -285,16 +285,17 @@ def mm_bias_qkv(a, b, bias, a_scales, b_scales, tokens: int, v_col0: int):
         _check_input(bias, "bias")
         if bias.dtype != torch.float32 or bias.numel() != n:
             raise RuntimeError("mm_bias_qkv: bias must be float32 with %d elements" % n)
-    if not (0 < v_col0 < n) or (n - v_col0) % 64 != 0:
+    if not (0 <= v_col0 < n) or (n - v_col0) % 64 != 0:
         raise RuntimeError("mm_bias_qkv: v_col0 = %d does not split N = %d into Q/K columns and heads of 64" % (v_col0, n))
     bsz = m // tokens
+    # (v_col0 == 0: a V projection of its own; qk comes back without columns)
     qk = torch.empty((bsz, tokens, v_col0), dtype=torch.bfloat16, device=a.device)
     vc = torch.empty((bsz, (n - v_col0) // 64, tokens, 64), dtype=torch.float8_e4m3fn, device=a.device)
     if m == 0:
         return qk, vc
     with torch.cuda.device(a.device):
         _lib.check(_lib.lib().q8_gemm_qkv(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
-                                          qk.data_ptr(), vc.data_ptr(), m, n, k, v_col0, tokens,
+                                          qk.data_ptr() if v_col0 else None, vc.data_ptr(), m, n, k, v_col0, tokens,
                                           Q8_I8 if a.dtype == torch.int8 else Q8_E4M3, _stream(a)))
     return qk, vc
 

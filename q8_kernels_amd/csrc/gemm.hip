@@ -411,14 +411,15 @@ extern "C" int q8_gemm_qkv(const void* A, const void* B, const float* bias, cons
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "q8_gemm_qkv";
     if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;
-    if (int st = check_gemm(who, A, B, C, 1, 1, M, N, K)) return st;
+    // (v_col0 == 0: a V projection of its own, every column goes to v_codes and C is not used)
+    if (int st = check_gemm(who, A, B, v_col0 == 0 ? v_codes : C, 1, 1, M, N, K)) return st;
     if (!sa || !sb || !v_codes) return fail(Q8_ERR_NULL, "%s: scales and v_codes are required", who);
     if (in_dtype != Q8_I8 && in_dtype != Q8_E4M3) return fail(Q8_ERR_DTYPE, "%s: input dtype %d", who, in_dtype);
     if ((reinterpret_cast<uintptr_t>(C) % 16) || (reinterpret_cast<uintptr_t>(v_codes) % 16))
         return fail(Q8_ERR_ALIGN, "%s: C and v_codes must be 16-byte aligned", who);
     // whole 256-column tiles on either side of the split, whole heads of 64 in the V part, whole batch elements in M
-    if (v_col0 <= 0 || v_col0 >= N || v_col0 % 256 != 0 || (N - v_col0) % 64 != 0)
-        return fail(Q8_ERR_SHAPE, "%s: v_col0 = %d must be a multiple of 256 inside N = %d with N - v_col0 a multiple of 64", who, v_col0, N);
+    if (v_col0 < 0 || v_col0 >= N || v_col0 % 256 != 0 || (N - v_col0) % 64 != 0)
+        return fail(Q8_ERR_SHAPE, "%s: v_col0 = %d must be a multiple of 256 below N = %d with N - v_col0 a multiple of 64", who, v_col0, N);
     if (tokens <= 0 || M % tokens != 0) return fail(Q8_ERR_SHAPE, "%s: M = %d must be a multiple of tokens = %d", who, M, tokens);
     GemmParams p{static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), bias, sa, sb, C, 1, 1, M, N, K};
     p.v_codes = static_cast<uint8_t*>(v_codes);

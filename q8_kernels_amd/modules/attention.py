@@ -7,6 +7,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from .. import _C
 from .. import functional as Q8F
 from .linear import Q8Linear
 from .rms_norm import RMSNorm
@@ -16,6 +17,9 @@ class Attention(nn.Module):
     # False runs the reference's operator sequence (rope, split heads, flash_attn_func, merge) kernel by kernel;
     # True (default) takes the fused prologue kernels where they apply. Both give the same bits.
     fuse_prologue = True
+    # True (default): on the fused self-attention path the V projection's GEMM writes the attention kernel's e4m3 operand
+    # itself; False: V passes through memory as bfloat16 and the prologue casts it. The same bits either way.
+    cast_v_in_gemm = True
 
     def __init__(self, query_dim: int, num_heads: int, head_dim: int, bias: bool = False, out_bias: bool = False,
                  out_dim: Optional[int] = None, qk_rms_norm: bool = False, kv_dim: Optional[int] = None,
@@ -83,8 +87,25 @@ class Attention(nn.Module):
                 return [layer(xq, xs, out_dtype=mm_out_dtype) for layer in layers]
             return [layer(x, out_dtype=mm_out_dtype) for layer in layers]
 
+        v_codes = None
         if encoder_hidden_states is None:
-            query, key, value = project([self.to_q, self.to_k, self.to_v], hidden_states)
+            value = None
+            x = hidden_states
+            k_in = self.to_v.in_features
+            if (self.fuse_prologue and self.cast_v_in_gemm and attn_type == "q8_kernels" and self.head_dim == 64 and type(self.to_v) is Q8Linear
+                    and mm_out_dtype == torch.bfloat16 and non_mm_precision == torch.bfloat16
+                    and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
+                    and k_in > 256 and k_in % 128 == 0 and not torch.is_grad_enabled()):
+                # self-attention on the fused path: the V projection's GEMM writes the attention kernel's e4m3 operand itself
+                # (the bf16-rounded result, cast, token-major per head), so V never exists as a bfloat16 tensor
+                if not isinstance(x, tuple) and x.is_cuda and x.dim() == 3 and Q8F.fused.can_fuse_hadamard_quantize(x):
+                    x = Q8F.fused.hadamard_quantize(x)
+                if isinstance(x, tuple) and x[0].dim() == 3 and x[0].dtype == torch.int8:
+                    query, key = project([self.to_q, self.to_k], x)
+                    v_codes = _C.mm_bias_qkv(x[0].reshape(-1, k_in), self.to_v.weight.data, self.to_v._bias(), x[1].reshape(-1),
+                                             self.to_v.scales, x[0].shape[1], 0)[1]
+            if v_codes is None:
+                query, key, value = project([self.to_q, self.to_k, self.to_v], x)
         else:
             (query,), (key, value) = project([self.to_q], hidden_states), project([self.to_k, self.to_v], kv_src)
         rope = encoder_hidden_states is None and self.use_rope
@@ -92,16 +113,17 @@ class Attention(nn.Module):
         if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64
                 and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
                 and non_mm_precision == torch.bfloat16 and query.dim() == 3
-                and all(t.dtype == torch.bfloat16 for t in (query, key, value))
-                and not (torch.is_grad_enabled() and any(t.requires_grad for t in (query, key, value)))):
+                and all(t.dtype == torch.bfloat16 for t in (query, key, value) if t is not None)
+                and not (torch.is_grad_enabled() and any(t.requires_grad for t in (query, key, value) if t is not None))):
             # qk-RMSNorm, RoPE, head split, Hadamard and the e4m3 cast in one prologue kernel, head-merged attention
             # output: the same bits as the sequence below
             hidden_states = Q8F.fused.flash_attn_token_major(
                 query, key, value, self.num_heads, batch_mask=attention_mask, apply_qk_hadamard=apply_qk_hadamard,
                 freqs_cis=freqs_cis if rope else None,
                 q_norm_weight=self._norm_weight(self.q_norm) if self.qk_rms_norm else None,
-                k_norm_weight=self._norm_weight(self.k_norm) if self.qk_rms_norm else None)
+                k_norm_weight=self._norm_weight(self.k_norm) if self.qk_rms_norm else None, v_codes=v_codes)
             return self._project_out(hidden_states, mm_out_dtype, non_mm_precision, residual, gate)
+        assert v_codes is None, "the V codes are only produced for the fused path"
         if self.qk_rms_norm:
             query = self.q_norm(query, non_mm_precision)
             key = self.k_norm(key, non_mm_precision)

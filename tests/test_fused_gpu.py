@@ -319,6 +319,45 @@ def test_prologues_feed_attention_like_the_functional_path(dev):
     assert_bit_equal(got, want, "attention output")
 
 
+def test_attention_module_v_cast_in_gemm_equals_both_other_paths(dev):
+    """Self-attention of the Attention module at a width the persistent GEMM takes (512): with cast_v_in_gemm the V
+    projection's GEMM writes the attention kernel's e4m3 operand itself; the output has the bits of the path where V
+    passes through memory as bfloat16 and of the operator-by-operator sequence. The calls into q8_gemm_qkv are counted."""
+    import torch.nn as nn
+    import q8_kernels_amd._C as C
+    from q8_kernels_amd.modules import Attention, Q8Linear
+    torch.manual_seed(5)
+    attn = Attention(512, 8, 64, bias=True, out_bias=True, qk_rms_norm=True, use_rope=True).to(dev)
+    for name in ("to_q", "to_k", "to_v", "to_out"):
+        m = getattr(attn, name)
+        src = nn.Linear(m.in_features, m.out_features).to(dev).to(BF16)
+        q = Q8Linear.from_linear(src)
+        m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+    x = torch.randn(2, 300, 512, device=dev).to(BF16)
+    ang = torch.rand(2, 300, 256, device=dev) * 6.28
+    freqs = (torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1))
+    kw = dict(freqs_cis=freqs, mm_out_dtype=BF16, attn_type="q8_kernels")
+    saved, calls = C.mm_bias_qkv, {"qkv": 0}
+    def counted(*a, **k):
+        calls["qkv"] += 1
+        return saved(*a, **k)
+    try:
+        C.mm_bias_qkv = counted
+        with torch.no_grad():
+            in_gemm = attn(x, **kw)
+            assert calls["qkv"] == 1, "the V projection did not take q8_gemm_qkv"
+            Attention.cast_v_in_gemm = False
+            through_memory = attn(x, **kw)
+            Attention.fuse_prologue = False
+            seq = attn(x, **kw)
+        assert calls["qkv"] == 1
+    finally:
+        C.mm_bias_qkv = saved
+        Attention.cast_v_in_gemm, Attention.fuse_prologue = True, True
+    assert_bit_equal(in_gemm, through_memory, "V cast in the GEMM vs V through memory")
+    assert_bit_equal(in_gemm, seq, "V cast in the GEMM vs operator sequence")
+
+
 def test_attention_module_fused_path_equals_operator_sequence(dev):
     import torch.nn as nn
     from q8_kernels_amd.modules import Attention, Q8Linear
