@@ -51,9 +51,9 @@ class LTXTransformerBlock(nn.Module):
                 and not (torch.is_grad_enabled() and (hidden_states.requires_grad or ada_values.requires_grad)))
         bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
         if fuse:
-            # the six modulation rows as contiguous bfloat16 slices of ONE copy (instead of six strided-to-contiguous copies
-            # further down): the same values, bf16(table + timestep)
-            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = bf(ada_values.transpose(1, 2)).unbind(dim=1)
+            # the six modulation rows as contiguous bfloat16 tensors [B, T, dim] cut from ONE copy laid out [6, B, T, dim]
+            # (instead of six strided-to-contiguous copies further down): the same values, bf16(table + timestep)
+            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = bf(ada_values.permute(2, 0, 1, 3)).unbind(dim=0)
 
         if fuse:  # (int8 codes, row scales) of the rotated, modulated norm: what attn1's projections would compute
             norm_hidden_states = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm1.weight, bf(scale_msa),
