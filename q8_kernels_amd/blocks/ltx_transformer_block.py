@@ -49,7 +49,8 @@ class LTXTransformerBlock(nn.Module):
         fuse = (self.fuse_prologue and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16
                 and non_mm_precision == torch.bfloat16 and hidden_states.dim() == 3 and hidden_states.shape[-1] % 8 == 0
                 and not (torch.is_grad_enabled() and (hidden_states.requires_grad or ada_values.requires_grad)))
-        bf = lambda t: t.to(torch.bfloat16).contiguous()  # noqa: E731
+        # (cast and layout change in one copy kernel; nothing at all for a contiguous bfloat16 tensor)
+        bf = lambda t: t.to(torch.bfloat16, memory_format=torch.contiguous_format)  # noqa: E731
         if fuse:
             # the six modulation rows as contiguous bfloat16 tensors [B, T, dim] cut from ONE copy laid out [6, B, T, dim]
             # (instead of six strided-to-contiguous copies further down): the same values, bf16(table + timestep)
