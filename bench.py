@@ -216,6 +216,51 @@ def _extras_gemm(dev, steps, warmup, g, out):
         del gxq, gwq
 
 
+def _time_replay(fn, calls=50, replays=4):
+    """Mean seconds per call of `fn` captured `calls` times into one HIP graph and replayed: for kernels that take less
+    time than a call's host side (a few microseconds), where back-to-back eager calls would time the host."""
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    graph, stream = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            fn()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(calls):
+                fn()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / (replays * calls)
+
+
+def _extras_gemm_small(dev, steps, warmup, g, out):
+    """The shapes beside the big projections: the K / V projection of the 256 text rows (small-problem kernel, 64x64 tiles),
+    a 2048-cube (128x128 tiles), and the QKV projection with the cast of V in its epilogue next to the plain GEMM."""
+    from q8_kernels_amd import _C
+    for mm, nn, kk in ((256, 4096, 2048), (2048, 2048, 2048)):
+        _, _, gb, gxq, gsx, gwq, gsw = _gemm_inputs(dev, mm, nn, kk, seed=4)
+        gb = gb.to(dev)
+        t = _time_replay(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, False, torch.bfloat16))
+        out["fp8_gemm_%dx%dx%d_graph_replay" % (mm, nn, kk)] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12}
+    mm, nn, kk = 12288, 6144, 2048
+    _, _, gb, gxq, gsx, gwq, gsw = _gemm_inputs(dev, mm, nn, kk, seed=5)
+    gb = gb.to(dev)
+    t, _ = _time(lambda: _C.fp8_mm_bias(gxq, gwq, gb, gsx, gsw, False, torch.bfloat16), steps, warmup)
+    out["fp8_gemm_qkv_12288x6144x2048"] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12,
+                                          "frac_of_fp8_peak": 2.0 * mm * nn * kk / t / 1e12 / FP8_PEAK_TFLOPS}
+    t, _ = _time(lambda: _C.mm_bias_qkv(gxq, gwq, gb, gsx, gsw, 6144, 4096), steps, warmup)
+    out["fp8_gemm_qkv_12288x6144x2048_v_cast_in_epilogue"] = {"ms": t * 1e3, "tflops": 2.0 * mm * nn * kk / t / 1e12,
+                                                             "frac_of_fp8_peak": 2.0 * mm * nn * kk / t / 1e12 / FP8_PEAK_TFLOPS}
+
+
 def _extras_library(dev, steps, warmup, g, out):
     """Yardstick, not product: the vendor library's fp8 GEMM (hipBLASLt through torch._scaled_mm, row-wise scales, bf16
     output, no bias, no activation) on the same operands, box and process as this repository's kernel with its fused
@@ -399,12 +444,12 @@ def _extras_attn_options(dev, steps, warmup, g, out):
     out["attn_self_fp8_per_token_scales_lazy_max"] = entry(t, "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>, Q8_ATTN_LAZY_MAX")
 
 
-EXTRA_GROUPS = {"attn": _extras_attn, "attn_options": _extras_attn_options, "gemm": _extras_gemm, "rows": _extras_rows, "blocks": _extras_blocks,
+EXTRA_GROUPS = {"attn": _extras_attn, "attn_options": _extras_attn_options, "gemm": _extras_gemm, "gemm_small": _extras_gemm_small, "rows": _extras_rows, "blocks": _extras_blocks,
                 "library": _extras_library}
 
 
 def _extras(dev, steps, warmup, only=None, skip=()):
-    """The other workloads of the metric. `only` (group names out of attn, attn_options, gemm, rows, blocks, library) restricts
+    """The other workloads of the metric. `only` (group names out of attn, attn_options, gemm, gemm_small, rows, blocks, library) restricts
     the run to those groups, `skip` leaves groups out, e.g. for a counter-collection run of one kernel."""
     out = {}
     for name, fn in EXTRA_GROUPS.items():
@@ -420,7 +465,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--only", default=None,
-                    help="comma-separated groups of the other workloads to run (attn, attn_options, gemm, rows, blocks, library)")
+                    help="comma-separated groups of the other workloads to run (attn, attn_options, gemm, gemm_small, rows, blocks, library)")
     ap.add_argument("--skip", default="", help="comma-separated groups of the other workloads to leave out")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
