@@ -63,8 +63,10 @@ def precompute_freqs_cis(indices_grid: torch.Tensor, dim: int, theta: float = 10
     else:
         raise ValueError("precompute_freqs_cis: spacing %r" % (spacing,))
     w = w * (math.pi / 2)
-    scale = torch.tensor([1.0 / m for m in max_pos], dtype=torch.float32, device=dev)
-    pos = indices_grid.to(torch.float32) * scale[None, :, None]     # [B, 3, T] fractional positions
+    # a true division, like the reference's indices_grid[:, i] / max_pos[i]: a multiplication by the rounded reciprocal
+    # differs by one ulp for max_pos = 20, and the highest frequency (theta * pi / 2) amplifies that to 2e-3 in the tables
+    div = torch.tensor([float(m) for m in max_pos], dtype=torch.float32, device=dev)
+    pos = indices_grid.to(torch.float32) / div[None, :, None]       # [B, 3, T] fractional positions
     if spacing != "exp_2":
         pos = pos * 2 - 1
     ang = pos.transpose(1, 2)[:, :, None, :] * w[None, None, :, None]  # [B, T, n, 3]: frequency-major, axis-minor

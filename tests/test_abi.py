@@ -258,3 +258,10 @@ def test_precompute_freqs_cis_matches_the_oracle_tables():
         assert cos.dtype == torch.float32 and cos.shape == (2, 60, dim)
         assert torch.allclose(cos, want_cos, atol=1e-6) and torch.allclose(sin, want_sin, atol=1e-6)
         assert torch.equal(cos[..., 0::2], cos[..., 1::2]) and torch.equal(sin[..., 0::2], sin[..., 1::2])
+    # the benchmark's 16 x 16 x 24 grid: frame indices up to 15 over max_pos 20, where a product with the rounded reciprocal
+    # of 20 differs from the reference's division by one ulp and the top frequency turns that into 2e-3 in the tables.
+    # Bit equality with the oracle's division-based restatement.
+    grid = video_index_grid(16, 16, 24, batch=1)
+    cos, sin = precompute_freqs_cis(grid, 2048)
+    want_cos, want_sin = O.ref_freqs_cis(grid, 2048)
+    assert torch.equal(cos, want_cos) and torch.equal(sin, want_sin)
