@@ -109,6 +109,24 @@ def _cpu_baseline_gemm(x, w, bias, budget_s=25.0):
                       % (x.shape[0], w.shape[0], x.shape[1], len(times), sec)}
 
 
+def _cpu_baseline_attn(heads=4, S=6144):
+    """The oracle's own fp8 Hadamard attention (oracle/q8_oracle.py: ref_flash_attn_func, i.e. FHT + e4m3 casts + float64
+    softmax attention with e4m3-rounded probabilities) on `heads` of the 64 (batch, head) pairs of config 3 at full sequence
+    length, on the host cores; the heads are independent, so the rate carries over and the full-size time is 64 / heads times
+    the measured one."""
+    from oracle import q8_oracle as O
+    g = torch.Generator().manual_seed(7)
+    q, k, v = (torch.randn(1, heads, S, 64, generator=g).to(torch.bfloat16) for _ in range(3))
+    t0 = time.perf_counter()
+    O.ref_flash_attn_func(q, k, v, None, None, True, out_dtype=torch.bfloat16)
+    sec = time.perf_counter() - t0
+    flop = 4.0 * heads * S * S * 64
+    return {"value": flop / sec / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "the oracle's ref_flash_attn_func on %d of the 64 (batch, head) pairs of B2 H32 S%d D64 (one run, %.1f s); "
+                      "heads are independent: the full configuration extrapolates to %.0f s" % (heads, S, sec, sec * 64 / heads),
+            "full_size_seconds_extrapolated": sec * 64 / heads}
+
+
 def _cpu_blas_gemm(x, w, bias):
     """Not the oracle: the same linear + bias + GELU as plain fp32 BLAS on the dequantised codes (torch.matmul on the host
     cores), the fastest CPU formulation at hand, reported beside the oracle's figure for scale."""
@@ -188,17 +206,35 @@ def _extras_attn(dev, steps, warmup, g, out):
     out["attn_cross_fp8_masked_per_token_scales"] = {
         "ms": t_scaled * 1e3, "gbs": byts_s / t_scaled / 1e9, "frac_of_hbm_peak": byts_s / t_scaled / 1e9 / HBM_PEAK_GBS,
         "tflops": 4.0 * B * H * S * N * 64 / t_scaled / 1e12, "shape": "B2 H32 Sq6144 Skv128 D64", "valid_lengths": lens.tolist(),
-        "kernel": "attn_fwd_kernel<bf16, per-token scales, 4 waves x 32 queries>"}
+        "kernel": "attn_short_kernel<bf16, per-token scales>"}
 
 
 def _extras_gemm(dev, steps, warmup, g, out):
     from q8_kernels_amd import _C
     # int8 GEMM (config 2)
-    a = torch.randint(-127, 128, (6144, 2048), generator=g, dtype=torch.int8).to(dev)
-    b = torch.randint(-127, 128, (2048, 2048), generator=g, dtype=torch.int8).to(dev)
-    sa, sb, bias = torch.rand(6144, generator=g).to(dev), torch.rand(2048, generator=g).to(dev), torch.randn(2048, generator=g).to(dev)
+    # (operands as config 2 defines them: symmetric per-row int8 quantisation, round half even, of N(0,1) and N(0,0.02))
+    a, sa = _C.tokenwise_quant(torch.randn(6144, 2048, generator=g).to(torch.bfloat16).to(dev), None, round_half_even=True)
+    b, sb = _C.tokenwise_quant((torch.randn(2048, 2048, generator=g) * 0.02).to(torch.bfloat16).to(dev), None, round_half_even=True)
+    bias = (torch.randn(2048, generator=g) * 0.02).to(dev)
     t, _ = _time(lambda: _C.q8_mm_bias(a, b, bias, sa, sb, False, torch.bfloat16), steps, warmup)
-    out["int8_gemm_6144x2048x2048"] = {"ms": t * 1e3, "tops": 2.0 * 6144 * 2048 * 2048 / t / 1e12}
+    ops = 2.0 * 6144 * 2048 * 2048
+    out["int8_gemm_6144x2048x2048"] = {"ms": t * 1e3, "tops": ops / t / 1e12,
+                                       "roofline": {"bound": "mfma", "achieved": ops / t / 1e12, "peak": FP8_PEAK_TFLOPS, "unit": "TOP/s",
+                                                    "frac": ops / t / 1e12 / FP8_PEAK_TFLOPS, "kernel": "gemm_persist_kernel<int8>",
+                                                    "ops_per_launch": ops, "avg_launch_us": t * 1e6}}
+    # the fp8 linear as the reference's FP8LinearFunc runs it (q8_kernels/functional/linear.py:138-159): the bf16 activation is
+    # quantized inside the call, the weight arrives quantized; with and without the fused GELU of the FFN's first layer
+    from q8_kernels_amd.functional.linear import fp8_linear
+    xb, _, lb, _, _, lwq, lsw = _gemm_inputs(dev, 6144, 8192, 2048)
+    xb, lb = xb.to(dev), lb.to(dev)
+    lflop = 2.0 * 6144 * 8192 * 2048
+    for name, gelu in (("fp8_linear_quant_plus_gemm_6144x8192x2048", False), ("fp8_linear_quant_plus_gemm_gelu_6144x8192x2048", True)):
+        t, _ = _time(lambda: fp8_linear(xb, lwq, lb, None, lsw, False, torch.bfloat16, fuse_gelu=gelu), steps, warmup)
+        out[name] = {"ms": t * 1e3, "tflops": lflop / t / 1e12, "frac_of_fp8_peak": lflop / t / 1e12 / FP8_PEAK_TFLOPS,
+                     "what": "bf16 [6144,2048] in -> per-token e4m3 quantizer -> GEMM + bias%s -> bf16; effective rate of the two launches" % (" + GELU" if gelu else "")}
+    tq, _ = _time(lambda: _C.tokenwise_quant(xb, E4M3), steps, warmup)
+    out["fp8_linear_quant_plus_gemm_6144x8192x2048"]["quantizer_alone_ms"] = tq * 1e3
+    del xb, lwq
     # fp8 GEMMs of the block without GELU: projection (K = 2048) and FFN down projection (K = 8192), M = 12288 tokens
     for name, (mm, nn, kk) in (("fp8_gemm_12288x2048x2048", (12288, 2048, 2048)), ("fp8_gemm_12288x2048x8192", (12288, 2048, 8192))):
         _, _, gb, gxq, gsx, gwq, gsw = _gemm_inputs(dev, mm, nn, kk, seed=2)
@@ -377,6 +413,72 @@ def _graph_replay_time(fn, steps, warmup):
     return t
 
 
+class _OpTimer:
+    """Stands in for the loaded C-ABI library while one block is profiled: every entry point that launches work is bracketed
+    by two HIP events on the launch stream, so that a block comes apart into its operators in call order."""
+    # positions of (M, N, K) and of the two batch counts among the entry point's arguments
+    _SHAPE_ARGS = {"q8_gemm": ((8, 9, 10), (6, 7)), "q8_gemm_residual": ((9, 10, 11), (7, 8)), "q8_gemm_qkv": ((7, 8, 9), None),
+                   "q8_gemm_gated_residual": ((9, 10, 11), None)}
+
+    def __init__(self, handle):
+        self._h = handle
+        self.calls = []
+
+    def __getattr__(self, name):
+        fn = getattr(self._h, name)
+        if not name.startswith("q8_") or name in ("q8_strerror", "q8_last_error", "q8_device_info", "q8_gemm_set_config",
+                                                  "q8_attn_set_config", "q8_gemm_last_kernel"):
+            return fn
+
+        def timed(*args):
+            label = name
+            if name in self._SHAPE_ARGS:
+                mnk, batch = self._SHAPE_ARGS[name]
+                label += " %dx%dx%d" % tuple(args[i] for i in mnk)
+                if batch is not None and max(args[batch[0]], args[batch[1]]) > 1:
+                    label += " x batch %d" % max(args[batch[0]], args[batch[1]])
+            elif name == "q8_attn_fwd":
+                label += " B%d H%d M%d N%d" % (args[8], args[9], args[10], args[11])
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            r = fn(*args)
+            b.record()
+            self.calls.append((label, a, b))
+            return r
+        return timed
+
+
+def _op_breakdown(fn, block_ms, reps=10):
+    """Per-operator times of one call of `fn` (a block): HIP events around every C-ABI entry point, averaged over `reps`
+    calls, in call order. `sum_ms` is the sum of the operators' own times, `span_ms` first start to last end (it also holds
+    what lies between the operators); `block_ms` is the block timed without the events."""
+    from q8_kernels_amd import _lib
+    real = _lib.lib()
+    timer = _OpTimer(real)
+    _ramp_clocks(fn, 0.15)
+    _lib._lib = timer
+    try:
+        runs = []
+        for _ in range(reps):
+            timer.calls = []
+            fn()
+            torch.cuda.synchronize()
+            runs.append(timer.calls)
+    finally:
+        _lib._lib = real
+    n = len(runs[0])
+    assert all(len(r) == n and [c[0] for c in r] == [c[0] for c in runs[0]] for r in runs), "the block's call sequence changed between runs"
+    ops = []
+    for i in range(n):
+        us = sorted(r[i][1].elapsed_time(r[i][2]) * 1e3 for r in runs)[len(runs) // 2]
+        ops.append({"op": runs[0][i][0], "us": round(us, 2)})
+    span = sorted(r[0][1].elapsed_time(r[-1][2]) for r in runs)[len(runs) // 2]
+    total = sum(o["us"] for o in ops) * 1e-3
+    return {"ops": ops, "sum_ms": total, "span_ms": span, "block_ms": block_ms, "sum_over_block": total / block_ms,
+            "how": "median over %d calls of HIP-event pairs around each C-ABI entry point, in call order; the event records "
+                   "themselves sit in the stream (two per operator), which is why the sum reads a few percent above block_ms" % reps}
+
+
 def _extras_blocks(dev, steps, warmup, g, out):
     from q8_kernels_amd import _C
     from q8_kernels_amd.blocks import Fp8DiTBlock
@@ -392,7 +494,8 @@ def _extras_blocks(dev, steps, warmup, g, out):
     out["dit_block"] = {"ms": t * 1e3, "gflop": 2079.0, "tflops": 2079.0e9 / t / 1e12, "shape": "tokens [2,6144,2048], text [2,128,2048]"}
     with torch.no_grad():
         t = _graph_replay_time(lambda: blk(hidden, text, (cosf, sinf), lens), max(3, steps // 4), max(1, warmup // 2))
-    out["dit_block"]["ms_graph_replay"] = t * 1e3
+        out["dit_block"]["ms_graph_replay"] = t * 1e3
+        out["dit_block"]["breakdown"] = _op_breakdown(lambda: blk(hidden, text, (cosf, sinf), lens), out["dit_block"]["ms"])
     del blk
     # the reference's own block: AdaLN-modulated LTXTransformerBlock on int8 (Hadamard-rotated) Q8Linear layers
     from q8_kernels_amd.blocks import LTXTransformerBlock
@@ -413,7 +516,9 @@ def _extras_blocks(dev, steps, warmup, g, out):
     with torch.no_grad():
         t = _graph_replay_time(lambda: ltx(hidden, (cosf, sinf), None, text, lens, timestep, attn_type="q8_kernels"),
                                max(3, steps // 4), max(1, warmup // 2))
-    out["ltx_transformer_block_int8"]["ms_graph_replay"] = t * 1e3
+        out["ltx_transformer_block_int8"]["ms_graph_replay"] = t * 1e3
+        out["ltx_transformer_block_int8"]["breakdown"] = _op_breakdown(
+            lambda: ltx(hidden, (cosf, sinf), None, text, lens, timestep, attn_type="q8_kernels"), out["ltx_transformer_block_int8"]["ms"])
 
 
 def _extras_attn_options(dev, steps, warmup, g, out):
@@ -528,15 +633,27 @@ def main():
     if not args.no_extras:
         only = None if args.only is None else set(args.only.split(","))
         result["extras"] = _extras(dev, args.steps, args.warmup, only, set(filter(None, args.skip.split(","))))
-        a = result["extras"].get("attn_self_fp8_per_token_scales")
-        if a is not None:
-            result["attn_tflops"] = a["tflops"]
-            result["attn_frac_of_fp8_peak"] = a["frac_of_fp8_peak"]
-            result["attn_roofline"] = result["extras"]["attn_self_fp8_reference_casts"]["roofline"]
+        # the self-attention of config 3 in its two quantisation modes, each with its own kernel, rate and roofline
+        for key, mode in (("attn_self_fp8_per_token_scales", "per_token_scales"), ("attn_self_fp8_reference_casts", "unit_scales")):
+            a = result["extras"].get(key)
+            if a is not None:
+                result["attn_%s_tflops" % mode] = a["tflops"]
+                result["attn_%s_frac_of_fp8_peak" % mode] = a["frac_of_fp8_peak"]
+                result["attn_%s_roofline" % mode] = a["roofline"]
+        if "int8_gemm_6144x2048x2048" in result["extras"]:
+            result["int8_gemm_roofline"] = result["extras"]["int8_gemm_6144x2048x2048"]["roofline"]
         if "dit_block" in result["extras"]:
             result["block_ms"] = result["extras"]["dit_block"]["ms"]
         if not args.no_cpu:
             result["extras"]["cpu_fp32_blas_linear_gelu"] = _cpu_blas_gemm(x, w, bias)
+            if only is None or "attn" in only:
+                result["attn_cpu_baseline"] = _cpu_baseline_attn()
+            if "dit_block" in result["extras"] and "attn_cpu_baseline" in result:
+                # derived, not run: the block's 1447 GFLOP of GEMMs at the oracle's measured GEMM rate plus its 631 GFLOP of
+                # attention at the oracle's measured attention rate (the row operators are negligible beside them)
+                sec = 1447.0e9 / (result["cpu_baseline"]["value"] * 1e12) + 631.4e9 / (result["attn_cpu_baseline"]["value"] * 1e12)
+                result["block_cpu_baseline"] = {"value": sec * 1e3, "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+                                                "sample": "derived from the two measured oracle rates (GEMM 1447 GFLOP, attention 631 GFLOP), not run as a block"}
     print(json.dumps(result))
 
 

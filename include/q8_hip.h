@@ -345,11 +345,13 @@ int q8_attn_fwd(const void* q, const void* k, const void* v, void* o, const int3
                 float softmax_scale, int out_dtype, int flags, q8_stream_t stream);
 
 /*
- * Workgroup-shape override for q8_attn_fwd: 0 = the default of the mode (unit scales: 8 waves x 32 queries, per-token
- * scales: 4 waves x 32 queries), 1 = 4 waves x 64 queries (Q8_V_DS only), 2 = 4 waves x 32 queries, 3 = as 0 without the
- * short-sequence kernel that otherwise takes N <= 128 (K and V of a (batch, head) resident in LDS, P rounded against the
- * final row maximum), 4 = 8 waves x 32 queries. All shapes of one kernel give the same bits. It holds for the calling thread only; meant for tests and tuning, no counterpart in the reference (whose
- * workgroup is fixed at 4 warps x 16 queries, csrc/flash_attention/flash_attention_cuda.cu:279-287).
+ * Workgroup-shape override for q8_attn_fwd: 0 = the default (N <= 128: the short-sequence kernel, K and V of a (batch, head)
+ * resident in LDS and P rounded against the final row maximum; longer sequences: the general kernel with 8 waves x 32 queries
+ * for unit scales, 4 waves x 32 queries for per-token scales). 1 .. 4 select the general kernel for every N, in the shape
+ * 1 = 4 waves x 64 queries (Q8_V_DS only), 2 = 4 waves x 32 queries, 3 = the default shape of the mode, 4 = 8 waves x 32
+ * queries. All shapes of the general kernel give the same bits. It holds for the calling thread only; meant for tests and
+ * tuning, no counterpart in the reference (whose workgroup is fixed at 4 warps x 16 queries,
+ * csrc/flash_attention/flash_attention_cuda.cu:279-287).
  */
 int q8_attn_set_config(int cfg);
 

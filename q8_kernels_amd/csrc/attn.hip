@@ -797,7 +797,8 @@ __global__ __launch_bounds__(256, (SCALED || VTOK) ? 2 : 3) void attn_short_kern
 using namespace q8;
 
 // per thread: 0 = default (unit scales: 8 waves x 32 queries; per-token scales: 4 waves x 32 queries), 1 = 4 waves x 64
-// queries, 2 = 4 waves x 32 queries, 3 = as 0 and without the short-sequence kernel for N <= 128, 4 = 8 waves x 32 queries
+// queries, 2 = 4 waves x 32 queries, 3 = the default shape of the mode, 4 = 8 waves x 32 queries; 1 .. 4 all select the general
+// kernel, also for N <= 128, which under 0 takes the short-sequence kernel
 static thread_local int g_attn_cfg = 0;
 
 extern "C" int q8_attn_set_config(int cfg) {
@@ -840,7 +841,7 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
     const bool msum = (flags & Q8_ATTN_SUM_ROUNDED_P) != 0;
     if (msum && cfg == 1)
         return fail(Q8_ERR_FLAGS, "q8_attn_fwd: the 4 waves x 64 queries tuning shape has no Q8_ATTN_SUM_ROUNDED_P form");
-    if (N <= 128 && cfg != 3) {
+    if (N <= 128 && cfg == 0) {  // (a shape override always means the general kernel in that shape)
         // K and V stay in LDS; enough workgroups of 4 waves to fill every CU once (three per CU with unit scales and V^T,
         // whose code fits 168 registers, two otherwise), each wave walking over several query tiles of every batch
         const long q_tiles = (M + 31) / 32;

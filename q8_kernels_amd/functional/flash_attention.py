@@ -24,11 +24,13 @@ def _pad_last(t: torch.Tensor, pad: int) -> torch.Tensor:
 
 def flash_attn_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: Optional[float] = None,
                     batch_mask: Optional[torch.Tensor] = None, apply_qk_hadamard: bool = False, *,
-                    out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+                    out_dtype: Optional[torch.dtype] = None, p_unit_range: bool = False) -> torch.Tensor:
     """q [B,H,M,D], k, v [B,H,N,D] (or v already transposed to [B,H,D,N]); 16-bit inputs are cast to e4m3
     (Q and K through the FHT when apply_qk_hadamard, with the softmax scale folded into both).
     batch_mask: int32 [B] valid KV lengths. Returns [B,H,M,D]; e4m3 like the reference unless `out_dtype`
-    (keyword only) asks for bfloat16."""
+    (keyword only) asks for bfloat16. `p_unit_range=True` (keyword only) rounds the probabilities exactly on the
+    reference's grid, e4m3(p) with p <= 1 (csrc/flash_attention/flash_attention_cuda.cu:197-221); the default rounds
+    e4m3(2^8 p), which keeps weights down to 2^-14 of the row maximum instead of flushing those below 2^-10 to zero."""
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     head_size_og = q.size(3)
@@ -54,5 +56,6 @@ def flash_attn_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_s
         q = q.to(_FP8) if _is_16bit(q) else q
         k = k.to(_FP8) if _is_16bit(k) else k
         kernel_scale = softmax_scale
-    o = _C.flash_attention(q.contiguous(), k.contiguous(), v.contiguous(), kernel_scale, batch_mask, out_dtype=out_dtype)
+    o = _C.flash_attention(q.contiguous(), k.contiguous(), v.contiguous(), kernel_scale, batch_mask, out_dtype=out_dtype,
+                            p_unit_range=p_unit_range)
     return o[..., :head_size_og]

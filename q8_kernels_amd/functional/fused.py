@@ -56,7 +56,8 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
                            softmax_scale: Optional[float] = None, batch_mask: Optional[torch.Tensor] = None,
                            apply_qk_hadamard: bool = False, freqs_cis=None, out_dtype: Optional[torch.dtype] = None,
                            per_token_scales: bool = False, q_norm_weight: Optional[torch.Tensor] = None,
-                           k_norm_weight: Optional[torch.Tensor] = None, v_codes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           k_norm_weight: Optional[torch.Tensor] = None, v_codes: Optional[torch.Tensor] = None,
+                           p_unit_range: bool = False) -> torch.Tensor:
     """q [B, M, H*64], k, v [B, N, H*64] bfloat16 projections (strided slices of a fused projection are read in
     place) -> attention output [B, M, H*64].
 
@@ -66,7 +67,8 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
     q_norm_weight / k_norm_weight (fp32 [H*64]) apply the qk-RMSNorm (over all heads of a token, no epsilon) first;
     freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape).
     Without per_token_scales the operands are cast to e4m3 exactly as flash_attn_func does; with it each
-    (token, head) row of q, k and v gets its own absmax scale."""
+    (token, head) row of q, k and v gets its own absmax scale. p_unit_range as in flash_attn_func (the reference's
+    probability grid)."""
     d = q.shape[-1] // num_heads
     if softmax_scale is None:
         softmax_scale = d ** (-0.5)
@@ -80,7 +82,7 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
             raise RuntimeError("flash_attn_token_major: v_codes replaces v for direct casts of a self-attention with head dim 64")
         qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, False,
                                       q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight)
-        return _C.flash_attention(qc, kc, v_codes, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+        return _C.flash_attention(qc, kc, v_codes, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True, p_unit_range=p_unit_range,
                                   v_token_major=True)
     if q.shape == k.shape == v.shape and d == 64:
         # self-attention: one pass over the three projections (the tables are read once, V is only cast and stays
@@ -90,8 +92,8 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         if per_token_scales:
             (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
             return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
-                                      v_scales=vs, token_major_out=True, v_token_major=True)
-        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                      v_scales=vs, token_major_out=True, p_unit_range=p_unit_range, v_token_major=True)
+        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True, p_unit_range=p_unit_range,
                                   v_token_major=True)
     if k.shape == v.shape and d == 64:
         # other queries than keys (cross-attention): the queries alone, keys and values together in a second launch, V
@@ -103,8 +105,8 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         if per_token_scales:
             (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
             return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
-                                      v_scales=vs, token_major_out=True, v_token_major=True)
-        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                      v_scales=vs, token_major_out=True, p_unit_range=p_unit_range, v_token_major=True)
+        return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True, p_unit_range=p_unit_range,
                                   v_token_major=True)
     if q.shape == k.shape:  # one pass over q and k
         qc, kc = _C.attn_prep_qk_pair(q, k, num_heads, cos, sin, apply_qk_hadamard, qk_scale, per_token_scales,
@@ -118,5 +120,5 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
     if per_token_scales:
         (qc, qs), (kc, ks), (vc, vs) = qc, kc, vc
         return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, q_scales=qs, k_scales=ks,
-                                  v_scales=vs, token_major_out=True)
-    return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True)
+                                  v_scales=vs, token_major_out=True, p_unit_range=p_unit_range)
+    return _C.flash_attention(qc, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True, p_unit_range=p_unit_range)

@@ -59,7 +59,13 @@ class Attention(nn.Module):
                 and (gate is None or gate.dtype == torch.bfloat16)):
             return self.to_out(hidden_states, out_dtype=mm_out_dtype, residual=residual.contiguous(), gate=gate)
         out = self.to_out(hidden_states, out_dtype=mm_out_dtype).to(non_mm_precision)
-        return out + residual if gate is None else out * gate + residual
+        if gate is None:
+            return out + residual
+        if (out.is_cuda and out.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 and gate.dtype == torch.bfloat16
+                and not (torch.is_grad_enabled() and any(t.requires_grad for t in (out, gate, residual)))):
+            # one rounding, like the epilogue form: fma(out, gate, residual) on the fused multiply-add kernel
+            return Q8F.fma.multiply_add(out.reshape(residual.shape), gate, residual.contiguous(), 0.0)
+        return out * gate + residual
 
     def forward(self, hidden_states, freqs_cis=None, encoder_hidden_states=None, attention_mask=None,
                 non_mm_precision=torch.bfloat16, mm_out_dtype=None, apply_qk_hadamard=True, attn_type="torch",
@@ -100,7 +106,9 @@ class Attention(nn.Module):
                 # (the bf16-rounded result, cast, token-major per head), so V never exists as a bfloat16 tensor
                 if not isinstance(x, tuple) and x.is_cuda and x.dim() == 3 and Q8F.fused.can_fuse_hadamard_quantize(x):
                     x = Q8F.fused.hadamard_quantize(x)
-                if isinstance(x, tuple) and x[0].dim() == 3 and x[0].dtype == torch.int8:
+                # (and the operand sizes the persistent GEMM addresses with 32-bit offsets; larger ones take the plain projection)
+                if (isinstance(x, tuple) and x[0].dim() == 3 and x[0].dtype == torch.int8
+                        and x[0].numel() < 2 ** 32 and self.to_v.weight.numel() < 2 ** 32):
                     query, key = project([self.to_q, self.to_k], x)
                     v_codes = _C.mm_bias_qkv(x[0].reshape(-1, k_in), self.to_v.weight.data, self.to_v._bias(), x[1].reshape(-1),
                                              self.to_v.scales, x[0].shape[1], 0)[1]

@@ -66,38 +66,52 @@ def attn_cfg(request):
     _lib.check(_lib.lib().q8_attn_set_config(0))
 
 
+@pytest.fixture(params=[False, True], ids=["p_2^8", "p_reference_grid"])
+def p_grid(request):
+    """The two grids the probabilities are rounded on: the kernel's default e4m3(2^8 p) (the oracle is then told
+    p_scale=256) and, with p_unit_range=True, the reference's own e4m3(p), p <= 1
+    (csrc/flash_attention/flash_attention_cuda.cu:197-221), checked against the oracle's default p_scale=1.
+    Yields (keyword arguments of the call, the oracle's p_scale)."""
+    return ({"p_unit_range": True}, 1.0) if request.param else ({}, 256.0)
+
+
 @pytest.mark.parametrize("m,n", [(256, 64), (64, 128), (1, 1), (33, 17), (255, 100), (257, 200), (300, 640), (512, 1000)])
-def test_attention_shapes(dev, attn_cfg, m, n):
+def test_attention_shapes(dev, attn_cfg, p_grid, m, n):
+    kw, p_scale = p_grid
     q, k, v = _inputs(m * 1000 + n, 2, 3, m, n)
-    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, out_dtype=torch.bfloat16, **kw)
     assert got.shape == (2, 3, m, 64) and got.dtype == torch.bfloat16
-    _check(got, q, k, v, 0.125, what="m=%d n=%d" % (m, n))
+    _check(got, q, k, v, 0.125, what="m=%d n=%d" % (m, n), p_scale=p_scale)
 
 
-def test_attention_fp8_output_default(dev):
-    q, k, v = _inputs(5, 1, 2, 130, 300)
-    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None)
+@pytest.mark.parametrize("m,n", [(130, 300), (200, 100)])
+def test_attention_fp8_output_default(dev, p_grid, m, n):
+    """e4m3 output (the reference's only output type) of the general and of the short-sequence kernel, on both grids"""
+    kw, p_scale = p_grid
+    q, k, v = _inputs(5, 1, 2, m, n)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, None, **kw)
     assert got.dtype == E4M3
-    want = O.ref_attention(q, k, v, 0.125, None, out_dtype=E4M3, p_scale=256.0)  # the kernel's default grid
+    want = O.ref_attention(q, k, v, 0.125, None, out_dtype=E4M3, p_scale=p_scale)
     g, w = got.cpu().float(), want.float()
     assert not torch.isnan(g).any()
     assert ((g - w).abs() <= 0.13 * w.abs() + 0.03).all()
 
 
 @pytest.mark.parametrize("lens", [[128, 16], [1, 64], [65, 127], [0, 100], [63, 200]])
-def test_attention_kv_length_mask(dev, attn_cfg, lens):
+def test_attention_kv_length_mask(dev, attn_cfg, p_grid, lens):
+    kw, p_scale = p_grid
     n = 128
     q, k, v = _inputs(sum(lens), 2, 4, 200, n)
     kv_len = torch.tensor(lens, dtype=torch.int32)
-    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, kv_len.to(dev), out_dtype=torch.bfloat16)
-    _check(got, q, k, v, 0.125, kv_len.clamp(max=n), what="lens=%s" % lens)
+    got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, kv_len.to(dev), out_dtype=torch.bfloat16, **kw)
+    _check(got, q, k, v, 0.125, kv_len.clamp(max=n), what="lens=%s" % lens, p_scale=p_scale)
     # masked keys and values have no influence at all
     k2, v2 = k.clone().view(torch.uint8), v.clone().view(torch.uint8)
     for b, ln in enumerate(lens):
         k2[b, :, min(ln, n):] = 0x55
         v2[b, :, min(ln, n):] = 0x7E
     got2 = _C().flash_attention(q.to(dev), k2.view(E4M3).to(dev), _vt(v2.view(E4M3)).to(dev), 0.125, kv_len.to(dev),
-                                out_dtype=torch.bfloat16)
+                                out_dtype=torch.bfloat16, **kw)
     assert torch.equal(got.cpu().view(torch.int16), got2.cpu().view(torch.int16))
     for b, ln in enumerate(lens):
         if ln == 0:
@@ -169,7 +183,14 @@ def test_attention_sum_rounded_p(dev, cfg, m, n, std):
         lazy = run(v, lazy_max=True)
     finally:
         _lib.check(_lib.lib().q8_attn_set_config(0))
-    assert torch.equal(got.cpu().view(torch.int16), run(v).cpu().view(torch.int16)), "config %d against the default shape" % cfg
+    # every shape of the general kernel gives the same bits; for N <= 128 the library's default is the short-sequence kernel
+    # (another rounding of P), so the general kernel's default shape (config 3) is the baseline there
+    _lib.check(_lib.lib().q8_attn_set_config(3 if (n <= 128 and cfg != 0) else 0))
+    try:
+        base = run(v)
+    finally:
+        _lib.check(_lib.lib().q8_attn_set_config(0))
+    assert torch.equal(got.cpu().view(torch.int16), base.cpu().view(torch.int16)), "config %d against the default shape" % cfg
     g = got.cpu().double()
     exact, wabs, uabs = O.ref_attention(q, k, v, 0.125, lens, round_p=False, return_weighted_abs=True)
     same_def = O.ref_attention(q, k, v, 0.125, lens, p_scale=256.0, sum_rounded=True)
@@ -210,7 +231,8 @@ def test_attention_reference_probability_range(dev):
     assert (dflt.cpu().double() - exact).abs().mean() < (ref_mode.cpu().double() - exact).abs().mean()
 
 
-def test_attention_per_token_scales(dev, attn_cfg):
+def test_attention_per_token_scales(dev, attn_cfg, p_grid):
+    kw, p_scale = p_grid
     g = torch.Generator().manual_seed(9)
     b, h, m, n = 2, 2, 150, 333
     qf = torch.randn(b, h, m, 64, generator=g) * (torch.rand(b, h, m, 1, generator=g) * 4 + 0.2)
@@ -219,8 +241,8 @@ def test_attention_per_token_scales(dev, attn_cfg):
     (q, sq), (k, sk), (v, sv) = (O.ref_quant(t.to(torch.bfloat16), E4M3) for t in (qf, kf, vf))
     lens = torch.tensor([333, 77], dtype=torch.int32)
     got = _C().flash_attention(q.to(dev), k.to(dev), _vt(v).to(dev), 0.125, lens.to(dev), out_dtype=torch.bfloat16,
-                               q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev))
-    _check(got, q, k, v, 0.125, lens, (sq, sk, sv), what="per-token scales")
+                               q_scales=sq.to(dev), k_scales=sk.to(dev), v_scales=sv.to(dev), **kw)
+    _check(got, q, k, v, 0.125, lens, (sq, sk, sv), what="per-token scales", p_scale=p_scale)
     full = torch.nn.functional.scaled_dot_product_attention(
         qf.double(), kf.double(), vf.double(),
         attn_mask=torch.zeros(b, 1, 1, n, dtype=torch.float64).masked_fill(
@@ -228,10 +250,11 @@ def test_attention_per_token_scales(dev, attn_cfg):
     assert cosine(got.cpu(), full) > 0.99
 
 
-def test_attention_config3_self_attention_hadamard(dev):
+def test_attention_config3_self_attention_hadamard(dev, p_grid):
     """B=2, H=32, S=6144, D=64, non-causal; Q/K/V bf16 ~ N(0,1) with one head-dim channel scaled x20; Q and K
     rotated by the normalised 64-point Hadamard transform, everything quantised per token to e4m3, softmax
     scale 1/8, bf16 output. The whole problem runs on the GPU; the oracle checks four (batch, head) pairs."""
+    kw, p_scale = p_grid
     C = _C()
     g = torch.Generator().manual_seed(3)
     B, H, S = 2, 32, 6144
@@ -242,7 +265,7 @@ def test_attention_config3_self_attention_hadamard(dev):
     qr, kr = C.fast_hadamard_transform(qd, 0.125, torch.bfloat16), C.fast_hadamard_transform(kd, 0.125, torch.bfloat16)
     (q8, sq), (k8, sk), (v8, sv) = C.tokenwise_quant(qr, E4M3), C.tokenwise_quant(kr, E4M3), C.tokenwise_quant(vd, E4M3)
     vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
-    out = C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv)
+    out = C.flash_attention(q8, k8, vt, 0.125, None, out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv, **kw)
     assert out.shape == (B, H, S, 64)
     for (b, h) in [(0, 0), (0, 17), (1, 5), (1, 31)]:
         sl = (slice(b, b + 1), slice(h, h + 1))
@@ -251,7 +274,7 @@ def test_attention_config3_self_attention_hadamard(dev):
         ov, osv = O.ref_quant(v[sl], E4M3)
         assert torch.equal(q8[sl].cpu().view(torch.uint8), oq.view(torch.uint8))
         assert torch.equal(sk[sl].cpu(), osk)
-        _check(out[sl], oq, ok, ov, 0.125, None, (osq, osk, osv), what="config 3 (b=%d,h=%d)" % (b, h))
+        _check(out[sl], oq, ok, ov, 0.125, None, (osq, osk, osv), what="config 3 (b=%d,h=%d)" % (b, h), p_scale=p_scale)
         # against attention on the unquantised bf16 inputs: with a x20 outlier channel in q and k the logits have a
         # standard deviation near 50 and single keys dominate, so e4m3 rounding of q and k can change the winner;
         # this measures the quantisation scheme, not the kernel
@@ -265,9 +288,10 @@ def test_attention_config3_self_attention_hadamard(dev):
     assert bool(((o <= vmax + slack) & (o >= vmin - slack)).all())
 
 
-def test_attention_config4_cross_attention_mask(dev):
+def test_attention_config4_cross_attention_mask(dev, p_grid):
     """B=2, H=32, 6144 queries, 128 text keys, valid lengths drawn from 16..128, reference-style direct casts with
     the Hadamard rotation (softmax scale folded into Q and K)."""
+    kw, p_scale = p_grid
     g = torch.Generator().manual_seed(4)
     B, H, M, N = 2, 32, 6144, 128
     q = torch.randn(B, H, M, 64, generator=g).to(torch.bfloat16)
@@ -275,21 +299,22 @@ def test_attention_config4_cross_attention_mask(dev):
     v = torch.randn(B, H, N, 64, generator=g).to(torch.bfloat16)
     lens = torch.randint(16, 129, (B,), generator=g, dtype=torch.int32)
     from q8_kernels_amd.functional.flash_attention import flash_attn_func
-    out = flash_attn_func(q.to(dev), k.to(dev), v.to(dev), None, lens.to(dev), True, out_dtype=torch.bfloat16)
+    out = flash_attn_func(q.to(dev), k.to(dev), v.to(dev), None, lens.to(dev), True, out_dtype=torch.bfloat16, **kw)
     assert out.shape == (B, H, M, 64)
     s = (1 / 64) ** 0.5 * (0.125 ** 0.5)
     q8, k8, v8 = O.ref_fht(q, s, E4M3), O.ref_fht(k, s, E4M3), O.e4m3_c10(v)
     hs = slice(0, 32, 11)
-    _check(out[:, hs], q8[:, hs], k8[:, hs], v8[:, hs], 1.0, lens, what="config 4")
+    _check(out[:, hs], q8[:, hs], k8[:, hs], v8[:, hs], 1.0, lens, what="config 4", p_scale=p_scale)
     mask = torch.zeros(B, 1, 1, N, dtype=torch.float64).masked_fill(~(torch.arange(N)[None, :] < lens[:, None])[:, None, None, :], float("-inf"))
     plain = torch.nn.functional.scaled_dot_product_attention(q[:, hs].double(), k[:, hs].double(), v[:, hs].double(), attn_mask=mask)
     assert cosine(out[:, hs].cpu(), plain) >= 0.998  # accuracy of the direct e4m3 casts, not of the kernel
 
 
-def test_attention_config4_cross_attention_mask_per_token_scales(dev):
+def test_attention_config4_cross_attention_mask_per_token_scales(dev, p_grid):
     """Config 4 with per-token e4m3 quantisation of Q, K (after the Hadamard rotation) and V: 6144 queries, 128 text keys,
     valid lengths drawn from 16..128. The whole problem runs on the GPU; the oracle checks four (batch, head) pairs, and
     masked keys and values have no influence at all."""
+    kw, p_scale = p_grid
     C = _C()
     g = torch.Generator().manual_seed(44)
     B, H, M, N = 2, 32, 6144, 128
@@ -300,21 +325,21 @@ def test_attention_config4_cross_attention_mask_per_token_scales(dev):
     qr, kr = C.fast_hadamard_transform(qd, 0.125, torch.bfloat16), C.fast_hadamard_transform(kd, 0.125, torch.bfloat16)
     (q8, sq), (k8, sk), (v8, sv) = C.tokenwise_quant(qr, E4M3), C.tokenwise_quant(kr, E4M3), C.tokenwise_quant(vd, E4M3)
     vt = v8.view(torch.uint8).transpose(2, 3).contiguous().view(E4M3)
-    out = C.flash_attention(q8, k8, vt, 0.125, lens.to(dev), out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv)
+    out = C.flash_attention(q8, k8, vt, 0.125, lens.to(dev), out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk, v_scales=sv, **kw)
     assert out.shape == (B, H, M, 64)
     for (b, h) in [(0, 0), (0, 21), (1, 7), (1, 31)]:
         sl = (slice(b, b + 1), slice(h, h + 1))
         oq, osq = O.ref_quant(O.ref_fht(q[sl], 0.125, torch.bfloat16), E4M3)
         ok, osk = O.ref_quant(O.ref_fht(k[sl], 0.125, torch.bfloat16), E4M3)
         ov, osv = O.ref_quant(v[sl], E4M3)
-        _check(out[sl], oq, ok, ov, 0.125, lens[b:b + 1], (osq, osk, osv), what="config 4 per token (b=%d,h=%d)" % (b, h))
+        _check(out[sl], oq, ok, ov, 0.125, lens[b:b + 1], (osq, osk, osv), what="config 4 per token (b=%d,h=%d)" % (b, h), p_scale=p_scale)
     k2, v2, sk2, sv2 = k8.clone().view(torch.uint8), v8.clone().view(torch.uint8), sk.clone(), sv.clone()
     for b in range(B):
         ln = int(lens[b])
         k2[b, :, ln:], v2[b, :, ln:], sk2[b, :, ln:], sv2[b, :, ln:] = 0x55, 0x7E, 1e3, 1e3
     vt2 = v2.transpose(2, 3).contiguous().view(E4M3)
     out2 = C.flash_attention(q8, k2.view(E4M3), vt2, 0.125, lens.to(dev), out_dtype=torch.bfloat16, q_scales=sq, k_scales=sk2,
-                             v_scales=sv2)
+                             v_scales=sv2, **kw)
     # (the common factor max_j sv_j runs over the valid keys only, so the masked scales must not show either)
     assert torch.equal(out.cpu().view(torch.int16), out2.cpu().view(torch.int16))
 

@@ -107,6 +107,40 @@ def test_int8_config2_bit_exact_and_dequant(dev):
     assert cosine(out.cpu(), ref) > 0.999
 
 
+
+@pytest.mark.parametrize("pin,kernel", [(44, K_PERSIST256), (43, K_PERSIST192)], ids=["256rows", "192rows"])
+@pytest.mark.parametrize("mnk", [(2304, 8192, 2048), (1600, 10248, 640)])
+def test_int8_persistent_kernel_accumulators_bit_exact(dev, pin, kernel, mnk):
+    """The persistent kernel (the one that serves config 2 and the block's int8 linears) has no int32 output; its
+    accumulators are observed through the bf16 store instead: with sparse operands in {-1, 0, 1} every |acc| stays far
+    below 256, where bf16 holds integers exactly, and with unit scales and no bias the stored value IS the accumulator
+    (csrc/gemm/q8_matmul_bias.cu:315-320: float(acc) * (sa * sb)). More tiles than CUs, both tile heights, one shape
+    with ragged edges in M and N; the oracle's integer matmul is evaluated in float32, exact for these magnitudes."""
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(m + n + k)
+
+    def sparse(rows):
+        u = torch.rand(rows, k, generator=g)
+        return ((u < 0.05).to(torch.int8) - (u > 0.95).to(torch.int8))
+
+    a, b = sparse(m), sparse(n)
+    # a few denser rows of either operand so that the accumulators are not all tiny (still far below 256)
+    a[::97] = ((torch.rand(a[::97].shape, generator=g) < 0.2).to(torch.int8))
+    b[::89] = ((torch.rand(b[::89].shape, generator=g) < 0.2).to(torch.int8))
+    want = a.float() @ b.float().T + 0.0  # (+ 0.0: a sum of negative zeros becomes the +0 of an integer zero)
+    assert want.abs().max() <= 256 and want.abs().max() >= 15
+    assert torch.equal(want[:64, :64].long(), O.ref_gemm_i32(a[:64], b[:64]).long())  # the float32 evaluation is the oracle's integers
+    ones_m, ones_n = torch.ones(m, device=dev), torch.ones(n, device=dev)
+    _set_cfg(4)
+    _set_cfg(pin)
+    try:
+        out = _C().q8_mm(a.to(dev), b.to(dev), ones_m, ones_n, False, torch.bfloat16)
+        assert _last_kernel() == kernel
+    finally:
+        _set_cfg(40)
+        _set_cfg(0)
+    assert_bit_equal(out[0], want.to(torch.bfloat16), "persistent int8 accumulators %s" % (mnk,))
+
 # ------------------------------------------------------------------ epilogue variants
 
 @pytest.mark.parametrize("in_dtype", ["i8", "fp8"])
