@@ -812,7 +812,7 @@ extern "C" int q8_attn_fwd(const void* q, const void* k, const void* v, void* o,
                            int64_t v_row_stride, float softmax_scale, int out_dtype, int flags, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (D != 64) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: head dim %d (only 64 is supported)", D);
-    if (B < 0 || H <= 0 || M < 0 || N <= 0) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
+    if (B < 0 || H <= 0 || M < 0 || N <= 0 || M > (1 << 30) || N > (1 << 30)) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B %d H %d M %d N %d", B, H, M, N);
     if (B == 0 || M == 0) return Q8_OK;  // no queries: nothing to compute or to write
     if (!q || !k || !v || !o) return fail(Q8_ERR_NULL, "q8_attn_fwd: null pointer");
     if ((long)B * H > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_fwd: B*H = %ld exceeds 65535", (long)B * H);

@@ -168,7 +168,8 @@ extern "C" int q8_fma(const void* x, int x_dtype, const void* y, int y_dtype, co
                       int out_dtype, int64_t rows, int dim, int64_t y_rows_every, int64_t z_rows_every, float scale_add,
                       q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (rows < 0 || dim <= 0 || dim % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_fma: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
+    if (rows < 0 || rows > ((int64_t)1 << 40) || dim <= 0 || dim % 8 != 0)
+        return fail(Q8_ERR_SHAPE, "q8_fma: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
     if (rows == 0) return Q8_OK;  // (with no rows the broadcast periods mean nothing; a caller with zero tokens passes 0)
     if (y_rows_every <= 0 || z_rows_every <= 0) return fail(Q8_ERR_SHAPE, "q8_fma: broadcast periods must be positive");
     if (!x || !y || !z || !out) return fail(Q8_ERR_NULL, "q8_fma: null pointer");
@@ -221,7 +222,8 @@ extern "C" int q8_gelu_backward(const void* x, int x_dtype, const void* grad, in
 extern "C" int q8_rope_backward(const void* grad, int grad_dtype, const float* cos_t, const float* sin_t, void* out,
                                 int out_dtype, int64_t rows, int dim, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (rows < 0 || dim <= 0 || dim % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_rope_backward: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
+    if (rows < 0 || rows > ((int64_t)1 << 40) || dim <= 0 || dim % 8 != 0)
+        return fail(Q8_ERR_SHAPE, "q8_rope_backward: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
     if (int st = check_ew("q8_rope_backward", grad, grad_dtype, out, out_dtype, rows * (int64_t)dim)) return st;
     if (rows == 0) return Q8_OK;
     if (!cos_t || !sin_t) return fail(Q8_ERR_NULL, "q8_rope_backward: null table");

@@ -589,7 +589,8 @@ extern "C" int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, 
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (B < 0 || S < 0 || H <= 0 || H > 65535 || B > 65535) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: B %d S %d H %d", B, S, H);
     if (D != 64) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: head dim %d (want 64)", D);
-    if (S_pad < S || S_pad % 16 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: S_pad %d must be a multiple of 16 >= S %d", S_pad, S);
+    if (S_pad < S || S_pad % 16 != 0 || S_pad > (1 << 30))
+        return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: S_pad %d must be a multiple of 16 >= S %d (at most 2^30)", S_pad, S);
     if (B == 0 || S_pad == 0) return Q8_OK;
     if (!x || !codes) return fail(Q8_ERR_NULL, "q8_attn_prep_v: null pointer");
     if (x_row_stride < (int64_t)H * D || x_row_stride % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_attn_prep_v: row stride %lld", (long long)x_row_stride);

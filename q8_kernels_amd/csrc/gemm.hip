@@ -344,6 +344,8 @@ static int check_gemm(const char* who, const void* A, const void* B, const void*
     if (!A || !B || !C) return fail(Q8_ERR_NULL, "%s: null pointer", who);
     if (M <= 0 || N <= 0 || K <= 0 || batch_a <= 0 || batch_b <= 0)
         return fail(Q8_ERR_SHAPE, "%s: M %d N %d K %d batch %d/%d must be positive", who, M, N, K, batch_a, batch_b);
+    // (2^30 keeps every rounded-up tile count of the launch geometry inside int)
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return fail(Q8_ERR_SHAPE, "%s: M %d N %d K %d too large", who, M, N, K);
     if (batch_a != batch_b && batch_a != 1 && batch_b != 1)
         return fail(Q8_ERR_SHAPE, "%s: batch mismatch %d vs %d", who, batch_a, batch_b);
     if (K % 16 != 0) return fail(Q8_ERR_SHAPE, "%s: K = %d must be a multiple of 16", who, K);

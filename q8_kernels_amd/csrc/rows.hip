@@ -168,7 +168,8 @@ extern "C" int q8_quant_rows(const void* x, int x_dtype, void* codes, int code_d
         return fail(Q8_ERR_DTYPE, "q8_quant_rows: code dtype %d (want I8 or E4M3)", code_dtype);
     const int esz = elem_size(x_dtype);
     if (esz == 0 || x_dtype == Q8_I8) return fail(Q8_ERR_DTYPE, "q8_quant_rows: input dtype %d", x_dtype);
-    if (x_row_stride < dim) return fail(Q8_ERR_SHAPE, "q8_quant_rows: row stride %lld < dim %d", (long long)x_row_stride, dim);
+    if (x_row_stride < dim || x_row_stride > ((int64_t)1 << 40))
+        return fail(Q8_ERR_SHAPE, "q8_quant_rows: row stride %lld (dim %d)", (long long)x_row_stride, dim);
     const int need = (x_dtype == Q8_E4M3) ? 8 : 16;
     if ((reinterpret_cast<uintptr_t>(x) % need) || ((x_row_stride * esz) % need) || (reinterpret_cast<uintptr_t>(codes) % 8) ||
         (reinterpret_cast<uintptr_t>(scales) % 4))
@@ -251,7 +252,8 @@ extern "C" int q8_rmsnorm(const void* x, int x_dtype, const float* w, void* y, i
 extern "C" int q8_rope(const void* x, int x_dtype, const float* cos_t, const float* sin_t, void* y, int y_dtype,
                        int64_t rows, int dim, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (rows < 0 || dim <= 0 || dim % 8 != 0) return fail(Q8_ERR_SHAPE, "q8_rope: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
+    if (rows < 0 || rows > ((int64_t)1 << 40) || dim <= 0 || dim % 8 != 0)
+        return fail(Q8_ERR_SHAPE, "q8_rope: rows %lld dim %d (dim %% 8 == 0)", (long long)rows, dim);
     if (rows == 0) return Q8_OK;
     if (int st = check_io("q8_rope", x, x_dtype, y, y_dtype)) return st;
     if (!cos_t || !sin_t) return fail(Q8_ERR_NULL, "q8_rope: null table");

@@ -516,7 +516,8 @@ inline int pow2_ceil(int d) {
 }
 
 inline int check_rows(const char* who, int64_t rows, int dim) {
-    if (rows < 0) return fail(Q8_ERR_SHAPE, "%s: rows = %lld", who, (long long)rows);
+    // (2^40 rows bound every rows * dim product and every rounded-up row count far below the range of int64)
+    if (rows < 0 || rows > ((int64_t)1 << 40)) return fail(Q8_ERR_SHAPE, "%s: rows = %lld", who, (long long)rows);
     if (dim <= 0 || dim % 8 != 0 || dim > 32768)
         return fail(Q8_ERR_SHAPE, "%s: dim = %d must be a multiple of 8 in [8, 32768]", who, dim);
     return Q8_OK;
