@@ -160,6 +160,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                                          (__attribute__((address_space(3))) void*)d1, 4, 0, 0);
     };
     int l_item = 0, l_k = 0, gl = 0;  // copy side: item, stage inside the item, global stage count
+    Item nxt{};                       // the tile the copy side moved to last: the compute side's next one
     auto issue_copy = [&](int i) {    // copy instruction i (0 .. NCOPY-1) of the copy side's current stage
         uint8_t* base = lds + (gl & 1) * kPipeStageBytes;
         const uint32_t k0 = copy_live ? (uint32_t)l_k << 7 : 0u;
@@ -176,6 +177,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         ++l_item;
         copy_live = l_item < count;
         const Item it = item_of(copy_live ? l_item : 0);
+        nxt = it;
         if (copy_live) set_src(it);
         else set_src_zeros();
         copy_params(it, l_item & 1, copy_live);
@@ -217,22 +219,17 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
 
     int g = 0;  // compute side: global stage count
     for (int item = 0; item < count; ++item) {
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][t][e] = 0;
-
-        for (int k = 0; k < KT; ++k, ++g) {
-            const bool last = (k == KT - 1);
+        // One K stage. FIRST (the first stage of a tile, peeled off the loop below) starts the accumulators from a
+        // constant zero in its first K half instead of clearing them beforehand.
+        auto stage = [&](auto first_tag, const bool last) {
+            constexpr bool FIRST = decltype(first_tag)::value;
             // f0: first K half of stage g (reads in flight); the copies of stage g+1 are in flight
             pipe_wait_frags(f0);
             read_half(f1, g, 1);
             pipe_pin(f0);
             // First half. Once the second half of stage g is in registers everywhere (barrier 1), buffer g & 1 is
             // free and the copies of stage g+2 start to trickle out, one per MFMA tile.
-            pipe_mfma<IN, MT>(f0, acc, [&](int j) {
+            pipe_mfma<IN, MT, FIRST>(f0, acc, [&](int j) {
                 if (j == MT - 1) {
                     pipe_wait_frags(f1);
                     __builtin_amdgcn_s_barrier();
@@ -257,7 +254,10 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
-        }
+            ++g;
+        };
+        stage(std::true_type{}, false);  // K > 256: never the last stage
+        for (int k = 1; k < KT; ++k) stage(std::false_type{}, k == KT - 1);
 
         // ---- epilogue of tile `item`: lane (r32, h) holds for MFMA tile (i, t) and register octet wp the 8 columns
         //      32 t + 16 wp + 8 h .. + 7 of the wave's 64-column slab, row 32 i + r32.
@@ -414,9 +414,13 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         if (m < M && n < N) *reinterpret_cast<v4u*>(cbase + (size_t)m * ldc + n) = outc[t][wp];
                     }
             } else {
+            // rows 16 half .. 16 half + 15 of the MFMA tile: their lanes write, then all lanes read 16 full rows. The
+            // two rounds use the same 2 KiB and are issued back to back without a wait in between: a wave's LDS
+            // instructions execute in order, so the reads of a round see its writes and the writes of the second
+            // round come after the reads of the first. Only the stores wait, for the data they send.
+            v4i w[2][2];
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                // rows 16 half .. 16 half + 15 of the MFMA tile: their lanes write, then all lanes store 16 full rows
                 if ((r32 >> 4) == half) {
                     const int row = r32 & 15;
 #pragma unroll
@@ -425,22 +429,24 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         for (int wp = 0; wp < 2; ++wp)
                             lds_write_b128(stage_out + row * 128 + (((4 * t + 2 * wp + h) ^ ((row >> 1) & 7)) * 16), outc[t][wp]);
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                v4i w[2];
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int row = 8 * j + (lane_e >> 3);
-                    w[j] = lds_read_b128<0>(stage_out + row * 128 + (((lane_e & 7) ^ ((row >> 1) & 7)) * 16));
+                    w[half][j] = lds_read_b128<0>(stage_out + row * 128 + (((lane_e & 7) ^ ((row >> 1) & 7)) * 16));
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0]), "+v"(w[1]) : : "memory");
+            }
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                if (half == 0) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(w[0][0]), "+v"(w[0][1]) : : "memory");
+                else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[1][0]), "+v"(w[1][1]) : : "memory");
                 if constexpr (RES) {
                     if (p.gate != nullptr) {
 #pragma unroll
                         for (int j = 0; j < 2; ++j)
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e], gg = (uint32_t)gq[e];
-                                w[j][e] = (int)pack2_bf16(
+                                const uint32_t a = (uint32_t)w[half][j][e], r = res[half][j][e], gg = (uint32_t)gq[e];
+                                w[half][j][e] = (int)pack2_bf16(
                                     __builtin_fmaf(__uint_as_float(a << 16), __uint_as_float(gg << 16), __uint_as_float(r << 16)),
                                     __builtin_fmaf(__uint_as_float(a & 0xffff0000u), __uint_as_float(gg & 0xffff0000u),
                                                    __uint_as_float(r & 0xffff0000u)));
@@ -450,9 +456,9 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         for (int j = 0; j < 2; ++j)
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                const uint32_t a = (uint32_t)w[j][e], r = res[half][j][e];
-                                w[j][e] = (int)pack2_bf16(__uint_as_float(a << 16) + __uint_as_float(r << 16),
-                                                          __uint_as_float(a & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
+                                const uint32_t a = (uint32_t)w[half][j][e], r = res[half][j][e];
+                                w[half][j][e] = (int)pack2_bf16(__uint_as_float(a << 16) + __uint_as_float(r << 16),
+                                                                __uint_as_float(a & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
                             }
                     }
                 }
@@ -460,12 +466,12 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                 for (int j = 0; j < 2; ++j) {
                     const int m = mw0 + 32 * i + 16 * half + 8 * j + (lane_e >> 3);
                     const int n = nw0 + (lane_e & 7) * 8;
-                    if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * ldc + n) = w[j];
+                    if (m < M && n < N) *reinterpret_cast<v4i*>(cbase + (size_t)m * ldc + n) = w[half][j];
                 }
             }
             }
         }
-        if (item + 1 < count) cur = item_of(item + 1);
+        cur = nxt;  // the copy side entered tile item + 1 two stages before this tile's last one (K > 256: and no further tile yet)
         read_half(f0, g, 0);  // first fragments of the next tile (its first two stages landed before barrier 2 above)
     }
     // drain: the look-ahead copies and fragment reads past the last stage target LDS / registers that nobody uses

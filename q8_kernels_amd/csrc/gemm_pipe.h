@@ -94,19 +94,21 @@ __device__ __forceinline__ void pipe_pin(PipeFragsT<MT>& f) {
 // The 2 MT (fp8) / 4 MT (int8) MFMAs of one K half. `between(j)` runs after the j-th of the 2 MT tiles with scheduling
 // fences around it, so that whatever it issues (one HBM->LDS copy) stays between two MFMAs: a wave that issued
 // all copies of a stage back to back would sit in the full vector-memory queue instead of feeding the matrix pipe.
-template <int IN, int MT, typename ACC, typename F>
+template <int IN, int MT, bool ZERO = false, typename ACC, typename F>
 __device__ __forceinline__ void pipe_mfma(const PipeFragsT<MT>& f, ACC (&acc)[MT][2], F between) {
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
+            // ZERO: the first products of a tile; the MFMA adds them to a constant zero instead of a cleared accumulator
+            const ACC c0 = ZERO ? ACC{} : acc[i][t];
             if constexpr (IN == Q8_I8) {
-                acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[t][0], f.a[i][0], acc[i][t], 0, 0, 0);
+                acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[t][0], f.a[i][0], c0, 0, 0, 0);
                 acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[t][1], f.a[i][1], acc[i][t], 0, 0, 0);
             } else {
                 const v8i bf = {f.b[t][0][0], f.b[t][0][1], f.b[t][0][2], f.b[t][0][3], f.b[t][1][0], f.b[t][1][1], f.b[t][1][2], f.b[t][1][3]};
                 const v8i af = {f.a[i][0][0], f.a[i][0][1], f.a[i][0][2], f.a[i][0][3], f.a[i][1][0], f.a[i][1][1], f.a[i][1][2], f.a[i][1][3]};
-                acc[i][t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf, af, acc[i][t], 0, 0, 0, 0, 0, 0);
+                acc[i][t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf, af, c0, 0, 0, 0, 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
             between(2 * i + t);
