@@ -119,7 +119,7 @@ __device__ __forceinline__ void store_o_tile(void* o, size_t row_off, int h, con
 // lane receives the complete row sum (both key halves) of that lane's own query: no cross-lane step, and the 32
 // additions per tile of the vector ALU are gone.
 template <int OUT, bool SCALED, int kQT, int kWaves, bool VTOK = false, bool MSUM = false>
-__global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 3 : 1) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 3 : (!SCALED && kWaves == 8 && kQT == 1) ? 4 : 1) void attn_fwd_kernel(const AttnParams p) {
     static_assert(!MSUM || (!SCALED && kQT == 1), "the matrix-pipe row sum is built for unit scales and one query tile per wave");
     constexpr int kBlockQ = kWaves * kQT * 32;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * kStage];
@@ -175,28 +175,44 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
     }
     // Every wave issues exactly one (4 waves: two) copy per tile, also for tiles past the end (from a block of
     // zeros into a free stage), so that "s_waitcnt vmcnt(n)" always means "all but the n youngest tiles".
+    // A tile that lies wholly inside the sequence (all but the last one) takes its source addresses from a uniform base,
+    // advanced on the scalar unit, plus a per-lane byte offset that never changes; only the last tile clamps its rows.
+    const uint32_t k_off = (uint32_t)k_src_row * 64u + (uint32_t)cchunk * 16u;
+    const bool v_off32 = VTOK || (uint64_t)p.v_row_stride * 64u < (1ull << 32);  // the per-lane V offset fits 32 bits
+    const uint32_t v_off = VTOK ? (uint32_t)crow * 64u + (uint32_t)vchunk * 16u
+                                : (uint32_t)crow * (uint32_t)p.v_row_stride + (uint32_t)cchunk * 16u;
     auto issue_loads = [&](int tile, bool real) {
         uint8_t* base = lds + (tile & (kStages - 1)) * kStage;
         const int kv0 = tile * kKV;
-        int kr = kv0 + k_src_row;
-        kr = kr < N ? kr : N - 1;
+        const bool inside = real && kv0 + kKV <= N && v_off32 && (VTOK || (int64_t)kv0 + kKV <= p.v_row_stride);  // uniform
         const uint8_t* zero = reinterpret_cast<const uint8_t*>(g_attn_zero16);
-        const uint8_t* ks = real ? Kg + (size_t)kr * 64 + cchunk * 16 : zero;
-        if (copy_k)
+        if (copy_k) {
+            const uint8_t* ks;
+            if (inside) {
+                ks = (Kg + (size_t)kv0 * 64) + k_off;
+            } else {
+                int kr = kv0 + k_src_row;
+                kr = kr < N ? kr : N - 1;
+                ks = real ? Kg + (size_t)kr * 64 + cchunk * 16 : zero;
+            }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
                                              (__attribute__((address_space(3))) void*)(base + cw * 1024), 16, 0, 0);
-        const uint8_t* vs;
-        if constexpr (VTOK) {
-            int vr = kv0 + crow;
-            vr = vr < N ? vr : N - 1;  // rows past the end repeat the last key; their probabilities are zero
-            vs = real ? Vg + (size_t)vr * 64 + vchunk * 16 : zero;
-        } else {
-            const int col = kv0 + cchunk * 16;
-            vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
         }
-        if (copy_v)
+        if (copy_v) {
+            const uint8_t* vs;
+            if (inside) {
+                vs = (VTOK ? Vg + (size_t)kv0 * 64 : Vg + kv0) + v_off;
+            } else if constexpr (VTOK) {
+                int vr = kv0 + crow;
+                vr = vr < N ? vr : N - 1;  // rows past the end repeat the last key; their probabilities are zero
+                vs = real ? Vg + (size_t)vr * 64 + vchunk * 16 : zero;
+            } else {
+                const int col = kv0 + cchunk * 16;
+                vs = (real && col < p.v_row_stride) ? (Vg + (size_t)crow * p.v_row_stride + col) : zero;
+            }
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
                                              (__attribute__((address_space(3))) void*)(base + 4096 + cw * 1024), 16, 0, 0);
+        }
         if constexpr (SCALED) {
             if (wave == 0) {  // the 64 key scales and value scales of the tile, one dword per lane
                 int key = kv0 + lane;
@@ -232,8 +248,9 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
 #pragma unroll
             for (int e = 0; e < 16; ++e) o_acc[t][d][e] = 0.f;
     float m_run[kQT], l_run[kQT];
+    float m_thr[kQT], m_sub[kQT];  // m_run + m_slack (the threshold of the next move), m_run - exp_bias: kept beside m_run, they change with it
 #pragma unroll
-    for (int t = 0; t < kQT; ++t) { m_run[t] = -INFINITY; l_run[t] = 0.f; }
+    for (int t = 0; t < kQT; ++t) { m_run[t] = m_thr[t] = m_sub[t] = -INFINITY; l_run[t] = 0.f; }
     v4f l_acc = {0.f, 0.f, 0.f, 0.f};  // MSUM: [0] = row sum of this lane's query
     v8i ones;                          // MSUM: this lane's 32 bytes of the ones-and-zeros matrix (e4m3 1.0 = 0x38)
     {
@@ -393,33 +410,37 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
                 for (int e = 0; e < 32; ++e)
                     if (kv0 + 32 * h + e >= valid) x[e] = -INFINITY;
             }
-            float mx = fmaxf(x[0], x[1]);
+            float mx = max_ieee(x[0], x[1]);
 #pragma unroll
-            for (int e = 2; e < 32; e += 2) mx = fmaxf(fmaxf(mx, x[e]), x[e + 1]);
-            mx = fmaxf(mx, lane_xor<32>(mx));
+            for (int e = 2; e < 32; e += 2) mx = max_ieee(max_ieee(mx, x[e]), x[e + 1]);
+            mx = half_pair_max(mx);
             const float c = sqc[qt];
             // The reference maximum m of a row moves (and O, l are rescaled) only when the tile's maximum exceeds it by
             // more than m_slack (0 unless Q8_ATTN_LAZY_MAX: the running maximum), so p <= 2^(p_shift + m_slack). Each
             // row decides for itself (its result does not depend on the rows it shares a wave with); the wave skips
             // the multiplications when no row moves.
             const float mxc = mx * c;
-            const bool grow = mxc > m_run[qt] + p.m_slack;
+            const bool grow = mxc > (MSUM ? m_run[qt] + p.m_slack : m_thr[qt]);  // (MSUM is short of registers: it recomputes the two)
             if (__builtin_amdgcn_ballot_w64(grow) != 0) {
                 const float alpha = grow ? fast_exp2(m_run[qt] - mxc) : 1.f;
                 m_run[qt] = grow ? mxc : m_run[qt];
+                if constexpr (!MSUM) {
+                    m_thr[qt] = m_run[qt] + p.m_slack;
+                    m_sub[qt] = m_run[qt] - exp_bias;
+                }
                 if constexpr (MSUM) l_acc[0] *= alpha; else l_run[qt] *= alpha;
 #pragma unroll
                 for (int d = 0; d < 2; ++d)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) o_acc[qt][d][e] *= alpha;
             }
-            const float m_sub = m_run[qt] - exp_bias;
+            const float ms = MSUM ? m_run[qt] - exp_bias : m_sub[qt];
             float psum = 0.f;
             float pr[32];
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
-                pr[e] = fast_exp2(fmaf(x[e], c, -m_sub));   // <= 2^(p_shift + m_slack) = 2^8 or 1: inside the e4m3 range
-                if constexpr (!MSUM) psum += pr[e];
+                pr[e] = fast_exp2(fmaf(x[e], c, -ms));   // <= 2^(p_shift + m_slack) = 2^8 or 1: inside the e4m3 range
+                if constexpr (!MSUM) psum = e ? psum + pr[e] : pr[0];
             }
             if constexpr (SCALED) {
                 if (qt == 0) {
@@ -437,7 +458,7 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
             v8i pf;
 #pragma unroll
             for (int w = 0; w < 8; ++w) {
-                uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
+                uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], any_u32(), false);
                 u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
                 pf[w] = (int)u;
             }
@@ -534,9 +555,9 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
             }
         }
 #pragma unroll
-        for (int e = 0; e < 32; e += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[kb][e]), x[kb][e + 1]);
+        for (int e = 0; e < 32; e += 2) mx = max_ieee(max_ieee(mx, x[kb][e]), x[kb][e + 1]);
     }
-    mx = fmaxf(mx, lane_xor<32>(mx));
+    mx = half_pair_max(mx);
     const float m_sub = mx * c - bias;  // the final maximum is known: the slack of Q8_ATTN_LAZY_MAX is head room not needed
     float psum = 0.f, psum_rounded = 0.f;
     v16f o_acc[2];
@@ -593,7 +614,7 @@ __device__ __forceinline__ void short_tile(const AttnParams& p, const v8i& qf, u
         }
 #pragma unroll
         for (int w = 0; w < 8; ++w) {
-            uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], 0u, false);
+            uint32_t u = cvt_pk_e4m3(pr[4 * w], pr[4 * w + 1], any_u32(), false);
             u = cvt_pk_e4m3(pr[4 * w + 2], pr[4 * w + 3], u, true);
             pf[w] = (int)u;
         }

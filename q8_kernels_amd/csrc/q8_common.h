@@ -43,6 +43,15 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t packed) {
     return __builtin_amdgcn_cvt_f32_fp8((int)packed, SEL);
 }
 
+// a register with unspecified contents (no instruction): the `old` operand of a conversion whose other half is written next
+// (used where the instruction count is the bound, the attention tile loop; elsewhere the fence of the volatile statement
+//  costs the scheduler more than the move it saves)
+__device__ __forceinline__ uint32_t any_u32() {
+    uint32_t u;
+    asm volatile("" : "=v"(u));
+    return u;
+}
+
 // Two fp32 -> two e4m3fn codes in the low or high half of a word, hardware RNE.
 __device__ __forceinline__ uint32_t cvt_pk_e4m3(float a, float b, uint32_t old, bool hi) {
     return hi ? (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true)
@@ -124,6 +133,15 @@ __device__ __forceinline__ float lane_xor(float x) {
     }
 }
 
+// IEEE-754 maximum (NaN-propagating; v_maximum3_f32 on gfx950). Unlike fmaxf it needs no canonicalization of operands the
+// compiler cannot prove free of signalling NaNs (MFMA results, lane swaps): one instruction per two new values.
+__device__ __forceinline__ float max_ieee(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+// max of a value over the two lanes l, l ^ 32: v_permlane32_swap of two copies leaves (low half, low half) in one and
+// (high half, high half) in the other, so every lane holds both values and no select is needed
+__device__ __forceinline__ float half_pair_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return max_ieee(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 template <int LANES>
 __device__ __forceinline__ float group_max(float v) {
     if constexpr (LANES > 1) v = fmaxf(v, lane_xor<1>(v));
