@@ -215,13 +215,22 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
         }
         if constexpr (SCALED) {
             if (wave == 0) {  // the 64 key scales and value scales of the tile, one dword per lane
-                int key = kv0 + lane;
-                key = key < N ? key : N - 1;
                 const float* zf = reinterpret_cast<const float*>(g_attn_zero16);
                 float* dst = lds_sc + (tile & (kStages - 1)) * 128;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sk + (size_t)bh * N + key : zf),
+                const float *ksrc, *vsrc;
+                if (inside) {  // uniform base of the tile + the lane's dword
+                    const uint32_t lane4 = (uint32_t)lane * 4u;
+                    ksrc = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(p.sk + (size_t)bh * N + kv0) + lane4);
+                    vsrc = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(p.sv + (size_t)bh * N + kv0) + lane4);
+                } else {
+                    int key = kv0 + lane;
+                    key = key < N ? key : N - 1;
+                    ksrc = real ? p.sk + (size_t)bh * N + key : zf;
+                    vsrc = real ? p.sv + (size_t)bh * N + key : zf;
+                }
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ksrc,
                                                  (__attribute__((address_space(3))) void*)dst, 4, 0, 0);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(real ? p.sv + (size_t)bh * N + key : zf),
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
                                                  (__attribute__((address_space(3))) void*)(dst + 64), 4, 0, 0);
             }
         }
