@@ -198,6 +198,14 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
         const unsigned so = (stage & 1) * kPipeStageBytes;
         pipe_read_frags<MT>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
     };
+    auto read_part = [&](PipeFragsT<MT>& f, int stage, int s, auto part) {  // one of the four parts of read_half
+        const unsigned so = (stage & 1) * kPipeStageBytes;
+        pipe_read_frags_part<MT, decltype(part)::value>(f, a_row + so + pc[s][0], a_row + so + pc[s][1], b_row + so + pc[s][0], b_row + so + pc[s][1]);
+    };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
+    using P3 = std::integral_constant<int, 3>;
 
     using acc_t = typename std::conditional<IN == Q8_I8, v16i, v16f>::type;
     acc_t acc[MT][2];
@@ -225,11 +233,21 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
             constexpr bool FIRST = decltype(first_tag)::value;
             // f0: first K half of stage g (reads in flight); the copies of stage g+1 are in flight
             pipe_wait_frags(f0);
-            read_half(f1, g, 1);
             pipe_pin(f0);
-            // First half. Once the second half of stage g is in registers everywhere (barrier 1), buffer g & 1 is
-            // free and the copies of stage g+2 start to trickle out, one per MFMA tile.
+            // First half. The operand reads of the second half go out a part after each of the first MFMAs, not as one
+            // burst: a wave that issues a dozen LDS reads back to back keeps the matrix pipe waiting, and its partner on
+            // the SIMD does the same at the same time. Once the second half of stage g is in registers everywhere
+            // (barrier 1), buffer g & 1 is free and the copies of stage g+2 start to trickle out, one per MFMA tile.
             pipe_mfma<IN, MT, FIRST>(f0, acc, [&](int j) {
+                if (j == 0) read_part(f1, g, 1, P0{});
+                if (j == 1) {
+                    read_part(f1, g, 1, P1{});
+                    if constexpr (MT == 3) read_part(f1, g, 1, P2{});
+                }
+                if (MT == 4 && j == 2) {
+                    read_part(f1, g, 1, P2{});
+                    read_part(f1, g, 1, P3{});
+                }
                 if (j == MT - 1) {
                     pipe_wait_frags(f1);
                     __builtin_amdgcn_s_barrier();
@@ -249,8 +267,20 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     if (moved) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NCOPY + 2) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NCOPY) : "memory");
                     __builtin_amdgcn_s_barrier();
-                    // the fragment registers are free for the epilogue after the last stage of a tile
-                    if (!last) read_half(f0, g + 1, 0);
+                    // the fragment registers are free for the epilogue after the last stage of a tile; the reads of the
+                    // next stage's first half are spread over the remaining MFMA slots like those above
+                    if (!last) {
+                        read_part(f0, g + 1, 0, P0{});
+                        if constexpr (MT == 3) read_part(f0, g + 1, 0, P1{});
+                    }
+                }
+                if (!last && j == 5) {
+                    if constexpr (MT == 4) read_part(f0, g + 1, 0, P1{});
+                    else read_part(f0, g + 1, 0, P2{});
+                }
+                if (!last && MT == 4 && j == 6) {
+                    read_part(f0, g + 1, 0, P2{});
+                    read_part(f0, g + 1, 0, P3{});
                 }
             });
             __builtin_amdgcn_sched_barrier(0);

@@ -56,6 +56,29 @@ __device__ __forceinline__ void pipe_read_frags(PipeFragsT<MT>& f, unsigned a0, 
     }
 }
 
+// The same reads in four parts, in the order in which the MFMAs of a K half need them: part 0 = B tile 0 and A tile 0
+// (4 reads), part 1 = B tile 1 and A tile 1 (4), part 2 = A tile 2 (2), part 3 = A tile 3 (2, MT = 4 only).
+template <int MT, int PART>
+__device__ __forceinline__ void pipe_read_frags_part(PipeFragsT<MT>& f, unsigned a0, unsigned a1, unsigned b0, unsigned b1) {
+    if constexpr (PART == 0) {
+        f.b[0][0] = lds_read_b128<0>(b0);
+        f.b[0][1] = lds_read_b128<0>(b1);
+        f.a[0][0] = lds_read_b128<0>(a0);
+        f.a[0][1] = lds_read_b128<0>(a1);
+    } else if constexpr (PART == 1) {
+        f.b[1][0] = lds_read_b128<4096>(b0);
+        f.b[1][1] = lds_read_b128<4096>(b1);
+        f.a[1][0] = lds_read_b128<4096>(a0);
+        f.a[1][1] = lds_read_b128<4096>(a1);
+    } else if constexpr (PART == 2) {
+        f.a[2][0] = lds_read_b128<8192>(a0);
+        f.a[2][1] = lds_read_b128<8192>(a1);
+    } else if constexpr (MT == 4) {
+        f.a[3][0] = lds_read_b128<12288>(a0);
+        f.a[3][1] = lds_read_b128<12288>(a1);
+    }
+}
+
 // Wait until every LDS read issued so far has landed; the fragments pass through the statement so that no
 // MFMA consuming them can be scheduled above it.
 template <int MT>
