@@ -118,6 +118,34 @@ def test_attention_kv_length_mask(dev, attn_cfg, p_grid, lens):
             assert (got[b].cpu().float() == 0).all()  # nothing to attend to: zeros
 
 
+@pytest.mark.parametrize("n", [100, 300])
+def test_attention_nan_codes(dev, attn_cfg, n):
+    """The e4m3 NaN code (0x7f) behaves as in float attention on the dequantised operands: in a valid key it makes every
+    query row of that (batch, head) NaN, in a query it makes that row NaN and no other, and in a key past the valid length
+    it has no influence at all (a masked VALUE must be finite: its weight is zero, and 0 * NaN is NaN in any arithmetic).
+    (100 keys: the short-sequence kernel, 300: the general one.)"""
+    q, k, v = _inputs(5, 2, 2, 150, n)
+    kv_len = torch.tensor([n, n - 40], dtype=torch.int32)
+    run = lambda q_, k_, v_: _C().flash_attention(q_.to(dev), k_.to(dev), _vt(v_).to(dev), 0.125, kv_len.to(dev),
+                                                  out_dtype=torch.bfloat16).cpu()
+    base = run(q, k, v)
+    assert not torch.isnan(base).any()
+    k2 = k.clone().view(torch.uint8)
+    k2[0, 1, 17, 3] = 0x7f               # a valid key of (batch 0, head 1)
+    k2[1, :, n - 40:, :] = 0x7f          # masked keys of batch 1
+    v2 = v.clone().view(torch.uint8)
+    v2[1, :, n - 40:, :] = 0x7e          # masked values of batch 1: the largest finite code
+    q2 = q.clone().view(torch.uint8)
+    q2[1, 0, 77, 40] = 0x7f              # one query row of (batch 1, head 0)
+    got = run(q2.view(E4M3), k2.view(E4M3), v2.view(E4M3))
+    assert torch.isnan(got[0, 1]).all()
+    assert torch.isnan(got[1, 0, 77]).all()
+    keep = torch.ones(2, 2, 150, dtype=torch.bool)
+    keep[0, 1] = False
+    keep[1, 0, 77] = False
+    assert torch.equal(got[keep].view(torch.int16), base[keep].view(torch.int16))
+
+
 def test_attention_large_logits_and_scale(dev):
     q, k, v = _inputs(77, 1, 2, 128, 256, std=4.0)
     for scale in (0.125, 0.02, 1.0):
