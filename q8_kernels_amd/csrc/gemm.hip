@@ -299,9 +299,12 @@ template <int IN, bool GELU, bool E4M3OUT = false>
 static int launch_persist(const GemmParams& p, hipStream_t stream) {
     const long batch = p.batch_a > p.batch_b ? p.batch_a : p.batch_b;
     const long tn = (p.N + kPipeBN - 1) / kPipeBN, cus = persist_cus();
+    // (with a residual the 256-row kernel is 256 registers short by a dozen: it spills copy offsets around its epilogue
+    //  and runs 10-15 % slower than its tile count says, measured; the 192-row kernel does not)
+    const double cost256 = (!E4M3OUT && p.residual != nullptr) ? 1.25 : 1.0;
     auto cost = [&](int bm) {
         const long tiles = (long)((p.M + bm - 1) / bm) * tn * batch;
-        return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? 1.0 : 1.2);
+        return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? cost256 : 1.2);
     };
     const bool small = g_persist_mt == 3 || (g_persist_mt == 0 && cost(192) < cost(256));
     if constexpr (!E4M3OUT && !GELU) {
