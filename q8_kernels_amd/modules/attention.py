@@ -20,6 +20,13 @@ class Attention(nn.Module):
     # True (default): on the fused self-attention path the V projection's GEMM writes the attention kernel's e4m3 operand
     # itself; False: V passes through memory as bfloat16 and the prologue casts it. The same bits either way.
     cast_v_in_gemm = True
+    # True (default): on the fused path the projections that share an input run as ONE GEMM over the concatenation of their
+    # weights - q, k, v of a self-attention (V leaves it as the attention kernel's e4m3 operand), k and v of a
+    # cross-attention - instead of one launch per layer. The concatenation is a copy made on first use and made again when a
+    # layer's weight, scales or bias is replaced or modified through the parameter (in-place writes through `.data` are not
+    # seen: call invalidate_fused_weights() after them). Every output column depends on its own weight row only and is
+    # accumulated in the same order whatever the tile it falls into: the same bits as the separate layers.
+    fuse_projections = True
 
     def __init__(self, query_dim: int, num_heads: int, head_dim: int, bias: bool = False, out_bias: bool = False,
                  out_dim: Optional[int] = None, qk_rms_norm: bool = False, kv_dim: Optional[int] = None,
@@ -42,6 +49,40 @@ class Attention(nn.Module):
         self.to_k = Q8Linear(kv_dim, self.inner_dim, bias=bias)
         self.to_v = Q8Linear(kv_dim, self.inner_dim, bias=bias)
         self.to_out = Q8Linear(self.inner_dim, out_dim, out_bias)
+
+    def invalidate_fused_weights(self):
+        """Drop the concatenated copies of the projection weights (they are rebuilt on the next call)."""
+        self.__dict__.pop("_fused_weights", None)
+
+    def _fused_weights_of(self, names):
+        """(weight, bias or None, scales) of the layers `names` concatenated along the output dimension; None when the
+        copy would have to be made while a graph is being captured (it would live in the graph's memory pool and die with
+        the graph: the caller then takes the separate layers)."""
+        layers = [getattr(self, n) for n in names]
+        tensors = [t for layer in layers for t in (layer.weight, layer.scales, layer.bias) if t is not None]
+        key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in tensors)
+        cache = self.__dict__.setdefault("_fused_weights", {})
+        hit = cache.get(names)
+        if hit is None or hit[0] != key:
+            if layers[0].weight.is_cuda and torch.cuda.is_current_stream_capturing():
+                return None
+            weight = torch.cat([layer.weight.data for layer in layers])
+            scales = torch.cat([layer.scales for layer in layers])
+            bias = None
+            if any(layer.bias is not None for layer in layers):
+                bias = torch.cat([layer.bias.data if layer.bias is not None
+                                  else torch.zeros(layer.out_features, dtype=torch.float32, device=weight.device) for layer in layers])
+            hit = cache[names] = (key, weight, bias, scales)
+        return hit[1], hit[2], hit[3]
+
+    def _can_fuse_projections(self, names, mm_out_dtype, non_mm_precision, attn_type):
+        layers = [getattr(self, n) for n in names]
+        k_in = layers[0].in_features
+        return (self.fuse_projections and self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64
+                and mm_out_dtype == torch.bfloat16 and non_mm_precision == torch.bfloat16 and not torch.is_grad_enabled()
+                and all(type(layer) is Q8Linear and layer.in_features == k_in and layer.out_features == self.inner_dim for layer in layers)
+                and (self.inner_dim in (64, 128, 256) or (self.inner_dim % 512 == 0 and self.inner_dim <= 4096))
+                and len(layers) * self.inner_dim * k_in < 2 ** 32)
 
     def _norm_weight(self, norm):
         if norm.weight is not None:
@@ -109,13 +150,40 @@ class Attention(nn.Module):
                 # (and the operand sizes the persistent GEMM addresses with 32-bit offsets; larger ones take the plain projection)
                 if (isinstance(x, tuple) and x[0].dim() == 3 and x[0].dtype == torch.int8
                         and x[0].numel() < 2 ** 32 and self.to_v.weight.numel() < 2 ** 32):
-                    query, key = project([self.to_q, self.to_k], x)
-                    v_codes = _C.mm_bias_qkv(x[0].reshape(-1, k_in), self.to_v.weight.data, self.to_v._bias(), x[1].reshape(-1),
-                                             self.to_v.scales, x[0].shape[1], 0)[1]
+                    if (self._can_fuse_projections(("to_q", "to_k", "to_v"), mm_out_dtype, non_mm_precision, attn_type)
+                            and (2 * self.inner_dim) % 256 == 0):
+                        # one GEMM over [Wq; Wk; Wv]: Q and K come back as the two halves of one bfloat16 tensor (read in place
+                        # by the prologue), the V columns as e4m3 codes
+                        fused = self._fused_weights_of(("to_q", "to_k", "to_v"))
+                    else:
+                        fused = None
+                    if fused is not None:
+                        qk, v_codes = _C.mm_bias_qkv(x[0].reshape(-1, k_in), fused[0], fused[1], x[1].reshape(-1), fused[2], x[0].shape[1],
+                                                     2 * self.inner_dim)
+                        query, key = qk[..., :self.inner_dim], qk[..., self.inner_dim:]
+                    else:
+                        query, key = project([self.to_q, self.to_k], x)
+                        v_codes = _C.mm_bias_qkv(x[0].reshape(-1, k_in), self.to_v.weight.data, self.to_v._bias(), x[1].reshape(-1),
+                                                 self.to_v.scales, x[0].shape[1], 0)[1]
             if v_codes is None:
                 query, key, value = project([self.to_q, self.to_k, self.to_v], x)
         else:
-            (query,), (key, value) = project([self.to_q], hidden_states), project([self.to_k, self.to_v], kv_src)
+            (query,) = project([self.to_q], hidden_states)
+            kv = None
+            if self._can_fuse_projections(("to_k", "to_v"), mm_out_dtype, non_mm_precision, attn_type):
+                xkv = kv_src
+                if not isinstance(xkv, tuple) and xkv.is_cuda and xkv.dim() == 3 and Q8F.fused.can_fuse_hadamard_quantize(xkv):
+                    xkv = Q8F.fused.hadamard_quantize(xkv)
+                if isinstance(xkv, tuple) and xkv[0].dim() == 3 and xkv[0].dtype == torch.int8:
+                    kv_src = xkv  # (should the separate layers run after all, they take these codes)
+                    fused = self._fused_weights_of(("to_k", "to_v"))
+                    if fused is not None:
+                        # one GEMM over [Wk; Wv]: K and V are the two halves of one tensor, read in place by the prologue
+                        kv = Q8F.linear.q8_linear(xkv[0], fused[0], fused[1], xkv[1], fused[2], False, mm_out_dtype)
+                        kv = kv.reshape(xkv[0].shape[0], xkv[0].shape[1], 2 * self.inner_dim)
+                        key, value = kv[..., :self.inner_dim], kv[..., self.inner_dim:]
+            if kv is None:
+                key, value = project([self.to_k, self.to_v], kv_src)
         rope = encoder_hidden_states is None and self.use_rope
         batch = query.shape[0]
         if (self.fuse_prologue and attn_type == "q8_kernels" and self.head_dim == 64

@@ -358,6 +358,57 @@ def test_attention_module_v_cast_in_gemm_equals_both_other_paths(dev):
     assert_bit_equal(in_gemm, seq, "V cast in the GEMM vs operator sequence")
 
 
+def test_attention_module_fused_projections_equal_separate_layers(dev):
+    """fuse_projections: q, k, v of a self-attention (one q8_gemm_qkv over the three weights) and k, v of a cross-attention
+    (one GEMM over the two) give the bits of one GEMM per layer; the concatenated weights follow a replaced layer weight."""
+    import torch.nn as nn
+    import q8_kernels_amd.functional.linear as FL
+    from q8_kernels_amd.modules import Attention, Q8Linear
+    torch.manual_seed(11)
+
+    def fill(attn):
+        for name in ("to_q", "to_k", "to_v", "to_out"):
+            m = getattr(attn, name)
+            q = Q8Linear.from_linear(nn.Linear(m.in_features, m.out_features).to(dev).to(BF16))
+            m.weight.data, m.scales.data, m.bias.data = q.weight.data, q.scales.data, q.bias.data
+        return attn
+
+    self_attn = fill(Attention(512, 8, 64, bias=True, out_bias=True, qk_rms_norm=True, use_rope=True).to(dev))
+    cross = fill(Attention(512, 8, 64, bias=True, out_bias=True, kv_dim=384).to(dev))
+    x = torch.randn(2, 300, 512, device=dev).to(BF16)
+    text = torch.randn(2, 40, 384, device=dev).to(BF16)
+    lens = torch.tensor([40, 13], dtype=torch.int32, device=dev)
+    ang = torch.rand(2, 300, 256, device=dev) * 6.28
+    freqs = (torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1))
+    kw_self = dict(freqs_cis=freqs, mm_out_dtype=BF16, attn_type="q8_kernels")
+    kw_cross = dict(encoder_hidden_states=text, attention_mask=lens, mm_out_dtype=BF16, attn_type="q8_kernels")
+    saved, calls = FL.q8_linear, {"n": 0}
+    def counted(*a, **k):
+        calls["n"] += 1
+        return saved(*a, **k)
+    try:
+        FL.q8_linear = counted
+        with torch.no_grad():
+            fused_self, n_self = self_attn(x, **kw_self), calls["n"]
+            fused_cross, n_cross = cross(x, **kw_cross), calls["n"] - n_self
+            # a replaced weight is seen
+            q = Q8Linear.from_linear(nn.Linear(384, 512).to(dev).to(BF16))
+            cross.to_k.weight.data, cross.to_k.scales.data = q.weight.data, q.scales.data
+            fused_cross2 = cross(x, **kw_cross)
+            Attention.fuse_projections = False
+            calls["n"] = 0
+            sep_self, m_self = self_attn(x, **kw_self), calls["n"]
+            sep_cross2, m_cross = cross(x, **kw_cross), calls["n"] - m_self
+    finally:
+        FL.q8_linear = saved
+        Attention.fuse_projections = True
+    assert (n_self, m_self) == (1, 3), "self-attention: %d / %d calls of q8_linear (the output projection; q, k on top without fusion)" % (n_self, m_self)
+    assert (n_cross, m_cross) == (3, 4), "cross-attention: %d / %d calls of q8_linear" % (n_cross, m_cross)
+    assert_bit_equal(fused_self, sep_self, "self-attention, fused projections vs separate layers")
+    assert_bit_equal(fused_cross2, sep_cross2, "cross-attention after a weight replacement, fused vs separate")
+    assert not torch.equal(fused_cross, fused_cross2), "the concatenated weights did not follow the replaced layer"
+
+
 def test_attention_module_fused_path_equals_operator_sequence(dev):
     import torch.nn as nn
     from q8_kernels_amd.modules import Attention, Q8Linear
