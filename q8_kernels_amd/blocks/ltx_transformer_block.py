@@ -40,21 +40,28 @@ class LTXTransformerBlock(nn.Module):
     def forward(self, hidden_states, freqs_cis, attention_mask, encoder_hidden_states, encoder_attention_mask,
                 timestep, mm_out_dtype=torch.bfloat16, non_mm_precision=torch.bfloat16, attn_type="torch"):
         num_ada_params = self.scale_shift_table.shape[0]
-        ada_values = self.scale_shift_table[None, None] + timestep.reshape(
-            hidden_states.shape[0], timestep.shape[1], num_ada_params, -1)
-        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada_values.unbind(dim=2)
-
+        timestep_rows = timestep.reshape(hidden_states.shape[0], timestep.shape[1], num_ada_params, -1)
         # the fused prologue goes through the C ABI and carries no gradient: it is taken only when neither the input nor
         # the modulation (scale_shift_table is a parameter, timestep may be the output of a trained embedding) needs one
         fuse = (self.fuse_prologue and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16
                 and non_mm_precision == torch.bfloat16 and hidden_states.dim() == 3 and hidden_states.shape[-1] % 8 == 0
-                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or ada_values.requires_grad)))
+                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or self.scale_shift_table.requires_grad
+                                                      or timestep.requires_grad)))
         # (cast and layout change in one copy kernel; nothing at all for a contiguous bfloat16 tensor)
         bf = lambda t: t.to(torch.bfloat16, memory_format=torch.contiguous_format)  # noqa: E731
-        if fuse:
-            # the six modulation rows as contiguous bfloat16 tensors [B, T, dim] cut from ONE copy laid out [6, B, T, dim]
-            # (instead of six strided-to-contiguous copies further down): the same values, bf16(table + timestep)
-            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = bf(ada_values.permute(2, 0, 1, 3)).unbind(dim=0)
+        if fuse and timestep_rows.dtype == self.scale_shift_table.dtype == torch.float32:
+            # the six modulation rows as contiguous bfloat16 tensors [B, T, dim] cut from ONE tensor laid out [6, B, T, dim],
+            # written by the addition itself (fp32 sum, rounded once on the way out: bf16(table + timestep), the values the
+            # separate cast gives) - one small kernel instead of an addition, a layout change and six casts
+            rows = torch.empty((num_ada_params,) + tuple(timestep_rows.shape[:2]) + (timestep_rows.shape[-1],),
+                               dtype=torch.bfloat16, device=hidden_states.device)
+            torch.add(self.scale_shift_table[None, None], timestep_rows, out=rows.permute(1, 2, 0, 3))
+            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = rows.unbind(dim=0)
+        else:
+            ada_values = self.scale_shift_table[None, None] + timestep_rows
+            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = ada_values.unbind(dim=2)
+            if fuse:
+                shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = bf(ada_values.permute(2, 0, 1, 3)).unbind(dim=0)
 
         if fuse:  # (int8 codes, row scales) of the rotated, modulated norm: what attn1's projections would compute
             norm_hidden_states = Q8F.fused.norm_modulate_quantize(hidden_states, self.norm1.weight, bf(scale_msa),
