@@ -384,6 +384,18 @@ def _extras_rows(dev, steps, warmup, g, out):
                           ("attn_prep_qkv_rope_fht_fp8", lambda: _C.attn_prep_qkv(xs, xs, xs, 32, cs3, sn3, True, 0.125), 17)):
         t, _ = _time(fn, steps, warmup)
         out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    # the paired prologue of a self-attention (Q and K) on the tables as the model builds them - every angle twice, one
+    # position grid for the batch - in full [2, 6144, 2048] (2 x 2 B in, 8 B of tables, 2 x 1 B out per element) and
+    # with the repeated values stored once ([1, 6144, 1024]: 1 B of tables per element), as the modules pass them
+    ang = torch.rand(1, 6144, 1024, generator=g) * 6.28
+    cf = torch.cos(ang).repeat_interleave(2, -1).expand(2, -1, -1).contiguous().to(dev)
+    sf = torch.sin(ang).repeat_interleave(2, -1).expand(2, -1, -1).contiguous().to(dev)
+    ch, sh = torch.cos(ang).to(dev), torch.sin(ang).to(dev)
+    for name, fn, bpe in (("attn_prep_qk_pair_rope_fht_fp8", lambda: _C.attn_prep_qk_pair(xs, xs, 32, cf, sf, True, 0.125), 14),
+                          ("attn_prep_qk_pair_rope_fht_fp8_compact_tables", lambda: _C.attn_prep_qk_pair(xs, xs, 32, ch, sh, True, 0.125), 7)):
+        t, _ = _time(fn, steps, warmup)
+        out[name] = {"ms": t * 1e3, "gbs": n * bpe / t / 1e9, "frac_of_hbm_peak": n * bpe / t / 1e9 / HBM_PEAK_GBS}
+    del cf, sf, ch, sh, ang
     # the same kernels with nothing left in any cache by the previous call (16 sets of inputs and outputs, 1.2-5 GB)
     copies = 16
     xc = [x.clone() for _ in range(copies)]

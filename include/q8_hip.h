@@ -81,6 +81,16 @@ enum {
                                   reference, which rescales against the running maximum in every tile.          */
 };
 
+/* q8_attn_prep_qk / _qk_pair / _qkv / _kv flags */
+enum {
+    Q8_PREP_FHT = 1,           /* D-point Hadamard transform * scale per head                                      */
+    Q8_PREP_PAIR_TABLES = 2,   /* cos, sin hold one entry per rotated pair, [rows, H*D/2], instead of one per
+                                  element: tables built by repeating every frequency twice
+                                  (q8_kernels/models/LTXVideo.py:95-148) carry each value twice                    */
+    Q8_PREP_SHARED_TABLES = 4  /* cos, sin hold the S positions of one batch element, [S, ...], and serve all B
+                                  batch elements, instead of one row per token [B*S, ...]                          */
+};
+
 const char* q8_strerror(int status);
 const char* q8_last_error(void);
 
@@ -203,8 +213,9 @@ int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, int apply_nor
  *
  * q8_attn_prep_qk: per token: [RMSNorm over the H*D row with fp32 weights norm_w [H*D], no epsilon (the qk-norm of
  *   q8_kernels/modules/attention.py:67-77), NULL = none] -> per head: [RoPE with tables cos, sin fp32 [B*S, H*D],
- *   both NULL = none] ->
- *   [D-point FHT * scale if apply_fht] -> e4m3 codes [B, H, S, D]. scales == NULL: direct c10 cast (the
+ *   both NULL = none; Q8_PREP_PAIR_TABLES / Q8_PREP_SHARED_TABLES in flags: the same values stored once, [B*S or S,
+ *   H*D or H*D/2], same results] ->
+ *   [D-point FHT * scale with Q8_PREP_FHT in flags] -> e4m3 codes [B, H, S, D]. scales == NULL: direct c10 cast (the
  *   reference's cast); otherwise one absmax scale per (token, head) to scales [B, H, S].
  *   D in {64, 128}; H * D in {64, 128, 256} or a multiple of 512 up to 4096.
  * q8_attn_prep_qk_pair: the same for Q and K of a self-attention in one pass (same S, same tables, read once).
@@ -218,20 +229,20 @@ int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, int apply_nor
  *   scales as above. D == 64.
  */
 int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* norm_w, const float* cos_t, const float* sin_t,
-                    void* codes, float* scales, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                    void* codes, float* scales, int B, int S, int H, int D, int flags, float scale, int mid_dtype,
                     q8_stream_t stream);
 int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
                          const float* norm_wq, const float* norm_wk, const float* cos_t, const float* sin_t,
                          void* codes_q, float* scales_q, void* codes_k, float* scales_k, int B, int S, int H, int D,
-                         int apply_fht, float scale, int mid_dtype, q8_stream_t stream);
+                         int flags, float scale, int mid_dtype, q8_stream_t stream);
 int q8_attn_prep_qkv(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride, const void* xv,
                      int64_t xv_row_stride, const float* norm_wq, const float* norm_wk, const float* cos_t,
                      const float* sin_t, void* codes_q, float* scales_q, void* codes_k, float* scales_k, void* codes_v,
-                     float* scales_v, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                     float* scales_v, int B, int S, int H, int D, int flags, float scale, int mid_dtype,
                      q8_stream_t stream);
 int q8_attn_prep_kv(const void* xk, int64_t xk_row_stride, const void* xv, int64_t xv_row_stride, const float* norm_wk,
                     const float* cos_t, const float* sin_t, void* codes_k, float* scales_k, void* codes_v, float* scales_v,
-                    int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype, q8_stream_t stream);
+                    int B, int S, int H, int D, int flags, float scale, int mid_dtype, q8_stream_t stream);
 int q8_attn_prep_v(const void* x, int64_t x_row_stride, void* codes, float* scales, int B, int S, int H, int D,
                    int S_pad, q8_stream_t stream);
 

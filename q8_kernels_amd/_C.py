@@ -496,28 +496,48 @@ def _norm_w(w, x):
     return w.contiguous()
 
 
+def _rope_tables(cos, sin, b, s, dim, who):
+    """The rotation tables of an attention prologue and the flag bits that describe their layout: float32 CUDA tensors
+    whose last dimension is H*D (one entry per element) or H*D/2 (one per rotated pair, Q8_PREP_PAIR_TABLES) and whose
+    leading dimensions hold B*S rows (one per token) or S rows (the positions of one batch element, serving all B:
+    Q8_PREP_SHARED_TABLES). Returns (cos, sin, flags)."""
+    if (cos is None) != (sin is None):
+        raise RuntimeError("%s: cos and sin come together" % who)
+    if cos is None:
+        return None, None, 0
+    flags = 0
+    for t in (cos, sin):
+        if t.dtype != torch.float32 or not t.is_cuda or t.shape != cos.shape or t.dim() < 2:
+            raise RuntimeError("%s: tables must be float32 CUDA tensors of one shape" % who)
+    last, rows = cos.shape[-1], cos.numel() // max(1, cos.shape[-1])
+    if last == dim // 2 and dim % 2 == 0 and last != dim:
+        flags |= _lib.Q8_PREP_PAIR_TABLES
+    elif last != dim:
+        raise RuntimeError("%s: the tables' last dimension must be H*D = %d or H*D/2" % (who, dim))
+    if rows == s and b > 1:
+        flags |= _lib.Q8_PREP_SHARED_TABLES
+    elif rows != b * s:
+        raise RuntimeError("%s: tables must hold one row per token (%d) or per position (%d)" % (who, b * s, s))
+    return cos.contiguous(), sin.contiguous(), flags
+
+
 def attn_prep_qk(x: torch.Tensor, num_heads: int, cos: Optional[torch.Tensor] = None,
                  sin: Optional[torch.Tensor] = None, apply_fht: bool = True, scale: float = 1.0,
                  per_token_scales: bool = False, *, round_intermediate: bool = True,
                  norm_weight: Optional[torch.Tensor] = None):
     """x [B, S, H*D] bfloat16 (a strided slice of a fused projection is fine) -> e4m3 [B, H, S, D]:
-    optional RMSNorm over the H*D row (norm_weight fp32 [H*D], no epsilon), optional RoPE (tables fp32 [B, S, H*D]), head split, optional D-point Hadamard transform times `scale`,
+    optional RMSNorm over the H*D row (norm_weight fp32 [H*D], no epsilon), optional RoPE (tables fp32 [B, S, H*D]; or the same values stored once, [S, H*D] for positions shared by the batch
+    and / or last dimension H*D/2 for one entry per rotated pair: functional.rope.compact_freqs_cis makes them), head split, optional D-point Hadamard transform times `scale`,
     then the direct e4m3 cast, or per-(token, head) absmax quantization when per_token_scales
     (returns (codes, scales [B, H, S]) in that case)."""
     x, b, s, d = _token_major(x, num_heads, "attn_prep_qk")
-    if (cos is None) != (sin is None):
-        raise RuntimeError("attn_prep_qk: cos and sin come together")
-    if cos is not None:
-        for t in (cos, sin):
-            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != x.numel():
-                raise RuntimeError("attn_prep_qk: tables must be float32 CUDA tensors of x's shape")
-        cos, sin = cos.contiguous(), sin.contiguous()
+    cos, sin, tflags = _rope_tables(cos, sin, b, s, num_heads * d, "attn_prep_qk")
     codes = torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty((b, num_heads, s), dtype=torch.float32, device=x.device) if per_token_scales else None
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().q8_attn_prep_qk(x.data_ptr(), x.stride(1), _ptr(_norm_w(norm_weight, x)), _ptr(cos), _ptr(sin),
                                               codes.data_ptr(),
-                                              _ptr(scales), b, s, num_heads, d, int(apply_fht), float(scale),
+                                              _ptr(scales), b, s, num_heads, d, int(apply_fht) | tflags, float(scale),
                                               Q8_BF16 if round_intermediate else Q8_F32, _stream(x)))
     return (codes, scales) if per_token_scales else codes
 
@@ -532,13 +552,7 @@ def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Opt
     k, bk, sk, dk = _token_major(k, num_heads, "attn_prep_qk_pair")
     if (bk, sk, dk) != (b, s, d):
         raise RuntimeError("attn_prep_qk_pair: q and k must have the same shape")
-    if (cos is None) != (sin is None):
-        raise RuntimeError("attn_prep_qk_pair: cos and sin come together")
-    if cos is not None:
-        for t in (cos, sin):
-            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != q.numel():
-                raise RuntimeError("attn_prep_qk_pair: tables must be float32 CUDA tensors of q's shape")
-        cos, sin = cos.contiguous(), sin.contiguous()
+    cos, sin, tflags = _rope_tables(cos, sin, b, s, num_heads * d, "attn_prep_qk_pair")
     mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=q.device)  # noqa: E731
     mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=q.device) if per_token_scales else None  # noqa: E731
     cq, ck, sq, sk_ = mk(), mk(), mks(), mks()
@@ -547,7 +561,7 @@ def attn_prep_qk_pair(q: torch.Tensor, k: torch.Tensor, num_heads: int, cos: Opt
                                                    _ptr(_norm_w(q_norm_weight, q)), _ptr(_norm_w(k_norm_weight, k)),
                                                    _ptr(cos), _ptr(sin),
                                                    cq.data_ptr(), _ptr(sq), ck.data_ptr(), _ptr(sk_), b, s, num_heads, d,
-                                                   int(apply_fht), float(scale),
+                                                   int(apply_fht) | tflags, float(scale),
                                                    Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))
     return ((cq, sq), (ck, sk_)) if per_token_scales else (cq, ck)
 
@@ -564,13 +578,7 @@ def attn_prep_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: 
     v, bv, sv, dv = _token_major(v, num_heads, "attn_prep_qkv")
     if (bk, sk, dk) != (b, s, d) or (bv, sv, dv) != (b, s, d):
         raise RuntimeError("attn_prep_qkv: q, k and v must have the same shape")
-    if (cos is None) != (sin is None):
-        raise RuntimeError("attn_prep_qkv: cos and sin come together")
-    if cos is not None:
-        for t in (cos, sin):
-            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != q.numel():
-                raise RuntimeError("attn_prep_qkv: tables must be float32 CUDA tensors of q's shape")
-        cos, sin = cos.contiguous(), sin.contiguous()
+    cos, sin, tflags = _rope_tables(cos, sin, b, s, num_heads * d, "attn_prep_qkv")
     mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=q.device)  # noqa: E731
     mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=q.device) if per_token_scales else None  # noqa: E731
     cq, ck, cv, sq, sk_, sv_ = mk(), mk(), mk(), mks(), mks(), mks()
@@ -578,7 +586,7 @@ def attn_prep_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: 
         _lib.check(_lib.lib().q8_attn_prep_qkv(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), v.data_ptr(), v.stride(1),
                                                _ptr(_norm_w(q_norm_weight, q)), _ptr(_norm_w(k_norm_weight, k)),
                                                _ptr(cos), _ptr(sin), cq.data_ptr(), _ptr(sq), ck.data_ptr(), _ptr(sk_),
-                                               cv.data_ptr(), _ptr(sv_), b, s, num_heads, d, int(apply_fht), float(scale),
+                                               cv.data_ptr(), _ptr(sv_), b, s, num_heads, d, int(apply_fht) | tflags, float(scale),
                                                Q8_BF16 if round_intermediate else Q8_F32, _stream(q)))
     return ((cq, sq), (ck, sk_), (cv, sv_)) if per_token_scales else (cq, ck, cv)
 
@@ -594,13 +602,7 @@ def attn_prep_kv(k: torch.Tensor, v: torch.Tensor, num_heads: int, cos: Optional
     v, bv, sv, dv = _token_major(v, num_heads, "attn_prep_kv")
     if (bv, sv, dv) != (b, s, d):
         raise RuntimeError("attn_prep_kv: k and v must have the same shape")
-    if (cos is None) != (sin is None):
-        raise RuntimeError("attn_prep_kv: cos and sin come together")
-    if cos is not None:
-        for t in (cos, sin):
-            if t.dtype != torch.float32 or not t.is_cuda or t.numel() != k.numel():
-                raise RuntimeError("attn_prep_kv: tables must be float32 CUDA tensors of k's shape")
-        cos, sin = cos.contiguous(), sin.contiguous()
+    cos, sin, tflags = _rope_tables(cos, sin, b, s, num_heads * d, "attn_prep_kv")
     mk = lambda: torch.empty((b, num_heads, s, d), dtype=torch.float8_e4m3fn, device=k.device)  # noqa: E731
     mks = lambda: torch.empty((b, num_heads, s), dtype=torch.float32, device=k.device) if per_token_scales else None  # noqa: E731
     ck, cv, sk_, sv_ = mk(), mk(), mks(), mks()
@@ -608,7 +610,7 @@ def attn_prep_kv(k: torch.Tensor, v: torch.Tensor, num_heads: int, cos: Optional
     with torch.cuda.device(k.device):
         _lib.check(_lib.lib().q8_attn_prep_kv(k.data_ptr(), k.stride(1), v.data_ptr(), v.stride(1), _ptr(nw), _ptr(cos), _ptr(sin),
                                               ck.data_ptr(), _ptr(sk_), cv.data_ptr(), _ptr(sv_), b, s, num_heads, d,
-                                              int(apply_fht), float(scale), Q8_BF16 if round_intermediate else Q8_F32, _stream(k)))
+                                              int(apply_fht) | tflags, float(scale), Q8_BF16 if round_intermediate else Q8_F32, _stream(k)))
     return ((ck, sk_), (cv, sv_)) if per_token_scales else (ck, cv)
 
 

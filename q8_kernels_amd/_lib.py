@@ -14,6 +14,7 @@ Q8_I8, Q8_E4M3, Q8_BF16, Q8_F16, Q8_F32 = 0, 1, 2, 3, 4
 Q8_QUANT_RNE, Q8_QUANT_SCALE_DIV = 1, 2
 Q8_V_DS, Q8_V_SD = 0, 1
 Q8_ATTN_SUM_ROUNDED_P, Q8_ATTN_P_UNIT_RANGE, Q8_ATTN_O_TOKEN_MAJOR, Q8_ATTN_LAZY_MAX = 1, 2, 4, 8
+Q8_PREP_FHT, Q8_PREP_PAIR_TABLES, Q8_PREP_SHARED_TABLES = 1, 2, 4
 # values of q8_gemm_last_kernel (tests)
 Q8_GEMM_KERNEL_PIPE256, Q8_GEMM_KERNEL_TILE128, Q8_GEMM_KERNEL_TILE64 = 1, 2, 3
 Q8_GEMM_KERNEL_PERSIST256, Q8_GEMM_KERNEL_PERSIST192, Q8_GEMM_KERNEL_RESIDUAL = 4, 5, 16

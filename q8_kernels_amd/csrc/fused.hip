@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
                                                               uint8_t* __restrict__ codes2, float* __restrict__ scales2,
                                                               const uint16_t* __restrict__ xv, int64_t xv_row_stride,
                                                               uint8_t* __restrict__ codes_v, float* __restrict__ scales_v,
-                                                              int64_t tokens, int S, int apply_fht, float scale,
+                                                              int64_t tokens, int S, int flags, float scale,
                                                               int mid_bf16) {
     static_assert(LH <= LANES, "a head may not span tokens");
     constexpr int DIM = LANES * CH * 8, D = LH * 8, H = DIM / D, NT = PAIR ? 2 : 1;
@@ -246,13 +246,12 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
         }
     }
     if (cs != nullptr) {
-        // interleaved pairs with per-element tables (csrc/ops/rope_cuda.cu:99-103)
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int64_t e = tok * DIM + (c * LANES + t) * 8;
-            float cv[8], sv[8];
-            load8<Q8_F32>(cs, e, cv);
-            load8<Q8_F32>(sn, e, sv);
+        // interleaved pairs (csrc/ops/rope_cuda.cu:99-103). The tables hold one entry per element, [rows, DIM], or with
+        // Q8_PREP_PAIR_TABLES one per rotated pair, [rows, DIM / 2] (tables built by repeating every frequency twice,
+        // q8_kernels/models/LTXVideo.py:95-148, carry each value twice); rows = the tokens, or with
+        // Q8_PREP_SHARED_TABLES the S positions of one batch element, which then serve every batch element.
+        const int64_t trow = (flags & Q8_PREP_SHARED_TABLES) ? s : tok;
+        auto rotate = [&](int c, const float (&cv)[8], const float (&sv)[8]) {
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 float o[8];
@@ -265,6 +264,31 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[n][c][i] = o[i];
             }
+        };
+        if (flags & Q8_PREP_PAIR_TABLES) {
+            v4f hc[CH], hs[CH];  // requested together: half the bytes, and one trip to memory for all chunks
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int64_t e = trow * (DIM / 2) + (c * LANES + t) * 4;
+                hc[c] = *reinterpret_cast<const v4f*>(cs + e);
+                hs[c] = *reinterpret_cast<const v4f*>(sn + e);
+            }
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                float cv[8], sv[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { cv[i] = hc[c][i >> 1]; sv[i] = hs[c][i >> 1]; }
+                rotate(c, cv, sv);
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int64_t e = trow * DIM + (c * LANES + t) * 8;
+                float cv[8], sv[8];
+                load8<Q8_F32>(cs, e, cv);
+                load8<Q8_F32>(sn, e, sv);
+                rotate(c, cv, sv);
+            }
         }
     }
 #pragma unroll
@@ -273,7 +297,7 @@ __global__ __launch_bounds__(kBlock) void attn_prep_qk_kernel(const uint16_t* __
         float* const sout = n == 0 ? scales : scales2;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            if (apply_fht) {
+            if (flags & Q8_PREP_FHT) {
                 fht_head<LH>(v[n][c], t, scale);
             }
             const int h = (c * LANES + t) / LH;
@@ -484,7 +508,7 @@ extern "C" int q8_norm_mod_fht_quant_rows(const void* x, const float* norm_w, in
 static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_stride, const void* x2, int64_t x2_row_stride,
                              const float* norm_w, const float* norm_w2, const float* cos_t, const float* sin_t, void* codes, float* scales, void* codes2,
                              float* scales2, const void* xv, int64_t xv_row_stride, void* codes_v, float* scales_v, int B, int S,
-                             int H, int D, int apply_fht, float scale, int mid_dtype, hipStream_t stream) {
+                             int H, int D, int flags, float scale, int mid_dtype, hipStream_t stream) {
     const bool pair = x2 != nullptr;
     if (B < 0 || S < 0 || H <= 0) return fail(Q8_ERR_SHAPE, "%s: B %d S %d H %d", who, B, S, H);
     if (D != 64 && D != 128) return fail(Q8_ERR_SHAPE, "%s: head dim %d (want 64 or 128)", who, D);
@@ -495,6 +519,9 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
     if ((int64_t)B * S == 0) return Q8_OK;
     if (!x || !codes || (pair && !codes2)) return fail(Q8_ERR_NULL, "%s: null pointer", who);
     if ((cos_t == nullptr) != (sin_t == nullptr)) return fail(Q8_ERR_NULL, "%s: cos and sin come together", who);
+    if (flags & ~(Q8_PREP_FHT | Q8_PREP_PAIR_TABLES | Q8_PREP_SHARED_TABLES)) return fail(Q8_ERR_FLAGS, "%s: unknown flag bits 0x%x", who, flags);
+    if (!cos_t && (flags & (Q8_PREP_PAIR_TABLES | Q8_PREP_SHARED_TABLES)))
+        return fail(Q8_ERR_FLAGS, "%s: table flags 0x%x without tables", who, flags);
     if (pair && ((scales == nullptr) != (scales2 == nullptr))) return fail(Q8_ERR_NULL, "%s: both scale outputs or none", who);
     if (x_row_stride < dim || x_row_stride % 8 != 0 || (pair && (x2_row_stride < dim || x2_row_stride % 8 != 0)))
         return fail(Q8_ERR_SHAPE, "%s: row stride %lld / %lld", who, (long long)x_row_stride, (long long)x2_row_stride);
@@ -519,7 +546,7 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
     static_cast<const uint16_t*>(x), x_row_stride, static_cast<const uint16_t*>(x2), x2_row_stride, norm_w, norm_w2,     \
         cos_t, sin_t,                                                                                                    \
         static_cast<uint8_t*>(codes), scales, static_cast<uint8_t*>(codes2), scales2,                                    \
-        static_cast<const uint16_t*>(xv), xv_row_stride, static_cast<uint8_t*>(codes_v), scales_v, tokens, S, apply_fht, \
+        static_cast<const uint16_t*>(xv), xv_row_stride, static_cast<uint8_t*>(codes_v), scales_v, tokens, S, flags, \
         scale, mid_dtype == Q8_BF16 ? 1 : 0
 #define PREP_LAUNCH(LANES, CH, LH)                                                                                       \
     if (pair) hipLaunchKernelGGL((attn_prep_qk_kernel<LANES, CH, LH, true>), dim3((unsigned)grid), dim3(kBlock), 0, stream, PREP_ARGS); \
@@ -546,41 +573,41 @@ static int attn_prep_qk_impl(const char* who, const void* x, int64_t x_row_strid
 }
 
 extern "C" int q8_attn_prep_qk(const void* x, int64_t x_row_stride, const float* norm_w, const float* cos_t,
-                               const float* sin_t, void* codes, float* scales, int B, int S, int H, int D, int apply_fht,
+                               const float* sin_t, void* codes, float* scales, int B, int S, int H, int D, int flags,
                                float scale, int mid_dtype, q8_stream_t stream_) {
     return attn_prep_qk_impl("q8_attn_prep_qk", x, x_row_stride, nullptr, 0, norm_w, nullptr, cos_t, sin_t, codes, scales, nullptr,
-                             nullptr, nullptr, 0, nullptr, nullptr, B, S, H, D, apply_fht, scale, mid_dtype,
+                             nullptr, nullptr, 0, nullptr, nullptr, B, S, H, D, flags, scale, mid_dtype,
                              static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_qk_pair(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride,
                                     const float* norm_wq, const float* norm_wk, const float* cos_t, const float* sin_t,
                                     void* codes_q, float* scales_q, void* codes_k, float* scales_k, int B, int S, int H,
-                                    int D, int apply_fht, float scale, int mid_dtype, q8_stream_t stream_) {
+                                    int D, int flags, float scale, int mid_dtype, q8_stream_t stream_) {
     if (!xk) return fail(Q8_ERR_NULL, "q8_attn_prep_qk_pair: null pointer");
     return attn_prep_qk_impl("q8_attn_prep_qk_pair", xq, xq_row_stride, xk, xk_row_stride, norm_wq, norm_wk, cos_t, sin_t, codes_q, scales_q,
-                             codes_k, scales_k, nullptr, 0, nullptr, nullptr, B, S, H, D, apply_fht, scale, mid_dtype,
+                             codes_k, scales_k, nullptr, 0, nullptr, nullptr, B, S, H, D, flags, scale, mid_dtype,
                              static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_qkv(const void* xq, int64_t xq_row_stride, const void* xk, int64_t xk_row_stride, const void* xv,
                                 int64_t xv_row_stride, const float* norm_wq, const float* norm_wk, const float* cos_t,
                                 const float* sin_t, void* codes_q, float* scales_q, void* codes_k, float* scales_k,
-                                void* codes_v, float* scales_v, int B, int S, int H, int D, int apply_fht, float scale,
+                                void* codes_v, float* scales_v, int B, int S, int H, int D, int flags, float scale,
                                 int mid_dtype, q8_stream_t stream_) {
     if (!xk || !xv) return fail(Q8_ERR_NULL, "q8_attn_prep_qkv: null pointer");
     return attn_prep_qk_impl("q8_attn_prep_qkv", xq, xq_row_stride, xk, xk_row_stride, norm_wq, norm_wk, cos_t, sin_t, codes_q, scales_q,
-                             codes_k, scales_k, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, apply_fht, scale, mid_dtype,
+                             codes_k, scales_k, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, flags, scale, mid_dtype,
                              static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int q8_attn_prep_kv(const void* xk, int64_t xk_row_stride, const void* xv, int64_t xv_row_stride, const float* norm_wk,
                                const float* cos_t, const float* sin_t, void* codes_k, float* scales_k, void* codes_v,
-                               float* scales_v, int B, int S, int H, int D, int apply_fht, float scale, int mid_dtype,
+                               float* scales_v, int B, int S, int H, int D, int flags, float scale, int mid_dtype,
                                q8_stream_t stream_) {
     if (!xv) return fail(Q8_ERR_NULL, "q8_attn_prep_kv: null pointer");
     return attn_prep_qk_impl("q8_attn_prep_kv", xk, xk_row_stride, nullptr, 0, norm_wk, nullptr, cos_t, sin_t, codes_k, scales_k, nullptr,
-                             nullptr, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, apply_fht, scale, mid_dtype,
+                             nullptr, xv, xv_row_stride, codes_v, scales_v, B, S, H, D, flags, scale, mid_dtype,
                              static_cast<hipStream_t>(stream_));
 }
 

@@ -14,6 +14,7 @@ from typing import Optional, Tuple
 import torch
 
 from .. import _C
+from . import rope as _rope
 
 _FP8 = torch.float8_e4m3fn
 
@@ -65,14 +66,16 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
     projection's GEMM wrote itself (_C.mm_bias_qkv); the prologue then handles q and k only.
 
     q_norm_weight / k_norm_weight (fp32 [H*64]) apply the qk-RMSNorm (over all heads of a token, no epsilon) first;
-    freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape).
+    freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape); they go
+    through rope.compact_freqs_cis, or may be given in one of its compact forms.
     Without per_token_scales the operands are cast to e4m3 exactly as flash_attn_func does; with it each
     (token, head) row of q, k and v gets its own absmax scale. p_unit_range as in flash_attn_func (the reference's
     probability grid)."""
     d = q.shape[-1] // num_heads
     if softmax_scale is None:
         softmax_scale = d ** (-0.5)
-    cos, sin = (None, None) if freqs_cis is None else freqs_cis
+    # the tables with their repeated values stored once (same bits, a quarter of the bytes when both properties hold)
+    cos, sin = (None, None) if freqs_cis is None else _rope.compact_freqs_cis(*freqs_cis)
     if apply_qk_hadamard:
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:

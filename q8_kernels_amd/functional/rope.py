@@ -78,3 +78,47 @@ def precompute_freqs_cis(indices_grid: torch.Tensor, dim: int, theta: float = 10
     cos[:, :, lead:] = ang.cos().repeat_interleave(2, dim=-1)
     sin[:, :, lead:] = ang.sin().repeat_interleave(2, dim=-1)
     return cos, sin
+
+
+# compact_freqs_cis: the most recent results, [(key, (cos, sin) as given, (cos, sin) compact)]
+_COMPACT_CACHE = []
+compact_tables = True  # False: the fused attention prologues read the tables as they are given
+
+
+def clear_compact_freqs_cache():
+    """Drops the compact tables kept by compact_freqs_cis, and its references to the tables they were made from."""
+    del _COMPACT_CACHE[:]
+
+
+def compact_freqs_cis(cos: torch.Tensor, sin: torch.Tensor, keep: int = 2):
+    """(cos, sin) float32 [B, T, dim] -> the same values stored once, for the fused attention prologues
+    (_C.attn_prep_qk and its siblings), which then read a quarter of the table bytes and give the same bits:
+
+      * tables whose two entries of every rotated pair are equal (precompute_freqs_cis repeats every angle twice, like
+        q8_kernels/models/LTXVideo.py:95-148) become [.., dim / 2], one entry per pair;
+      * tables that are the same for every batch element (one position grid for the whole batch) become [1, T, ..].
+
+    Whether a table has these properties is read off its values (two comparisons over the tables, with a device
+    synchronisation), once: the result is kept for the last `keep` table pairs, keyed by their storage, shape and
+    version counter, together with a reference to the tables themselves, so that the storage cannot be handed to
+    another tensor while the entry lives (clear_compact_freqs_cache drops both). In-place changes through torch bump the
+    version counter and are seen; writes that bypass it are not. Tables that have neither property, that require a
+    gradient, or that are first met while a graph is being captured (no synchronisation allowed) come back unchanged."""
+    if (not compact_tables or cos.dim() != 3 or cos.shape != sin.shape or not cos.is_cuda or not sin.is_cuda
+            or cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.requires_grad or sin.requires_grad):
+        return cos, sin
+    key = (cos.data_ptr(), cos._version, sin.data_ptr(), sin._version, tuple(cos.shape), cos.stride(), sin.stride())
+    for k, _, res in _COMPACT_CACHE:
+        if k == key:
+            return res
+    if torch.cuda.is_current_stream_capturing():
+        return cos, sin
+    c, s = cos, sin
+    if c.shape[-1] % 2 == 0 and torch.equal(c[..., 0::2], c[..., 1::2]) and torch.equal(s[..., 0::2], s[..., 1::2]):
+        c, s = c[..., 0::2], s[..., 0::2]
+    if c.shape[0] > 1 and bool((c == c[:1]).all()) and bool((s == s[:1]).all()):
+        c, s = c[:1], s[:1]
+    res = (cos, sin) if c is cos else (c.contiguous(), s.contiguous())
+    _COMPACT_CACHE.insert(0, (key, (cos, sin), res))
+    del _COMPACT_CACHE[max(1, keep):]
+    return res

@@ -34,6 +34,7 @@ def test_header_enums_match_python_constants():
     text = open(HEADER).read()
     for name in ("Q8_I8", "Q8_E4M3", "Q8_BF16", "Q8_F16", "Q8_F32", "Q8_QUANT_RNE", "Q8_QUANT_SCALE_DIV",
                  "Q8_V_DS", "Q8_V_SD", "Q8_ATTN_SUM_ROUNDED_P", "Q8_ATTN_P_UNIT_RANGE", "Q8_ATTN_O_TOKEN_MAJOR", "Q8_ATTN_LAZY_MAX",
+                 "Q8_PREP_FHT", "Q8_PREP_PAIR_TABLES", "Q8_PREP_SHARED_TABLES",
                  "Q8_GEMM_KERNEL_PIPE256", "Q8_GEMM_KERNEL_TILE128", "Q8_GEMM_KERNEL_TILE64", "Q8_GEMM_KERNEL_PERSIST256",
                  "Q8_GEMM_KERNEL_PERSIST192", "Q8_GEMM_KERNEL_RESIDUAL"):
         m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
@@ -99,6 +100,10 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     assert L.q8_attn_prep_qk(16, 512, None, None, None, 16, None, 1, 5, 12, 64, 1, 1.0, B16, None) == -3   # H * D = 768
     assert L.q8_attn_prep_qk(16, 500, None, None, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -3    # stride < H * D
     assert L.q8_attn_prep_qk(16, 512, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1      # cos without sin
+    assert L.q8_attn_prep_qk(16, 512, None, 16, 16, 16, None, 1, 5, 8, 64, 8, 1.0, B16, None) == -6        # unknown flag bit
+    assert L.q8_attn_prep_qk(16, 512, None, None, None, 16, None, 1, 5, 8, 64, 1 | _lib.Q8_PREP_PAIR_TABLES, 1.0, B16, None) == -6  # table flag, no tables
+    assert L.q8_attn_prep_qk_pair(16, 512, 16, 512, None, None, None, None, 16, None, 16, None, 1, 5, 8, 64,
+                                  _lib.Q8_PREP_SHARED_TABLES, 1.0, B16, None) == -6
     assert L.q8_attn_prep_qk_pair(16, 512, None, 512, None, None, None, None, 16, None, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
     assert L.q8_attn_prep_qk_pair(16, 512, 16, 512, None, None, None, None, 16, 16, 16, None, 1, 5, 8, 64, 1, 1.0, B16, None) == -1
     # q8_attn_prep_qkv(xq, sq, xk, sk, xv, sv, nwq, nwk, cos, sin, cq, scq, ck, sck, cv, scv, B, S, H, D, fht, scale, mid, stream)

@@ -197,6 +197,84 @@ def test_attn_prep_qk(dev, shape, rope, fht, scaled):
         assert_bit_equal(got, want, "codes")
 
 
+def _pair_tables(b, s, dim, g, shared):
+    """tables in the layout the LTX transformer builds (every angle twice); shared: one grid for the whole batch"""
+    ang = torch.rand(1 if shared else b, s, dim // 2, generator=g) * 6.28
+    cos, sin = torch.cos(ang).repeat_interleave(2, -1), torch.sin(ang).repeat_interleave(2, -1)
+    return cos.expand(b, -1, -1).contiguous(), sin.expand(b, -1, -1).contiguous()
+
+
+@pytest.mark.parametrize("shape", [(2, 70, 8, 64), (3, 33, 32, 64), (2, 19, 8, 128), (1, 9, 24, 64), (2, 5, 1, 64), (2, 130, 64, 64)])
+@pytest.mark.parametrize("form", ["pairs", "shared", "pairs+shared"])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_attn_prep_compact_tables_give_the_bits_of_full_tables(dev, shape, form, scaled):
+    """The rotation tables with their repeated values stored once ([.., H*D/2]: one entry per rotated pair; [1, S, ..]: one
+    position grid for all batch elements) through all four prologues, with the qk-norm in front: bit-equal to the full
+    [B, S, H*D] tables, which test_attn_prep_qk checks against the oracle."""
+    b, s, h, d = shape
+    dim = h * d
+    g = torch.Generator().manual_seed(b * 1000 + s + dim)
+    q, k, v = ((torch.randn(b, s, dim, generator=g) * 1.5).to(BF16).to(dev) for _ in range(3))
+    wq, wk = (1 + 0.1 * torch.randn(dim, generator=g)).to(dev), (1 + 0.1 * torch.randn(dim, generator=g)).to(dev)
+    cos, sin = _pair_tables(b, s, dim, g, "shared" in form)
+    cc, sc = cos, sin
+    if "pairs" in form:
+        cc, sc = cc[..., 0::2], sc[..., 0::2]
+    if "shared" in form:
+        cc, sc = cc[:1], sc[:1]
+    full, comp = (cos.to(dev), sin.to(dev)), (cc.contiguous().to(dev), sc.contiguous().to(dev))
+    scale = (d ** -0.5) * (0.125 ** 0.5)
+    flat = lambda r: [t for part in (r if isinstance(r, (tuple, list)) else (r,)) for t in (part if isinstance(part, (tuple, list)) else (part,))]  # noqa: E731
+    calls = [lambda t: _C().attn_prep_qk(q, h, t[0], t[1], True, scale, scaled, norm_weight=wq),
+             lambda t: _C().attn_prep_qk_pair(q, k, h, t[0], t[1], True, scale, scaled, q_norm_weight=wq, k_norm_weight=wk),
+             lambda t: _C().attn_prep_kv(k, v, h, t[0], t[1], False, 1.0, scaled)]
+    if d == 64:
+        calls.append(lambda t: _C().attn_prep_qkv(q, k, v, h, t[0], t[1], True, scale, scaled))
+    for i, call in enumerate(calls):
+        for a, c in zip(flat(call(full)), flat(call(comp))):
+            assert_bit_equal(c, a, "%s call %d" % (form, i))
+
+
+def test_compact_freqs_cis_detects_caches_and_follows_changes(dev):
+    """compact_freqs_cis on the tables precompute_freqs_cis builds (both properties), on tables with one property or none,
+    the cache (same objects back, dropped by clear_compact_freqs_cache), an in-place change of the tables, and the
+    fused attention path with and without it: same bits."""
+    from q8_kernels_amd.functional import fused as FU, rope as R
+    R.clear_compact_freqs_cache()
+    cos, sin = R.precompute_freqs_cis(R.video_index_grid(3, 4, 5, batch=2, device=dev), 512)
+    c, s = R.compact_freqs_cis(cos, sin)
+    assert c.shape == (1, 60, 256) and s.shape == (1, 60, 256)
+    assert torch.equal(c[0].repeat_interleave(2, -1), cos[1]) and torch.equal(s[0].repeat_interleave(2, -1), sin[0])
+    c2, s2 = R.compact_freqs_cis(cos, sin)
+    assert c2 is c and s2 is s                     # from the cache
+    g = torch.Generator().manual_seed(3)
+    q, k, v = ((torch.randn(2, 60, 512, generator=g)).to(BF16).to(dev) for _ in range(3))
+    on = FU.flash_attn_token_major(q, k, v, 8, None, None, True, (cos, sin), BF16)
+    R.compact_tables = False
+    try:
+        assert R.compact_freqs_cis(cos, sin)[0] is cos
+        off = FU.flash_attn_token_major(q, k, v, 8, None, None, True, (cos, sin), BF16)
+    finally:
+        R.compact_tables = True
+    assert_bit_equal(on, off, "fused attention with compact tables")
+    # one batch element moved: no longer shared, still one entry per pair; seen through the version counter
+    cos[1, 7] = cos[1, 8]
+    sin[1, 7] = sin[1, 8]
+    c3, s3 = R.compact_freqs_cis(cos, sin)
+    assert c3.shape == (2, 60, 256) and torch.equal(c3.repeat_interleave(2, -1), cos)
+    assert_bit_equal(FU.flash_attn_token_major(q, k, v, 8, None, None, True, (cos, sin), BF16),
+                     FU.flash_attn_token_major(q, k, v, 8, None, None, True, (c3.repeat_interleave(2, -1), s3.repeat_interleave(2, -1)), BF16),
+                     "after the change")
+    # pairs differ: only the batch property is left; neither: the tables themselves
+    cb, sb = torch.randn(1, 60, 512, device=dev).expand(2, -1, -1).contiguous(), torch.randn(1, 60, 512, device=dev).expand(2, -1, -1).contiguous()
+    assert R.compact_freqs_cis(cb, sb)[0].shape == (1, 60, 512)
+    cn, sn = torch.randn(2, 60, 512, device=dev), torch.randn(2, 60, 512, device=dev)
+    assert R.compact_freqs_cis(cn, sn)[0] is cn
+    assert len(R._COMPACT_CACHE) == 2              # the last two table pairs
+    R.clear_compact_freqs_cache()
+    assert R._COMPACT_CACHE == []
+
+
 @pytest.mark.parametrize("shape", [(2, 70, 8, 64), (1, 33, 32, 64), (2, 7, 2, 128)])
 @pytest.mark.parametrize("rope", [False, True])
 @pytest.mark.parametrize("scaled", [False, True])
