@@ -296,9 +296,13 @@ int q8_gemm_gated_residual(const void* A, const void* B, const float* bias, cons
  * q8_kernels/modules/attention.py:67-105). M rows = batch elements of `tokens` tokens each. Runs on the persistent kernel
  * only: N % 8 == 0, K % 128 == 0, K > 256; v_col0 a multiple of 256, N - v_col0 a multiple of 64 (Q8_ERR_SHAPE otherwise).
  * v_col0 == 0 is a V projection of its own (a separate to_v layer): every column goes to v_codes, C may be NULL.
+ * v_fht_scale != 0: the bf16-rounded results of every head of 64 go through the 64-point Hadamard transform times
+ * v_fht_scale before the cast, hadamard_transform(x, scale, out_type=e4m3) of q8_kernels/functional/flash_attention.py:47-51:
+ * with v_col0 == 0 the Q (or K) operand of an attention with apply_qk_hadamard straight from its projection, the bits of
+ * q8_gemm followed by q8_attn_prep_qk without tables. 0 = the plain cast. Finite and not negative.
  */
 int q8_gemm_qkv(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C, void* v_codes,
-                int M, int N, int K, int v_col0, int tokens, int in_dtype, q8_stream_t stream);
+                int M, int N, int K, int v_col0, int tokens, float v_fht_scale, int in_dtype, q8_stream_t stream);
 
 /*
  * Kernel override for q8_gemm / q8_gemm_i32: 0 = choose by problem size (default), 1 = pipelined 256x256 tiles with

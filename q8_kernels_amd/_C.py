@@ -264,12 +264,15 @@ def fp8_mm_bias(a, b, bias, a_scales, b_scales, fuse_gelu: bool, out_type: Optio
     return _mm(a, b, bias, a_scales, b_scales, fuse_gelu, out_type, torch.float8_e4m3fn, "fp8_mm_bias", residual, gate)
 
 
-def mm_bias_qkv(a, b, bias, a_scales, b_scales, tokens: int, v_col0: int):
+def mm_bias_qkv(a, b, bias, a_scales, b_scales, tokens: int, v_col0: int, fht_scale: float = 0.0):
     """The GEMM of a fused QKV projection with the cast of V in its epilogue: a [B*S, K] codes (int8 or e4m3, rows of B
     batch elements of `tokens` tokens), b [N, K], fp32 bias [N] or None, fp32 row / column scales. Returns (qk, v_codes):
     qk bfloat16 [B, S, v_col0] (the Q and K columns as q8_mm_bias / fp8_mm_bias give them) and v_codes e4m3
     [B, (N - v_col0) / 64, S, 64], the bf16-rounded V columns cast to e4m3 token-major per head, what attn_prep_qkv
-    produces from the bfloat16 projection and flash_attention takes with v_token_major=True."""
+    produces from the bfloat16 projection and flash_attention takes with v_token_major=True.
+    fht_scale != 0: every head of the v_codes columns goes through the 64-point Hadamard transform times fht_scale
+    before the cast, what attn_prep_qk(x, heads, None, None, True, fht_scale) makes of the bfloat16 projection: with
+    v_col0 == 0 the query (or key) operand of an attention with apply_qk_hadamard straight from its projection."""
     _check_input(a, "a")
     _check_input(b, "b")
     if a.dtype != b.dtype or a.dtype not in (torch.int8, torch.float8_e4m3fn) or a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
@@ -296,7 +299,7 @@ def mm_bias_qkv(a, b, bias, a_scales, b_scales, tokens: int, v_col0: int):
     with torch.cuda.device(a.device):
         _lib.check(_lib.lib().q8_gemm_qkv(a.data_ptr(), b.data_ptr(), _ptr(bias), a_scales.data_ptr(), b_scales.data_ptr(),
                                           qk.data_ptr() if v_col0 else None, vc.data_ptr(), m, n, k, v_col0, tokens,
-                                          Q8_I8 if a.dtype == torch.int8 else Q8_E4M3, _stream(a)))
+                                          float(fht_scale), Q8_I8 if a.dtype == torch.int8 else Q8_E4M3, _stream(a)))
     return qk, vc
 
 

@@ -48,7 +48,7 @@ SIGNATURES = {
     "q8_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "q8_gemm_residual": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "q8_gemm_gated_residual": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i, _i, _i, _i, _i, _vp]),
-    "q8_gemm_qkv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "q8_gemm_qkv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "q8_gemm_i32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "q8_gemm_set_config": (_i, [_i]),
     "q8_attn_set_config": (_i, [_i]),

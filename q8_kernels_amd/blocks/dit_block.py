@@ -21,6 +21,10 @@ class Fp8DiTBlock(nn.Module):
     # True (default): RMSNorm + quantizer, the attention prologues and the residual additions run fused into their
     # neighbours; False: one operator per step of the docstring's sequence. Both give the same bits.
     fuse = True
+    # True (default): the cross-attention's queries leave their projection's GEMM as the attention kernel's e4m3 operand
+    # (Hadamard transform per head and cast in the epilogue); False: the projection is written as bfloat16 and the
+    # attention prologue reads it back. Same bits.
+    fuse_query_epilogue = True
 
     def __init__(self, dim: int = 2048, num_heads: int = 32, head_dim: int = 64, ffn_dim: int = 8192,
                  text_dim: int = 2048, device=None):
@@ -96,11 +100,20 @@ class Fp8DiTBlock(nn.Module):
                                                  apply_qk_hadamard=True, freqs_cis=freqs_cis, out_dtype=bf16)
         hidden = self._lin(self.to_out, a, residual=hidden)
         # cross-attention to the text states
-        q2 = self._norm_lin(self.norm2, self.to_q2, hidden)
         kv2 = self._lin(self.to_kv2, text)  # k and v are read in place, like q, k, v of the self-attention
         k2, v2 = kv2[..., :d], kv2[..., d:]
-        a = Q8F.fused.flash_attn_token_major(q2, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
-                                             out_dtype=bf16)
+        if self.fuse_query_epilogue and self.head_dim == 64 and d > 256 and d % 128 == 0:
+            # the queries leave their projection's GEMM as the attention kernel's operand: Hadamard transform per head and
+            # e4m3 cast in the epilogue (no rotation and no norm lies between the projection and the attention here)
+            codes, scales = Q8F.fused.rms_norm_quantize(hidden, self.norm2.weight, torch.float8_e4m3fn)
+            _, q_codes = _C.mm_bias_qkv(codes.reshape(-1, d), self.to_q2.weight.data, self.to_q2.bias.data, scales.reshape(-1),
+                                        self.to_q2.scales, hidden.shape[1], 0, Q8F.fused.qk_hadamard_scale(self.head_dim))
+            a = Q8F.fused.flash_attn_token_major(None, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
+                                                 out_dtype=bf16, q_codes=q_codes)
+        else:
+            q2 = self._norm_lin(self.norm2, self.to_q2, hidden)
+            a = Q8F.fused.flash_attn_token_major(q2, k2, v2, h, batch_mask=text_lens, apply_qk_hadamard=True,
+                                                 out_dtype=bf16)
         hidden = self._lin(self.to_out2, a, residual=hidden)
         # feed-forward
         up = self._norm_lin(self.norm3, self.ff_up, hidden, fuse_gelu=True)

@@ -276,7 +276,7 @@ static int persist_cus() {
     return cus;
 }
 
-template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT, bool VSPLIT = false>
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT, int VSPLIT = 0>
 static int launch_persist_mt(const GemmParams& p, hipStream_t stream) {
     constexpr int BM = 64 * MT;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + kPipeBN - 1) / kPipeBN;
@@ -301,15 +301,18 @@ static int launch_persist(const GemmParams& p, hipStream_t stream) {
     const long tn = (p.N + kPipeBN - 1) / kPipeBN, cus = persist_cus();
     // (with a residual the 256-row kernel is 256 registers short by a dozen: it spills copy offsets around its epilogue
     //  and runs 10-15 % slower than its tile count says, measured; the 192-row kernel does not)
-    const double cost256 = (!E4M3OUT && p.residual != nullptr) ? 1.25 : 1.0;
+    //  (the same holds for the Hadamard form of the head-major epilogue)
+    const double cost256 = (!E4M3OUT && (p.residual != nullptr || (p.v_codes != nullptr && p.v_fht_scale != 0.f))) ? 1.25 : 1.0;
     auto cost = [&](int bm) {
         const long tiles = (long)((p.M + bm - 1) / bm) * tn * batch;
         return (double)((tiles + cus - 1) / cus) * bm * (bm == 256 ? cost256 : 1.2);
     };
     const bool small = g_persist_mt == 3 || (g_persist_mt == 0 && cost(192) < cost(256));
     if constexpr (!E4M3OUT && !GELU) {
+        if (p.v_codes != nullptr && p.v_fht_scale != 0.f)
+            return small ? launch_persist_mt<IN, false, 3, false, false, 2>(p, stream) : launch_persist_mt<IN, false, 4, false, false, 2>(p, stream);
         if (p.v_codes != nullptr)
-            return small ? launch_persist_mt<IN, false, 3, false, false, true>(p, stream) : launch_persist_mt<IN, false, 4, false, false, true>(p, stream);
+            return small ? launch_persist_mt<IN, false, 3, false, false, 1>(p, stream) : launch_persist_mt<IN, false, 4, false, false, 1>(p, stream);
     }
     if constexpr (!E4M3OUT) {
         if (p.residual != nullptr)
@@ -412,7 +415,7 @@ extern "C" int q8_gemm_residual(const void* A, const void* B, const float* bias,
 }
 
 extern "C" int q8_gemm_qkv(const void* A, const void* B, const float* bias, const float* sa, const float* sb, void* C, void* v_codes,
-                           int M, int N, int K, int v_col0, int tokens, int in_dtype, q8_stream_t stream_) {
+                           int M, int N, int K, int v_col0, int tokens, float v_fht_scale, int in_dtype, q8_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "q8_gemm_qkv";
     if (gemm_output_is_empty(1, 1, M, N, K)) return Q8_OK;
@@ -426,8 +429,10 @@ extern "C" int q8_gemm_qkv(const void* A, const void* B, const float* bias, cons
     if (v_col0 < 0 || v_col0 >= N || v_col0 % 256 != 0 || (N - v_col0) % 64 != 0)
         return fail(Q8_ERR_SHAPE, "%s: v_col0 = %d must be a multiple of 256 below N = %d with N - v_col0 a multiple of 64", who, v_col0, N);
     if (tokens <= 0 || M % tokens != 0) return fail(Q8_ERR_SHAPE, "%s: M = %d must be a multiple of tokens = %d", who, M, tokens);
+    if (!(v_fht_scale >= 0.f) || v_fht_scale > 3.0e38f) return fail(Q8_ERR_SHAPE, "%s: v_fht_scale = %g must be finite and not negative", who, (double)v_fht_scale);
     GemmParams p{static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), bias, sa, sb, C, 1, 1, M, N, K};
     p.v_codes = static_cast<uint8_t*>(v_codes);
+    p.v_fht_scale = v_fht_scale;
     p.v_col0 = v_col0;
     p.v_tokens = tokens;
     p.v_heads = (N - v_col0) / 64;

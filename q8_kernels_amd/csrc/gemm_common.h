@@ -22,6 +22,9 @@ struct GemmParams {
     // C then has ldc = v_col0 columns per row
     uint8_t* v_codes = nullptr;
     int v_col0 = 0, v_tokens = 0, v_heads = 0;
+    // != 0: the 64 columns of every head go through the 64-point Hadamard transform times this factor before the cast (the
+    // queries or keys of an attention with apply_qk_hadamard, q8_kernels/functional/flash_attention.py:47-51)
+    float v_fht_scale = 0.f;
 };
 
 __device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0, 0, 0, 0};

@@ -62,11 +62,14 @@ __device__ __forceinline__ void tile_of_id(int bid, int nb, int tiles_m, int til
 // results are rounded to bf16 like the others, then cast to e4m3 (the c10 cast of q8_kernels/functional/flash_attention.py:
 // 38-45) and written token-major per head, [B, H, S, 64], the Q8_V_SD operand of the attention kernel: what the attention
 // prologue otherwise produces from the bf16 projection. C holds the other columns only (p.v_col0 per row).
-template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false, bool VSPLIT = false>
+// VSPLIT == 2: the bf16-rounded results of a head (a wave's 64-column slab) go through the 64-point Hadamard transform
+// times p.v_fht_scale before the cast: the Q or K operand of an attention with apply_qk_hadamard
+// (q8_kernels/functional/flash_attention.py:47-51) straight from the projection.
+template <int IN, bool GELU, int MT, bool RES, bool E4M3OUT = false, int VSPLIT = 0>
 __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, int tiles_m, int tiles_n, int total) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     static_assert(!(RES && E4M3OUT), "the residual epilogue writes bf16");
-    static_assert(!VSPLIT || (!RES && !E4M3OUT), "the V split belongs to the plain bf16 epilogue");
+    static_assert(VSPLIT == 0 || (!RES && !E4M3OUT), "the V split belongs to the plain bf16 epilogue");
     constexpr int BM = 64 * MT, BN = kPipeBN;
     constexpr int NCOPY = MT + 4;  // copy instructions per wave and stage: MT row groups of A, 4 of B
     const int tid = threadIdx.x, lane = tid & 63;
@@ -323,10 +326,10 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                      : "memory");
         const bool rows16 = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;  // e4m3 output: rows start 16-byte aligned
         (void)rows16;
-        const int ldc = VSPLIT ? p.v_col0 : N;  // columns per row of C
-        const bool vtile = VSPLIT && cur.n0 >= p.v_col0;  // uniform: this tile holds V columns
+        const int ldc = VSPLIT != 0 ? p.v_col0 : N;  // columns per row of C
+        const bool vtile = VSPLIT != 0 && cur.n0 >= p.v_col0;  // uniform: this tile holds V columns
         (void)vtile;
-        uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + (VSPLIT ? (size_t)cur.z * M * ldc : zc);
+        uint16_t* const cbase = reinterpret_cast<uint16_t*>(p.C) + (VSPLIT != 0 ? (size_t)cur.z * M * ldc : zc);
         const uint16_t* const rbase = reinterpret_cast<const uint16_t*>(p.residual) + zc;
         v4i gq = v4i{0, 0, 0, 0};  // the gate of the 8 columns this lane stores (RES with p.gate)
         if constexpr (RES) {
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                         outc[t][wp] = v4u{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
                     }
                 }
-                if constexpr (VSPLIT) {
+                if constexpr (VSPLIT == 1) {
                     if (vtile) {
                         // the wave's 64-column slab is one head: codes of the bf16-rounded results, the two lanes of a row
                         // swap a chunk as below and store 16 bytes each of the (token, head) row
@@ -423,7 +426,76 @@ __global__ __launch_bounds__(512) void gemm_persist_kernel(const GemmParams p, i
                     }
                 }
             }
-            if constexpr (VSPLIT) {
+            if constexpr (VSPLIT == 2) {
+                if (vtile) {
+                    // Column c = 32 t + 16 wp + 8 h + e of the head: the butterflies run over the bits of c from the lowest
+                    // up, as the row kernels' transform does (registers e, the lane half h, registers wp and t), every
+                    // stage the plain (a + b, a - b), so signed zeros come out as there too.
+                    float x[2][2][8];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int wp = 0; wp < 2; ++wp) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                x[t][wp][2 * e] = __uint_as_float(outc[t][wp][e] << 16);
+                                x[t][wp][2 * e + 1] = __uint_as_float(outc[t][wp][e] & 0xffff0000u);
+                            }
+#pragma unroll
+                            for (int sft = 1; sft < 8; sft <<= 1)
+#pragma unroll
+                                for (int e = 0; e < 8; ++e)
+                                    if ((e & sft) == 0) {
+                                        const float a = x[t][wp][e], b = x[t][wp][e + sft];
+                                        x[t][wp][e] = a + b;
+                                        x[t][wp][e + sft] = a - b;
+                                    }
+                            // lane halves: after the swap of two copies every lane holds the lower half's value (a) and
+                            // the upper half's (b); the lower half keeps a + b, the upper a - b
+                            const float sgn = h ? -1.0f : 1.0f;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x[t][wp][e]), __float_as_uint(x[t][wp][e]), false, false);
+                                x[t][wp][e] = __builtin_fmaf(__uint_as_float(r[1]), sgn, __uint_as_float(r[0]));
+                            }
+                        }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float a = x[t][0][e], b = x[t][1][e];
+                            x[t][0][e] = a + b;
+                            x[t][1][e] = a - b;
+                        }
+                    const int m = mw0 + 32 * i + r32;
+                    const int bb = m / p.v_tokens, ss = m - bb * p.v_tokens, head = (nw0 - p.v_col0) >> 6;
+                    uint8_t* const dst = p.v_codes + (((size_t)cur.z * (M / p.v_tokens) + bb) * p.v_heads + head) * (size_t)p.v_tokens * 64 +
+                                         (size_t)ss * 64 + 16 * h;
+                    uint32_t e8[2][2][2];
+#pragma unroll
+                    for (int wp = 0; wp < 2; ++wp) {
+                        float y[2][8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float a = x[0][wp][e], b = x[1][wp][e];
+                            y[0][e] = (a + b) * p.v_fht_scale;
+                            y[1][e] = (a - b) * p.v_fht_scale;
+                        }
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) {
+                            e8[t][wp][0] = pack4_e4m3_c10(y[t][0], y[t][1], y[t][2], y[t][3]);
+                            e8[t][wp][1] = pack4_e4m3_c10(y[t][4], y[t][5], y[t][6], y[t][7]);
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(e8[t][0][0], e8[t][1][0], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(e8[t][0][1], e8[t][1][1], false, false);
+                        if (m < M && nw0 + 32 * t + 16 * h < N) *reinterpret_cast<v4u*>(dst + 32 * t) = v4u{s0[0], s1[0], s0[1], s1[1]};
+                    }
+                }
+            }
+            if constexpr (VSPLIT != 0) {
                 if (vtile) continue;
             }
             if constexpr (E4M3OUT) {

@@ -53,17 +53,29 @@ def norm_modulate_quantize(x: torch.Tensor, norm_weight: Optional[torch.Tensor],
     return codes, scales
 
 
+def qk_hadamard_scale(head_dim: int, softmax_scale: Optional[float] = None) -> float:
+    """The factor flash_attn_func folds into the Hadamard transform of q and k when apply_qk_hadamard is set
+    (q8_kernels/functional/flash_attention.py:47-51): sqrt(1 / D) * sqrt(softmax_scale)."""
+    if softmax_scale is None:
+        softmax_scale = head_dim ** (-0.5)
+    return math.sqrt(1 / head_dim) * math.sqrt(softmax_scale)
+
+
 def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int,
                            softmax_scale: Optional[float] = None, batch_mask: Optional[torch.Tensor] = None,
                            apply_qk_hadamard: bool = False, freqs_cis=None, out_dtype: Optional[torch.dtype] = None,
                            per_token_scales: bool = False, q_norm_weight: Optional[torch.Tensor] = None,
                            k_norm_weight: Optional[torch.Tensor] = None, v_codes: Optional[torch.Tensor] = None,
-                           p_unit_range: bool = False) -> torch.Tensor:
+                           p_unit_range: bool = False, q_codes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [B, M, H*64], k, v [B, N, H*64] bfloat16 projections (strided slices of a fused projection are read in
     place) -> attention output [B, M, H*64].
 
     v_codes (instead of v, which is then None; direct casts only): the e4m3 V operand [B, H, N, 64] that the QKV
     projection's GEMM wrote itself (_C.mm_bias_qkv); the prologue then handles q and k only.
+
+    q_codes (instead of q, which is then None; direct casts with apply_qk_hadamard, no rotation, no q-norm): the e4m3 Q
+    operand [B, H, M, 64] that the query projection's GEMM wrote itself (_C.mm_bias_qkv with v_col0 = 0 and
+    fht_scale = qk_hadamard_scale(64, softmax_scale)); k and v [B, N, H*64] then go through one prologue launch.
 
     q_norm_weight / k_norm_weight (fp32 [H*64]) apply the qk-RMSNorm (over all heads of a token, no epsilon) first;
     freqs_cis = (cos, sin) fp32 tables of q's shape then rotates q and k (k must then have q's shape); they go
@@ -71,7 +83,7 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
     Without per_token_scales the operands are cast to e4m3 exactly as flash_attn_func does; with it each
     (token, head) row of q, k and v gets its own absmax scale. p_unit_range as in flash_attn_func (the reference's
     probability grid)."""
-    d = q.shape[-1] // num_heads
+    d = (q_codes if q is None else q).shape[-1] // (1 if q is None else num_heads)
     if softmax_scale is None:
         softmax_scale = d ** (-0.5)
     # the tables with their repeated values stored once (same bits, a quarter of the bytes when both properties hold)
@@ -80,6 +92,14 @@ def flash_attn_token_major(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nu
         qk_scale, kernel_scale = math.sqrt(1 / d) * math.sqrt(softmax_scale), 1.0
     else:
         qk_scale, kernel_scale = 1.0, softmax_scale
+    if q_codes is not None:
+        if (q is not None or per_token_scales or not apply_qk_hadamard or freqs_cis is not None or q_norm_weight is not None
+                or v_codes is not None or d != 64 or k.shape != v.shape or q_codes.dtype != _FP8):
+            raise RuntimeError("flash_attn_token_major: q_codes replaces q for direct casts with apply_qk_hadamard, head dim 64, "
+                               "no rotation and no q-norm")
+        kc, vc = _C.attn_prep_kv(k, v, num_heads, None, None, True, qk_scale, False, norm_weight=k_norm_weight)
+        return _C.flash_attention(q_codes, kc, vc, kernel_scale, batch_mask, out_dtype=out_dtype, token_major_out=True,
+                                  p_unit_range=p_unit_range, v_token_major=True)
     if v_codes is not None:
         if per_token_scales or v is not None or d != 64 or q.shape != k.shape:
             raise RuntimeError("flash_attn_token_major: v_codes replaces v for direct casts of a self-attention with head dim 64")

@@ -137,13 +137,14 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 8, 768, 16, 1536, 8, 384, I8, 0, None) == -4       # gate alignment
     assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 16, 768, 16, 1536, 8, 256, I8, 0, None) == -3      # K must exceed 256
     assert L.q8_gemm_gated_residual(16, 16, None, 16, 16, 16, 16, 768, 16, 0, 8, 384, I8, 0, None) == 0          # no rows
-    # q8_gemm_qkv(A, B, bias, sa, sb, C, v_codes, M, N, K, v_col0, tokens, in_dtype, stream)
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, None, 64, 768, 384, 512, 32, I8, None) == -1     # no v_codes
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 384, 576, 32, I8, None) == -3       # split off a tile boundary
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 384, 512, 48, I8, None) == -3       # rows are not whole batch elements
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 256, 512, 32, I8, None) == -3       # K must exceed 256
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 8, 64, 768, 384, 512, 32, I8, None) == -4        # v_codes alignment
-    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 0, 768, 384, 512, 32, I8, None) == 0         # no rows
+    # q8_gemm_qkv(A, B, bias, sa, sb, C, v_codes, M, N, K, v_col0, tokens, v_fht_scale, in_dtype, stream)
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, None, 64, 768, 384, 512, 32, 0.0, I8, None) == -1     # no v_codes
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 384, 576, 32, 0.0, I8, None) == -3       # split off a tile boundary
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 384, 512, 48, 0.0, I8, None) == -3       # rows are not whole batch elements
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 256, 512, 32, 0.0, I8, None) == -3       # K must exceed 256
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 8, 64, 768, 384, 512, 32, 0.0, I8, None) == -4        # v_codes alignment
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 64, 768, 384, 512, 32, -1.0, I8, None) == -3      # a negative Hadamard factor
+    assert L.q8_gemm_qkv(16, 16, None, 16, 16, 16, 16, 0, 768, 384, 512, 32, 0.0, I8, None) == 0         # no rows
     assert L.q8_gemm_set_config(7) == -6
     assert L.q8_attn_set_config(5) == -6 and L.q8_attn_set_config(-1) == -6
     # q8_attn_fwd(q, k, v, o, kv_len, sq, sk, sv, B, H, M, N, D, v_layout, v_row_stride, scale, out_dtype, flags, stream)

@@ -414,6 +414,12 @@ def test_dit_block_config5_full_size_properties(dev):
             seq = blk(*args)
         finally:
             Fp8DiTBlock.fuse = True
+        try:
+            Fp8DiTBlock.fuse_query_epilogue = False   # the cross-attention's queries through bfloat16 and the prologue
+            by_prologue = blk(*args)
+        finally:
+            Fp8DiTBlock.fuse_query_epilogue = True
+    assert_bit_equal(got, by_prologue, "config 5, queries cast in the GEMM epilogue vs by the attention prologue")
     assert got.shape == (2, 6144, 2048) and got.dtype == torch.bfloat16
     assert torch.isfinite(got.float()).all()
     assert_bit_equal(got, again, "config 5, second run")

@@ -498,3 +498,40 @@ def test_qkv_gemm_casts_v_in_its_epilogue(dev, in_dtype, shape, rows):
         _C().mm_bias_qkv(*args, s, v0 + 64)       # the split is not on a tile boundary
     with pytest.raises(RuntimeError):
         _C().mm_bias_qkv(*args, s + 1, v0)        # rows are not whole batch elements
+
+
+@pytest.mark.parametrize("in_dtype", ["fp8", "i8"])
+@pytest.mark.parametrize("shape", [(2, 96, 512, 384, 0), (1, 200, 768, 640, 256), (3, 192, 1024, 512, 0), (1, 333, 256, 1024, 0)])
+@pytest.mark.parametrize("rows", [43, 44], ids=["tile192", "tile256"])
+def test_qkv_gemm_hadamard_of_the_heads_in_its_epilogue(dev, in_dtype, shape, rows):
+    """q8_gemm_qkv with a Hadamard factor: the head-major e4m3 columns are the 64-point transform (times the factor) of the
+    plain GEMM's bf16 result per head, bit-equal to the oracle's hadamard_transform(out_type=e4m3) of that result and to
+    the attention prologue run on it; rows of zeros (a zero row scale) keep the signs of their zeros. The other columns
+    are those of the plain GEMM."""
+    b, s, n, k, v0 = shape
+    g = torch.Generator().manual_seed(n + k + s)
+    if in_dtype == "i8":
+        a, w = _rand_i8(g, b * s, k), _rand_i8(g, n, k)
+        sa, sw = torch.rand(b * s, generator=g) * 2e-3 + 1e-4, torch.rand(n, generator=g) * 2e-2 + 1e-3
+        mmb = _C().q8_mm_bias
+    else:
+        a, w = O.e4m3_c10(torch.randn(b * s, k, generator=g) * 50), O.e4m3_c10(torch.randn(n, k, generator=g) * 50)
+        sa, sw = torch.rand(b * s, generator=g) * 1e-2 + 1e-4, torch.rand(n, generator=g) * 1e-2 + 1e-4
+        mmb = _C().fp8_mm_bias
+    sa[3] = 0.0                                   # a token whose projection is the bias alone
+    bias = torch.randn(n, generator=g)
+    bias[v0:v0 + 64] = -0.0                        # ... and in its first head zeros of either sign (acc * 0 - 0)
+    args = (a.to(dev), w.to(dev), bias.to(dev), sa.to(dev), sw.to(dev))
+    scale = (64 ** -0.5) * (0.125 ** 0.5)
+    _set_cfg(rows)
+    try:
+        qk, vc = _C().mm_bias_qkv(*args, s, v0, scale)
+        assert _last_kernel() in PERSISTENT_KERNELS
+    finally:
+        _set_cfg(40)
+    want = mmb(*args, False, torch.bfloat16).reshape(b, s, n)
+    assert torch.equal(qk.view(torch.int16), want[..., :v0].contiguous().view(torch.int16)), "the other columns"
+    h = (n - v0) // 64
+    heads = want[..., v0:].cpu().reshape(b, s, h, 64).transpose(1, 2).contiguous()
+    assert_bit_equal(vc, O.ref_fht(heads, scale, E4M3), "against the oracle's transform of the bf16 projection")
+    assert_bit_equal(vc, _C().attn_prep_qk(want[..., v0:], h, None, None, True, scale), "against the attention prologue")
