@@ -126,6 +126,26 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
 
     float v[CH][8];
     load_row<Q8_BF16, LANES, CH>(xr, t, row_ok, dim, full, v);
+    // Norm weights and bfloat16 modulation rows are requested with the row, the latter as raw words (up to 4 chunks per
+    // thread): asked for chunk by chunk where they are used, every chunk waits for trips to the cache of its own.
+    constexpr bool EARLY = CH <= 4;
+    constexpr int EC = EARLY ? CH : 1;
+    float wv[EC][8];
+    v4u rs[EC], rt[EC];
+    const bool early_w = EARLY && apply_norm && w != nullptr;
+    const bool early_mod = EARLY && ms != nullptr && mod_dtype == Q8_BF16;
+    const int64_t mrow = row_ok ? row / rows_per_mod : 0;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const int e = (c * LANES + t) * 8;
+        if (full || e < dim) {
+            if (early_w) load8<Q8_F32>(w, e, wv[c]);
+            if (early_mod) {
+                rs[c] = *reinterpret_cast<const v4u*>(reinterpret_cast<const uint16_t*>(ms) + mrow * dim + e);
+                rt[c] = *reinterpret_cast<const v4u*>(reinterpret_cast<const uint16_t*>(mt) + mrow * dim + e);
+            }
+        }
+    }
     if (apply_norm) {
         float ss[1] = {0.f};
 #pragma unroll
@@ -139,10 +159,10 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
             const int e = (c * LANES + t) * 8;
             if (e >= dim) continue;
             if (w != nullptr) {
-                float wv[8];
-                load8<Q8_F32>(w, e, wv);
+                if (!early_w) load8<Q8_F32>(w, e, wv[EARLY ? c : 0]);
+                const float (&wc)[8] = wv[EARLY ? c : 0];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[c][i] = (v[c][i] * rstd) * wv[i];
+                for (int i = 0; i < 8; ++i) v[c][i] = (v[c][i] * rstd) * wc[i];
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[c][i] = v[c][i] * rstd;
@@ -151,14 +171,23 @@ __global__ __launch_bounds__(kBlock) void norm_mod_fht_quant_kernel(const void* 
         }
     }
     if (ms != nullptr) {
-        const int64_t mrow = row_ok ? row / rows_per_mod : 0;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int e = (c * LANES + t) * 8;
             if (e >= dim) continue;
             float sv[8], tv[8];
-            load8_any(ms, mod_dtype, mrow * dim + e, sv);
-            load8_any(mt, mod_dtype, mrow * dim + e, tv);
+            if (early_mod) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sv[2 * i] = __uint_as_float(rs[EARLY ? c : 0][i] << 16);
+                    sv[2 * i + 1] = __uint_as_float(rs[EARLY ? c : 0][i] & 0xffff0000u);
+                    tv[2 * i] = __uint_as_float(rt[EARLY ? c : 0][i] << 16);
+                    tv[2 * i + 1] = __uint_as_float(rt[EARLY ? c : 0][i] & 0xffff0000u);
+                }
+            } else {
+                load8_any(ms, mod_dtype, mrow * dim + e, sv);
+                load8_any(mt, mod_dtype, mrow * dim + e, tv);
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[c][i] = __builtin_fmaf(v[c][i], sv[i] + scale_add, tv[i]);
             round_mid8<Q8_BF16>(v[c]);

@@ -82,15 +82,15 @@ int main(int argc, char** argv) {
         note(q8_fht_quant_rows(P, D, P, D, PF, L, I, F, D, I % 8, nullptr));
         note(q8_rmsnorm_quant_rows(P, D, PF, P, D, PF, PF, L, I, F, D, I % 8, nullptr));
         note(q8_norm_mod_fht_quant_rows(P, PF, I % 2, P, P, D, L, F, I % 2, F, P, D, PF, L, I, I % 8, nullptr));
-        note(q8_attn_prep_qk(P, L, PF, PF, PF, P, PF, I, I, I, I, I % 2, F, D, nullptr));
-        note(q8_attn_prep_qk_pair(P, L, P, L, PF, PF, PF, PF, P, PF, P, PF, I, I, I, I, I % 2, F, D, nullptr));
-        note(q8_attn_prep_qkv(P, L, P, L, P, L, PF, PF, PF, PF, P, PF, P, PF, P, PF, I, I, I, I, I % 2, F, D, nullptr));
-        note(q8_attn_prep_kv(P, L, P, L, PF, PF, PF, P, PF, P, PF, I, I, I, I, I % 2, F, D, nullptr));
+        note(q8_attn_prep_qk(P, L, PF, PF, PF, P, PF, I, I, I, I, I % 9, F, D, nullptr));
+        note(q8_attn_prep_qk_pair(P, L, P, L, PF, PF, PF, PF, P, PF, P, PF, I, I, I, I, I % 9, F, D, nullptr));
+        note(q8_attn_prep_qkv(P, L, P, L, P, L, PF, PF, PF, PF, P, PF, P, PF, P, PF, I, I, I, I, I % 9, F, D, nullptr));
+        note(q8_attn_prep_kv(P, L, P, L, PF, PF, PF, P, PF, P, PF, I, I, I, I, I % 9, F, D, nullptr));
         note(q8_attn_prep_v(P, L, P, PF, I, I, I, I, I, nullptr));
         note(q8_gemm(P, P, PF, PF, PF, P, I, I, I, I, I, D, D, I % 2, nullptr));
         note(q8_gemm_residual(P, P, PF, PF, PF, P, P, I, I, I, I, I, D, I % 2, nullptr));
         note(q8_gemm_gated_residual(P, P, PF, PF, PF, P, P, L, P, I, I, I, D, I % 2, nullptr));
-        note(q8_gemm_qkv(P, P, PF, PF, PF, P, P, I, I, I, I, I, D, nullptr));
+        note(q8_gemm_qkv(P, P, PF, PF, PF, P, P, I, I, I, I, I, F, D, nullptr));
         note(q8_gemm_i32(static_cast<const int8_t*>(P), static_cast<const int8_t*>(P), static_cast<int32_t*>(P), I, I, I, nullptr));
         note(q8_attn_fwd(P, P, P, P, static_cast<const int32_t*>(P), PF, PF, PF, I, I, I, I, (rnd() % 4) ? 64 : I, I % 3, L, F, D, I % 32,
                          nullptr));
@@ -105,7 +105,10 @@ int main(int argc, char** argv) {
     note(q8_gemm(p, p, pf, pf, pf, p, 1, 1, 300, 200, 144, Q8_I8, Q8_E4M3, 0, nullptr));
     note(q8_gemm_residual(p, p, pf, pf, pf, p, p, 2, 1, 6144, 2048, 2048, Q8_E4M3, 0, nullptr));
     note(q8_gemm_gated_residual(p, p, pf, pf, pf, p, p, 6144, p, 12288, 2048, 2048, Q8_I8, 0, nullptr));
-    note(q8_gemm_qkv(p, p, pf, pf, pf, p, p, 12288, 6144, 2048, 4096, 6144, Q8_E4M3, nullptr));
+    note(q8_gemm_qkv(p, p, pf, pf, pf, p, p, 12288, 6144, 2048, 4096, 6144, 0.f, Q8_E4M3, nullptr));
+    note(q8_gemm_qkv(p, p, pf, pf, pf, nullptr, p, 12288, 2048, 2048, 0, 6144, 0.0442f, Q8_E4M3, nullptr));
+    note(q8_attn_prep_qk_pair(p, 6144, p, 6144, nullptr, nullptr, pf, pf, p, nullptr, p, nullptr, 2, 6144, 32, 64,
+                              Q8_PREP_FHT | Q8_PREP_PAIR_TABLES | Q8_PREP_SHARED_TABLES, 0.0442f, Q8_BF16, nullptr));
     note(q8_attn_fwd(p, p, p, p, nullptr, nullptr, nullptr, nullptr, 2, 32, 6144, 6144, 64, Q8_V_DS, 6144, 0.125f, Q8_BF16, 0, nullptr));
     note(q8_attn_fwd(p, p, p, p, static_cast<const int32_t*>(p), pf, pf, pf, 2, 32, 6144, 128, 64, Q8_V_SD, 64, 0.125f, Q8_E4M3, 0, nullptr));
     std::printf("abi_driver: %ld calls, %ld returned Q8_OK, no sanitizer report\n", g_calls, g_ok);
