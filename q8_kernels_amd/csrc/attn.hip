@@ -127,7 +127,17 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what is derived from it stays off the VALU
     const int ql = lane & 31, h = lane >> 5;
-    const int bh = blockIdx.y, b = bh / p.H;
+    // Workgroups are handed to the 8 XCDs (each with an L2 of its own) round-robin in launch order. With the query blocks of
+    // a (batch, head) next to each other in that order every L2 would see the keys and values of every (batch, head) in
+    // flight (about 21 x 0.8 MB at S = 6144); instead the launch order is re-read so that all query blocks of a
+    // (batch, head) run on one XCD, which then walks through its share of the (batch, head) pairs one after the other.
+    int bx = blockIdx.x, bh = blockIdx.y;
+    if ((gridDim.y & 7) == 0) {
+        const int nx = gridDim.x, lin = bh * nx + bx, slot = lin >> 3;
+        bh = (lin & 7) * (gridDim.y >> 3) + slot / nx;
+        bx = slot - (slot / nx) * nx;
+    }
+    const int b = bh / p.H;
     const int M = p.M, N = p.N;
     int valid = N;
     if (p.kv_len) {
@@ -137,7 +147,7 @@ __global__ __launch_bounds__(kWaves * 64, (SCALED && kWaves == 4 && kQT == 1) ? 
     const uint8_t* Qg = p.q + (size_t)bh * M * 64;
     const uint8_t* Kg = p.k + (size_t)bh * N * 64;
     const uint8_t* Vg = p.v + (size_t)bh * 64 * (VTOK ? (size_t)N : (size_t)p.v_row_stride);
-    const int q0 = blockIdx.x * kBlockQ + wave * (kQT * 32);
+    const int q0 = bx * kBlockQ + wave * (kQT * 32);
     // output row r of this (batch, head): element offset o_base + r * o_rs
     const bool o_tok = (p.flags & Q8_ATTN_O_TOKEN_MAJOR) != 0;
     const size_t o_base = o_tok ? ((size_t)b * M * p.H + (size_t)(bh - b * p.H)) * 64 : (size_t)bh * M * 64;
