@@ -86,7 +86,10 @@ class Fp8DiTBlock(nn.Module):
         bf16 = torch.bfloat16
         d, h = self.dim, self.num_heads
         # self-attention: q, k, v are read in place from the fused projection by the attention prologue kernels
-        if self.head_dim == 64 and d > 256 and d % 128 == 0:
+        # (what the persistent GEMM kernel takes: K = d a multiple of 128 above 256, operands below 2^32 bytes)
+        gemm_writes_codes = (self.head_dim == 64 and d > 256 and d % 128 == 0 and hidden.numel() < 2 ** 32
+                             and self.to_qkv.weight.numel() < 2 ** 32)
+        if gemm_writes_codes:
             # the V columns leave the projection's GEMM as the attention kernel's e4m3 operand, token-major per head
             # (shapes of the persistent GEMM kernel: K = d a multiple of 128 above 256, the split 2 d on a tile boundary)
             codes, scales = Q8F.fused.rms_norm_quantize(hidden, self.norm1.weight, torch.float8_e4m3fn)
@@ -102,7 +105,7 @@ class Fp8DiTBlock(nn.Module):
         # cross-attention to the text states
         kv2 = self._lin(self.to_kv2, text)  # k and v are read in place, like q, k, v of the self-attention
         k2, v2 = kv2[..., :d], kv2[..., d:]
-        if self.fuse_query_epilogue and self.head_dim == 64 and d > 256 and d % 128 == 0:
+        if self.fuse_query_epilogue and gemm_writes_codes:
             # the queries leave their projection's GEMM as the attention kernel's operand: Hadamard transform per head and
             # e4m3 cast in the epilogue (no rotation and no norm lies between the projection and the attention here)
             codes, scales = Q8F.fused.rms_norm_quantize(hidden, self.norm2.weight, torch.float8_e4m3fn)
