@@ -138,3 +138,69 @@ def test_gemm_random_shapes(dev, sweep_seed):
         # far in GELU's negative tail the oracle's float64 1 + tanh cancels to zero while the kernel keeps the tiny value
         diff = torch.where((got.cpu().float() - want.float()).abs() <= 1e-7, torch.zeros_like(diff), diff)
         assert int(diff.max()) <= 1, what + ": %d ulp" % int(diff.max())
+
+
+@pytest.mark.parametrize("sweep_seed", [41, 42])
+def test_head_major_epilogue_and_compact_tables_random_shapes(dev, sweep_seed):
+    """The GEMM epilogue that transforms and casts heads (q8_gemm_qkv with a Hadamard factor) on random head counts, splits,
+    depths, token counts, batches, operand types and tile heights: the plain columns are the plain GEMM's, the codes the
+    oracle's hadamard_transform(out_type=e4m3) of its bf16 result. The attention prologues on rotation tables that store
+    repeated values once (per pair, per batch, both), random shapes and options: bit-equal to the full tables."""
+    from q8_kernels_amd import _lib
+    rnd = random.Random(sweep_seed)
+    for case in range(20):
+        seed = rnd.randint(0, 1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        heads, v0 = rnd.choice([1, 2, 3, 4, 8, 12, 32]), rnd.choice([0, 0, 256, 512])
+        n, k = v0 + 64 * heads, 128 * rnd.randint(3, 12)
+        tokens, b = rnd.choice([1, 5, 33, 64, 200, 257, 700]), rnd.choice([1, 1, 2, 3])
+        m, i8 = b * tokens, rnd.random() < 0.5
+        if i8:
+            a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+            w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int8)
+            sa, sw = torch.rand(m, generator=g) * 2e-3 + 1e-4, torch.rand(n, generator=g) * 2e-2 + 1e-3
+        else:
+            a, w = O.e4m3_c10(torch.randn(m, k, generator=g) * 30), O.e4m3_c10(torch.randn(n, k, generator=g) * 30)
+            sa, sw = torch.rand(m, generator=g) * 1e-2 + 1e-4, torch.rand(n, generator=g) * 1e-2 + 1e-4
+        bias = torch.randn(n, generator=g)
+        args = (a.to(dev), w.to(dev), bias.to(dev), sa.to(dev), sw.to(dev))
+        scale, rows = rnd.choice([0.0442, 0.125, 1.0]), rnd.choice([40, 43, 44])
+        what = "sweep %d case %d seed %d: heads=%d v0=%d k=%d tokens=%d b=%d int8=%s rows=%d scale=%g" % (
+            sweep_seed, case, seed, heads, v0, k, tokens, b, i8, rows, scale)
+        _gemm_cfg(rows)
+        try:
+            qk, vc = _C().mm_bias_qkv(*args, tokens, v0, scale)
+        finally:
+            _gemm_cfg(40)
+        want = (_C().q8_mm_bias if i8 else _C().fp8_mm_bias)(*args, False, BF16).reshape(b, tokens, n)
+        assert_bit_equal(qk, want[..., :v0].contiguous(), what + " plain columns")
+        assert_bit_equal(vc, O.ref_fht(want[..., v0:].cpu().reshape(b, tokens, heads, 64).transpose(1, 2).contiguous(), scale, E4M3), what + " codes")
+        # the prologues on compact tables
+        d, h = rnd.choice([64, 64, 128]), rnd.choice([1, 2, 4, 8, 16, 32, 64])
+        dim = h * d
+        if dim not in (64, 128, 256) and (dim % 512 or dim > 4096):
+            continue
+        s, bb = rnd.choice([1, 3, 17, 64, 130, 301]), rnd.choice([1, 2, 3, 5])
+        q, kk, v = ((torch.randn(bb, s, dim, generator=g) * 1.5).to(BF16).to(dev) for _ in range(3))
+        shared = rnd.random() < 0.6
+        ang = torch.rand(1 if shared else bb, s, dim // 2, generator=g) * 6.28
+        cos = torch.cos(ang).repeat_interleave(2, -1).expand(bb, -1, -1).contiguous().to(dev)
+        sin = torch.sin(ang).repeat_interleave(2, -1).expand(bb, -1, -1).contiguous().to(dev)
+        form = rnd.choice(["pairs", "shared", "both"]) if shared else "pairs"
+        tc, ts = (cos, sin) if form == "shared" else (cos[..., 0::2], sin[..., 0::2])
+        if form != "pairs":
+            tc, ts = tc[:1], ts[:1]
+        tc, ts = tc.contiguous(), ts.contiguous()
+        scaled, fht = rnd.random() < 0.5, rnd.random() < 0.7
+        wq = (1 + 0.1 * torch.randn(dim, generator=g)).to(dev) if rnd.random() < 0.5 else None
+        what = "sweep %d case %d seed %d: tables b=%d s=%d h=%d d=%d form=%s scaled=%s fht=%s norm=%s" % (
+            sweep_seed, case, seed, bb, s, h, d, form, scaled, fht, wq is not None)
+        calls = [lambda c_, s_: _C().attn_prep_qk(q, h, c_, s_, fht, 0.0442, scaled, norm_weight=wq),
+                 lambda c_, s_: _C().attn_prep_qk_pair(q, kk, h, c_, s_, fht, 0.0442, scaled, q_norm_weight=wq, k_norm_weight=wq),
+                 lambda c_, s_: _C().attn_prep_kv(kk, v, h, c_, s_, fht, 0.0442, scaled, norm_weight=wq)]
+        if d == 64:
+            calls.append(lambda c_, s_: _C().attn_prep_qkv(q, kk, v, h, c_, s_, fht, 0.0442, scaled, q_norm_weight=wq, k_norm_weight=wq))
+        flat = lambda r: [t for part in (r if isinstance(r, (tuple, list)) else (r,)) for t in (part if isinstance(part, (tuple, list)) else (part,))]  # noqa: E731
+        for i, call in enumerate(calls):
+            for full_t, compact_t in zip(flat(call(cos, sin)), flat(call(tc, ts))):
+                assert_bit_equal(compact_t, full_t, what + " call %d" % i)
