@@ -158,6 +158,17 @@ int q8_fma(const void* x, int x_dtype, const void* y, int y_dtype, const void* z
            q8_stream_t stream);
 
 /*
+ * The modulation rows of an AdaLN block: rows[p, r, :] = bf16(table[p, :] + timestep[r, p*dim .. (p+1)*dim)).
+ * Replaces the torch expression `scale_shift_table[None, None] + timestep.reshape(B, T, P, dim)` and its unbind
+ * (q8_kernels/blocks/ltx_transformer_block.py:30-36) followed by the casts of its six slices: table fp32 [params, dim],
+ * timestep fp32 [tokens, params * dim] (tokens = B * T), rows bf16 [params, tokens, dim] - each parameter's rows
+ * contiguous, the layout q8_norm_mod_fht_quant_rows and q8_gemm_gated_residual read. The sum is formed in fp32 and
+ * rounded once. dim % 8 == 0, 1 <= params <= 64; all pointers 16-byte aligned.
+ */
+int q8_adaln_rows(const float* table, const float* timestep, void* rows, int params, int64_t tokens, int dim,
+                  q8_stream_t stream);
+
+/*
  * tanh-GELU and the operators of the backward pass (the LoRA fine-tuning path of the reference).
  *   q8_gelu             replaces ops._C.gelu_forward      (csrc/ops/gelu_act.cpp, kernel gelu_forward_cuda.cu:12-16,73-100)
  *   q8_gelu_backward    replaces ops._C.gelu_backward     (kernel gelu_backward_cuda.cu:67-105): out = grad * dGELU(x)

@@ -641,6 +641,26 @@ def _rows2d(t, name):
     return t2 if t2.is_contiguous() else t2.contiguous()
 
 
+def adaln_rows(table: torch.Tensor, timestep: torch.Tensor) -> torch.Tensor:
+    """The modulation rows of an AdaLN block (q8_kernels/blocks/ltx_transformer_block.py:30-36): table float32 [P, dim],
+    timestep float32 [B, T, P * dim] -> bfloat16 [P, B, T, dim] = bf16(table[p] + timestep[b, t, p*dim:(p+1)*dim]); slice p
+    is the contiguous [B, T, dim] tensor that `(table[None, None] + timestep.reshape(B, T, P, dim)).unbind(2)[p]` gives after
+    its cast to bfloat16."""
+    _require_gpu(table, "table")
+    _require_gpu(timestep, "timestep")
+    if table.dtype != torch.float32 or timestep.dtype != torch.float32 or table.dim() != 2 or timestep.dim() != 3:
+        raise RuntimeError("adaln_rows: table float32 [P, dim] and timestep float32 [B, T, P*dim]")
+    p, dim = table.shape
+    b, t, pd = timestep.shape
+    if pd != p * dim:
+        raise RuntimeError("adaln_rows: timestep's last dimension %d is not %d parameters x %d" % (pd, p, dim))
+    table, timestep = table.contiguous(), timestep.contiguous()
+    rows = torch.empty((p, b, t, dim), dtype=torch.bfloat16, device=table.device)
+    with torch.cuda.device(table.device):
+        _lib.check(_lib.lib().q8_adaln_rows(table.data_ptr(), timestep.data_ptr(), rows.data_ptr(), p, b * t, dim, _stream(table)))
+    return rows
+
+
 def fma_8bit(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, scale_add: float = 0.0, *,
              out_type: Optional[torch.dtype] = None) -> torch.Tensor:
     """csrc/ops/fma.cpp:63-112: x * (y + scale_add) + z for x [B, T, dim] e4m3, y and z [B, T or 1, dim]

@@ -32,6 +32,7 @@ SIGNATURES = {
     "q8_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i64, _i, _f, _vp]),
     "q8_rope": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i64, _i, _vp]),
     "q8_fma": (_i, [_vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i, _i64, _i64, _f, _vp]),
+    "q8_adaln_rows": (_i, [_vp, _vp, _vp, _i, _i64, _i, _vp]),
     "q8_gelu": (_i, [_vp, _i, _vp, _i, _i64, _vp]),
     "q8_gelu_backward": (_i, [_vp, _i, _vp, _i, _vp, _i, _i64, _vp]),
     "q8_rope_backward": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i64, _i, _vp]),

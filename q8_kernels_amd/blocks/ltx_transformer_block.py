@@ -8,6 +8,7 @@ them with torch element-wise kernels that round to bfloat16 after every operatio
 import torch
 import torch.nn as nn
 
+from .. import _C
 from .. import functional as Q8F
 from ..modules.attention import Attention
 from ..modules.ffn import FeedForward
@@ -52,10 +53,14 @@ class LTXTransformerBlock(nn.Module):
         if fuse and timestep_rows.dtype == self.scale_shift_table.dtype == torch.float32:
             # the six modulation rows as contiguous bfloat16 tensors [B, T, dim] cut from ONE tensor laid out [6, B, T, dim],
             # written by the addition itself (fp32 sum, rounded once on the way out: bf16(table + timestep), the values the
-            # separate cast gives) - one small kernel instead of an addition, a layout change and six casts
-            rows = torch.empty((num_ada_params,) + tuple(timestep_rows.shape[:2]) + (timestep_rows.shape[-1],),
-                               dtype=torch.bfloat16, device=hidden_states.device)
-            torch.add(self.scale_shift_table[None, None], timestep_rows, out=rows.permute(1, 2, 0, 3))
+            # separate cast gives) - one small kernel (q8_adaln_rows; torch's strided, casting addition takes 10 us for these
+            # 24 K elements) instead of an addition, a layout change and six casts
+            if timestep_rows.shape[-1] % 8 == 0 and num_ada_params <= 64 and timestep.dim() == 3:
+                rows = _C.adaln_rows(self.scale_shift_table.data, timestep)
+            else:
+                rows = torch.empty((num_ada_params,) + tuple(timestep_rows.shape[:2]) + (timestep_rows.shape[-1],),
+                                   dtype=torch.bfloat16, device=hidden_states.device)
+                torch.add(self.scale_shift_table[None, None], timestep_rows, out=rows.permute(1, 2, 0, 3))
             shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = rows.unbind(dim=0)
         else:
             ada_values = self.scale_shift_table[None, None] + timestep_rows

@@ -157,6 +157,25 @@ static bool is_8or16(int dt) { return dt == Q8_BF16 || dt == Q8_E4M3; }
 static bool is_operand(int dt) { return dt == Q8_BF16 || dt == Q8_E4M3 || dt == Q8_F32; }
 static bool aligned_for(const void* p, int dt) { return (reinterpret_cast<uintptr_t>(p) % (dt == Q8_E4M3 ? 8 : 16)) == 0; }
 
+// The modulation rows of an AdaLN block (q8_kernels/blocks/ltx_transformer_block.py:30-36): rows[p, r, :] =
+// bf16(table[p, :] + timestep[r, p * dim .. (p + 1) * dim)), the fp32 sum rounded once, row-major per parameter p so that
+// each of the `params` modulation tensors is contiguous. One 8-element chunk per thread.
+__global__ __launch_bounds__(kBlock) void adaln_rows_kernel(const float* __restrict__ table, const float* __restrict__ timestep,
+                                                            uint16_t* __restrict__ rows, int params, int64_t tokens, int chunks_per_row,
+                                                            int64_t nchunks) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= nchunks) return;
+    const int c = (int)(idx % chunks_per_row);
+    const int64_t pr = idx / chunks_per_row, p = pr / tokens, r = pr - p * tokens;
+    float a[8], b[8];
+    load8<Q8_F32>(table, (p * chunks_per_row + c) * 8, a);
+    load8<Q8_F32>(timestep, ((r * params + p) * chunks_per_row + c) * 8, b);
+    v4u o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack2_bf16(a[2 * i] + b[2 * i], a[2 * i + 1] + b[2 * i + 1]);
+    *reinterpret_cast<v4u*>(rows + idx * 8) = o;
+}
+
 static int grid_for(const char* who, int64_t nchunks, unsigned* grid) {
     const int64_t g = (nchunks + kBlock - 1) / kBlock;
     if (g > 0x7fffffffLL) return fail(Q8_ERR_SHAPE, "%s: too many elements", who);
@@ -192,6 +211,23 @@ static int check_ew(const char* who, const void* x, int xd, const void* out, int
     if (!is_8or16(xd) || !is_8or16(od)) return fail(Q8_ERR_DTYPE, "%s: dtypes (%d -> %d) must be BF16 or E4M3", who, xd, od);
     if (!aligned_for(x, xd) || !aligned_for(out, od)) return fail(Q8_ERR_ALIGN, "%s: operands must be 16-byte (8-byte for e4m3) aligned", who);
     return Q8_OK;
+}
+
+extern "C" int q8_adaln_rows(const float* table, const float* timestep, void* rows, int params, int64_t tokens, int dim,
+                             q8_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (params <= 0 || params > 64 || tokens < 0 || tokens > ((int64_t)1 << 32) || dim <= 0 || dim % 8 != 0)
+        return fail(Q8_ERR_SHAPE, "q8_adaln_rows: params %d tokens %lld dim %d (dim %% 8 == 0)", params, (long long)tokens, dim);
+    if (tokens == 0) return Q8_OK;
+    if (!table || !timestep || !rows) return fail(Q8_ERR_NULL, "q8_adaln_rows: null pointer");
+    if (!aligned16(table) || !aligned16(timestep) || !aligned16(rows))
+        return fail(Q8_ERR_ALIGN, "q8_adaln_rows: table, timestep and rows must be 16-byte aligned");
+    unsigned grid;
+    const int64_t nchunks = (int64_t)params * tokens * (dim / 8);
+    if (int st = grid_for("q8_adaln_rows", nchunks, &grid)) return st;
+    hipLaunchKernelGGL(adaln_rows_kernel, dim3(grid), dim3(kBlock), 0, stream, table, timestep, static_cast<uint16_t*>(rows), params,
+                       tokens, dim / 8, nchunks);
+    return launch_status("q8_adaln_rows");
 }
 
 extern "C" int q8_gelu(const void* x, int x_dtype, void* out, int out_dtype, int64_t n, q8_stream_t stream_) {

@@ -75,6 +75,7 @@ int main(int argc, char** argv) {
         note(q8_rmsnorm(P, D, PF, P, D, PF, L, I, F, nullptr));
         note(q8_rope(P, D, PF, PF, P, D, L, I, nullptr));
         note(q8_fma(P, D, P, D, P, D, P, D, L, I, L, L, F, nullptr));
+        note(q8_adaln_rows(PF, PF, P, I, L, I, nullptr));
         note(q8_gelu(P, D, P, D, L, nullptr));
         note(q8_gelu_backward(P, D, P, D, P, D, L, nullptr));
         note(q8_rope_backward(P, D, PF, PF, P, D, L, I, nullptr));

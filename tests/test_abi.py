@@ -88,6 +88,12 @@ def test_argument_validation_of_the_fused_and_elementwise_entry_points():
     assert L.q8_fma(16, F32, 16, F32, 16, F32, 16, E4, 4, 64, 1, 1, 0.0, None) == -2
     assert L.q8_fma(16, B16, 8, B16, 16, F32, 16, E4, 4, 64, 1, 1, 0.0, None) == -4
     assert L.q8_gelu(16, B16, 16, B16, 12, None) == -3
+    # q8_adaln_rows(table, timestep, rows, params, tokens, dim, stream)
+    assert L.q8_adaln_rows(None, None, None, 6, 0, 2048, None) == 0        # no tokens
+    assert L.q8_adaln_rows(16, 16, None, 6, 2, 2048, None) == -1
+    assert L.q8_adaln_rows(16, 16, 16, 6, 2, 2044, None) == -3             # dim % 8
+    assert L.q8_adaln_rows(16, 16, 16, 0, 2, 2048, None) == -3
+    assert L.q8_adaln_rows(16, 8, 16, 6, 2, 2048, None) == -4
     assert L.q8_gelu_backward(16, B16, None, B16, 16, B16, 64, None) == -1
     assert L.q8_rope_backward(16, B16, None, 16, 16, B16, 4, 64, None) == -1
     assert L.q8_rmsnorm_backward(16, B16, None, 16, B16, None, 16, B16, 4, 64, None) == -1

@@ -447,3 +447,19 @@ def test_convert_state_dict_loads_into_the_block(dev):
     missing, unexpected = blk.load_state_dict({k[len(p):]: v for k, v in new.items() if k.startswith(p)}, strict=True)
     assert not missing and not unexpected
     assert blk.ff.proj_down.weight.dtype == torch.int8 and blk.attn1.to_q.scales.dtype == torch.float32
+
+
+@pytest.mark.parametrize("shape", [(2, 1, 6, 2048), (3, 5, 6, 512), (1, 1, 2, 8), (2, 700, 6, 64)])
+def test_adaln_rows(dev, shape):
+    """q8_adaln_rows: bf16(table + timestep) per modulation parameter, each parameter's rows contiguous - the bits of the
+    torch expression of the block (q8_kernels/blocks/ltx_transformer_block.py:30-36) followed by the cast."""
+    b, t, p, dim = shape
+    g = torch.Generator().manual_seed(b * 100 + t + dim)
+    table = (torch.randn(p, dim, generator=g) / dim ** 0.5)
+    ts = torch.randn(b, t, p * dim, generator=g) * 0.3
+    got = _C().adaln_rows(table.to(dev), ts.to(dev))
+    want = (table[None, None] + ts.reshape(b, t, p, dim)).to(torch.bfloat16).permute(2, 0, 1, 3).contiguous()
+    assert got.shape == (p, b, t, dim) and got.is_contiguous()
+    assert_bit_equal(got, want, "modulation rows")
+    with pytest.raises(RuntimeError):
+        _C().adaln_rows(table.to(dev), ts[..., :-8].to(dev))
