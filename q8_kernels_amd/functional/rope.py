@@ -107,7 +107,7 @@ def compact_freqs_cis(cos: torch.Tensor, sin: torch.Tensor, keep: int = 2):
     if (not compact_tables or cos.dim() != 3 or cos.shape != sin.shape or not cos.is_cuda or not sin.is_cuda
             or cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.requires_grad or sin.requires_grad):
         return cos, sin
-    key = (cos.data_ptr(), cos._version, sin.data_ptr(), sin._version, tuple(cos.shape), cos.stride(), sin.stride())
+    key = (cos.device, cos.data_ptr(), cos._version, sin.data_ptr(), sin._version, tuple(cos.shape), cos.stride(), sin.stride())
     for k, _, res in _COMPACT_CACHE:
         if k == key:
             return res
